@@ -1,0 +1,668 @@
+"""Pins the CPU oracle against every known-answer value the reference's own
+unit tests hold for this path, and against independent closed forms.
+
+Reference test locations are cited per test (paths relative to the reference
+checkout).  None of these tests touches a GPU.
+"""
+import math
+import struct
+
+import numpy as np
+import pytest
+
+Q4K, Q5K, Q6K, Q8_0, Q2K, Q3K, Q5_0, F16, F32, BF16 = range(10)
+
+
+def close(a, b):
+    # crates/allpaka-backend/src/ops/mod.rs:25-27
+    return abs(a - b) < 1e-5 * (1.0 + abs(b))
+
+
+def f16le(ora, x):
+    return list(struct.pack("<H", ora.f32_to_f16(x)))
+
+
+# --------------------------------------------------------------- f16 <-> f32
+def test_f16_specials(ora):
+    # crates/allpaka-gguf/src/dequant.rs:303-315
+    for x in [1.0, -1.0, 0.5, 2.0, 65504.0, 0.099975586]:
+        back = ora.f16_to_f32(ora.f32_to_f16(x))
+        assert abs(back - x) <= abs(x) * 1e-3
+    assert ora.f16_to_f32(0x0000) == 0.0 and math.copysign(1, ora.f16_to_f32(0x0000)) == 1
+    assert ora.f16_to_f32(0x8000) == 0.0 and math.copysign(1, ora.f16_to_f32(0x8000)) == -1
+    assert math.isinf(ora.f16_to_f32(0x7C00))
+    assert math.isnan(ora.f16_to_f32(0x7C01))
+    assert abs(ora.f16_to_f32(0x0001) - 2.0 ** -24) < 1e-12
+
+
+def test_f16_round_trip_list(ora):
+    # crates/allpaka-backend/src/ops/mod.rs:35-69
+    cases = [0.0, -0.0, 1.0, -1.0, 0.5, 2.0, 65504.0, -65504.0, 1e-5, -1e-5, 6.0e-8, 1.0 / 3.0, 1e8, -1e8,
+             math.inf, -math.inf, 0.30078125, 1.0009765625]
+    for x in cases:
+        h = ora.f32_to_f16(x)
+        back = ora.f16_to_f32(h)
+        if abs(x) > 65519.0:
+            assert back == math.copysign(math.inf, x)
+        assert ora.f32_to_f16(back) == h, f"{x} does not settle"
+    assert math.isnan(ora.f16_to_f32(ora.f32_to_f16(math.nan)))
+
+
+def test_f16_to_f32_exhaustive_vs_numpy(ora):
+    codes = np.arange(65536, dtype=np.uint16)
+    got = ora.f16_bits_to_f32(codes)
+    want = codes.view(np.float16).astype(np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+    # NaN payloads: frac << 13 kept (crates/allpaka-dtype/src/lib.rs:142)
+    assert np.array_equal(got[nan].view(np.uint32), want[nan].view(np.uint32) & ~np.uint32(0) | 0)
+
+
+def test_f32_to_f16_rne_vs_numpy(ora):
+    rng = np.random.default_rng(7)
+    # random bit patterns across every exponent, plus exact half-way cases
+    bits = rng.integers(0, 2 ** 32, size=400000, dtype=np.uint64).astype(np.uint32)
+    x = bits.view(np.float32)
+    x = x[~np.isnan(x)]
+    ties = (np.arange(0, 2048, dtype=np.float32) + 0.5) * np.float32(2.0 ** -10) + np.float32(1.0)
+    sub = (np.arange(0, 2048, dtype=np.float32) + 0.5) * np.float32(2.0 ** -24)
+    x = np.concatenate([x, ties, -ties, sub, -sub, np.float32([65504, 65519.9, 65520, 65536, 1e-8, 2.98e-8, 2.99e-8])])
+    got = ora.f32_to_f16_bits(x)
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).view(np.uint16)
+    assert np.array_equal(got, want)
+
+
+# ------------------------------------------------------------- block geometry
+def test_block_geometry(ora):
+    # crates/allpaka-dtype/src/lib.rs:478-492, crates/allpaka-backend/src/gpu/common.rs:106-151
+    assert ora.expected_bytes(Q4K, 512) == 288
+    assert ora.expected_bytes(99, 64) is None
+    assert ora.expected_bytes(Q4K, 300) is None
+    assert ora.expected_bytes(Q6K, 256) == 210
+    assert ora.expected_bytes(Q8_0, 64) == 68
+    assert ora.expected_bytes(F16, 10) == 20
+    assert ora.expected_bytes(F32, 3) == 12
+    assert ora.expected_bytes(Q4K, 100) is None
+    assert ora.expected_bytes(Q4K, 128) is None
+    assert ora.expected_bytes(Q5_0, 128) == 88
+    assert ora.expected_bytes(Q8_0, 1024) == 1088
+    assert ora.expected_bytes(Q4K, 5120) == 2880
+    for fmt in range(0, 6):
+        assert ora.embed_row_groups(fmt, 512) == 2 and ora.embed_row_groups(fmt, 128) == 1
+    for fmt in range(6, 10):
+        assert ora.embed_row_groups(fmt, 512) == 16 and ora.embed_row_groups(fmt, 128) == 4
+    assert ora.FMT == {"Q4K": 0, "Q5K": 1, "Q6K": 2, "Q8_0": 3, "Q2K": 4, "Q3K": 5, "Q5_0": 6, "F16": 7, "F32": 8, "BF16": 9}
+
+
+# -------------------------------------------------------------------- dequant
+def test_q8_0_known_answer(ora):
+    # dequant.rs:317-331
+    block = np.zeros(34, np.uint8)
+    block[0:2] = f16le(ora, 0.5)
+    block[2] = 10
+    block[3] = np.uint8(-20 & 0xFF)
+    block[33] = 127
+    out = ora.dequant(Q8_0, block, 32)
+    assert out[0] == 5.0 and out[1] == -10.0 and out[31] == 63.5 and out[2] == 0.0
+
+
+def test_scale_min_k4_known_answer(ora):
+    # dequant.rs:429-444
+    packed = np.zeros(12, np.uint8)
+    packed[0] = 33
+    packed[4] = 21
+    packed[9] = (0b1001 << 4) | 0b0110
+    packed[1] |= 0b10 << 6
+    packed[5] |= 0b01 << 6
+    assert ora.scale_min_k4(0, packed) == (33.0, 21.0)
+    assert ora.scale_min_k4(5, packed) == (38.0, 25.0)
+
+
+def test_q4_k_known_answer(ora):
+    # dequant.rs:448-468
+    block = np.zeros(144, np.uint8)
+    block[0:2] = f16le(ora, 1.0)
+    block[2:4] = f16le(ora, 1.0)
+    block[4], block[5], block[8], block[9] = 2, 3, 1, 2
+    block[16] = 0x75
+    out = ora.dequant(Q4K, block, 256)
+    assert out[0] == 9.0 and out[1] == -1.0 and out[32] == 19.0 and out[33] == -2.0
+    assert np.all(out[64:] == 0.0)
+
+
+def test_q2_k_known_answers(ora):
+    # dequant.rs:335-372
+    block = np.zeros(84, np.uint8)
+    block[80:82] = f16le(ora, 1.0)
+    block[:16] = np.arange(16)
+    block[16:80] = 0b11100100
+    out = ora.dequant(Q2K, block, 256)
+    assert np.all(out[:16] == 0) and np.all(out[32:48] == 2.0) and np.all(out[112:128] == 21.0)
+    assert np.all(out[128:144] == 0) and np.all(out[240:256] == 45.0)
+    block = np.zeros(84, np.uint8)
+    block[80:82] = f16le(ora, 1.0)
+    block[82:84] = f16le(ora, 2.0)
+    block[0] = 0x51
+    assert np.all(ora.dequant(Q2K, block, 256)[:16] == -10.0)
+
+
+def test_q6_k_known_answers(ora):
+    # dequant.rs:376-425
+    block = np.zeros(210, np.uint8)
+    block[208:210] = f16le(ora, 1.0)
+    block[192:208] = 1
+    block[0] = 0x05
+    block[128] = 0b00000001
+    block[35] = 0x02
+    block[131] = 0b00001000
+    block[7] |= 0x90
+    block[135] |= 0b00010000
+    block[41] |= 0xF0
+    block[137] |= 0b11000000
+    out = ora.dequant(Q6K, block, 256)
+    assert out[0] == -11.0 and out[35] == 2.0 and out[71] == -7.0 and out[105] == 31.0 and out[1] == -32.0
+    assert np.all(out[128:] == -32.0)
+    block = np.zeros(210, np.uint8)
+    block[208:210] = f16le(ora, 0.5)
+    block[192] = np.uint8(-2 & 0xFF)
+    out = ora.dequant(Q6K, block, 256)
+    assert out[0] == 32.0 and out[16] == 0.0
+
+
+def test_q5_k_known_answer(ora):
+    # dequant.rs:472-495
+    block = np.zeros(176, np.uint8)
+    block[0:2] = f16le(ora, 1.0)
+    block[4:8] = 1
+    block[12:16] = 0x01
+    block[16] = 0b00001001
+    out = ora.dequant(Q5K, block, 256)
+    assert out[0] == 16.0 and out[1] == 0.0 and out[32] == 0.0 and out[96] == 16.0 and out[97] == 0.0
+
+
+def test_q3_k_known_answers(ora):
+    # dequant.rs:499-547
+    block = np.zeros(110, np.uint8)
+    block[108:110] = f16le(ora, 1.0)
+    block[96:104] = 0x11
+    block[104:108] = 0b10101010
+    block[0:32] = 0xFF
+    assert np.all(ora.dequant(Q3K, block, 256) == 0.0)
+    b2 = block.copy()
+    b2[0] = 0xFE
+    o2 = ora.dequant(Q3K, b2, 256)
+    assert o2[0] == -4.0 and np.all(o2[1:] == 0.0)
+    b3 = block.copy()
+    b3[0] = (~(1 << 4)) & 0xFF
+    o3 = ora.dequant(Q3K, b3, 256)
+    assert o3[128] == -4.0 and np.all(o3[:128] == 0.0)
+    block = np.zeros(110, np.uint8)
+    block[108:110] = f16le(ora, 1.0)
+    block[96] = 0x02
+    block[104] = 0b10
+    block[32] = 0b10
+    assert ora.dequant(Q3K, block, 256)[0] == 2.0 * (2.0 - 4.0)
+
+
+def test_q3_k_scale_unpack_matches_the_swar_form(ora):
+    # crates/allpaka-dtype/src/lib.rs:395-404 (SWAR) vs the per-scale rule :461-476
+    packed = bytes([0x12, 0x34, 0x56, 0x78, 0x9A, 0xBC, 0xDE, 0xF0, 0x1B, 0xE4, 0x27, 0xB1])
+    a0, a1, tmp = struct.unpack("<III", packed)
+    k1, k2 = 0x03030303, 0x0F0F0F0F
+    u = [(a0 & k2) | ((tmp & k1) << 4), (a1 & k2) | (((tmp >> 2) & k1) << 4),
+         ((a0 >> 4) & k2) | (((tmp >> 4) & k1) << 4), ((a1 >> 4) & k2) | (((tmp >> 6) & k1) << 4)]
+    swar = np.frombuffer(struct.pack("<IIII", *u), np.int8)
+    # run one Q3_K block whose only non-trivial part is the scales: quant = 1 everywhere
+    block = np.zeros(110, np.uint8)
+    block[0:32] = 0xFF
+    block[32:96] = 0b01010101
+    block[96:108] = np.frombuffer(packed, np.uint8)
+    block[108:110] = f16le(ora, 1.0)
+    out = ora.dequant(Q3K, block, 256).reshape(16, 16)
+    assert np.array_equal(out[:, 0], (swar.astype(np.int32) - 32).astype(np.float32))
+
+
+def test_wrong_byte_count_is_an_error(ora):
+    # dequant.rs:549-554
+    for fmt, nbytes, n in [(Q8_0, 33, 32), (Q2K, 84, 255), (99, 4, 1)]:
+        with pytest.raises(ora.OracleError):
+            ora.dequant(fmt, np.zeros(nbytes, np.uint8), n)
+
+
+def _np_q8_0(raw, n):
+    b = raw.reshape(-1, 34)
+    d = b[:, :2].copy().view(np.float16).astype(np.float32)
+    q = b[:, 2:].view(np.int8).astype(np.float32)
+    return (d * q).reshape(-1)[:n]
+
+
+def _np_q4_k(raw):
+    """Independent second decoder (vectorised, ggml's published layout)."""
+    b = raw.reshape(-1, 144)
+    d = b[:, 0:2].copy().view(np.float16).astype(np.float32)[:, 0]
+    dmin = b[:, 2:4].copy().view(np.float16).astype(np.float32)[:, 0]
+    s = b[:, 4:16].astype(np.uint32)
+    sc = np.zeros((b.shape[0], 8), np.uint32)
+    mn = np.zeros((b.shape[0], 8), np.uint32)
+    sc[:, :4] = s[:, 0:4] & 63
+    mn[:, :4] = s[:, 4:8] & 63
+    sc[:, 4:] = (s[:, 8:12] & 0xF) | ((s[:, 0:4] >> 6) << 4)
+    mn[:, 4:] = (s[:, 8:12] >> 4) | ((s[:, 4:8] >> 6) << 4)
+    qs = b[:, 16:].reshape(-1, 4, 32)
+    q = np.stack([qs & 0xF, qs >> 4], axis=2).reshape(-1, 8, 32).astype(np.float32)
+    dsc = (d[:, None] * sc.astype(np.float32)).astype(np.float32)
+    dm = (dmin[:, None] * mn.astype(np.float32)).astype(np.float32)
+    prod = (dsc[:, :, None] * q).astype(np.float32)
+    return (prod - dm[:, :, None]).astype(np.float32).reshape(-1)
+
+
+def test_q8_0_and_q4_k_vs_independent_numpy_decoder(ora):
+    rng = np.random.default_rng(11)
+    raw = rng.integers(0, 256, size=34 * 64, dtype=np.uint8)
+    blk = raw.reshape(-1, 34)
+    # keep scales finite but include f16 subnormals
+    sc = rng.integers(0, 0x3C00, size=64, dtype=np.uint16)
+    sc[:8] = np.arange(8, dtype=np.uint16)  # 0 and the smallest subnormals
+    blk[:, 0:2] = sc.view(np.uint8).reshape(-1, 2)
+    got = ora.dequant(Q8_0, raw, 32 * 64)
+    assert np.array_equal(got.view(np.uint32), _np_q8_0(raw, 32 * 64).view(np.uint32))
+
+    raw = rng.integers(0, 256, size=144 * 200, dtype=np.uint8)
+    blk = raw.reshape(-1, 144)
+    dd = rng.integers(0, 0x3C00, size=(200, 2), dtype=np.uint16)
+    dd[:4] = [[0, 1], [1, 0], [2, 3], [0x3FF, 0x400]]
+    blk[:, 0:4] = dd.view(np.uint8).reshape(-1, 4)
+    got = ora.dequant(Q4K, raw, 256 * 200)
+    assert np.array_equal(got.view(np.uint32), _np_q4_k(raw).view(np.uint32))
+
+
+def test_q4_k_all_nibble_sub_block_cases(ora):
+    # brute force: every (byte value, sub-block pair) with distinct scales/mins
+    for pair in range(4):
+        block = np.zeros(144, np.uint8)
+        block[0:2] = f16le(ora, 0.25)
+        block[2:4] = f16le(ora, 0.125)
+        packed = np.zeros(12, np.uint8)
+        want_sc, want_mn = [], []
+        for j in range(8):
+            sc, mn = (5 * j + 3) % 64, (11 * j + 7) % 64
+            want_sc.append(sc), want_mn.append(mn)
+            if j < 4:
+                packed[j] |= sc & 63
+                packed[j + 4] |= mn & 63
+            else:
+                packed[j + 4] |= (sc & 0xF) | ((mn & 0xF) << 4)
+                packed[j - 4] |= (sc >> 4) << 6
+                packed[j] |= (mn >> 4) << 6
+        block[4:16] = packed
+        for j in range(8):
+            assert ora.scale_min_k4(j, packed) == (float(want_sc[j]), float(want_mn[j]))
+        for start in range(0, 256, 32):
+            block[16 + pair * 32:16 + pair * 32 + 32] = np.arange(start, start + 32, dtype=np.uint8)
+            out = ora.dequant(Q4K, block, 256)
+            for l in range(32):
+                byte = start + l
+                assert out[pair * 64 + l] == 0.25 * want_sc[2 * pair] * (byte & 0xF) - 0.125 * want_mn[2 * pair]
+                assert out[pair * 64 + 32 + l] == 0.25 * want_sc[2 * pair + 1] * (byte >> 4) - 0.125 * want_mn[2 * pair + 1]
+
+
+def test_quantmat_row_errors(ora):
+    # crates/allpaka-backend/src/quantmat/mod.rs:39-89, 923-937
+    data = np.zeros(34 * 2, np.uint8)
+    assert ora.quantmat_row(data, Q8_0, 1, 64, 0).shape == (64,)
+    with pytest.raises(ora.OracleError):
+        ora.quantmat_row(data, Q8_0, 1, 64, 1)  # row(1) of a 1-row matrix
+    with pytest.raises(ora.OracleError):
+        ora.quantmat_row(data, Q8_0, 1, 48, 0)  # ragged row
+    with pytest.raises(ora.OracleError):
+        ora.quantmat_row(data[:-1], Q8_0, 1, 64, 0)  # wrong byte count
+    with pytest.raises(ora.OracleError):
+        ora.quantmat_row(data, Q8_0, 1, 64, 0, dst_len=32)
+    with pytest.raises(ora.OracleError):
+        ora.embed_rows(data, Q8_0, 1, 64, [0, 1])  # token >= vocab
+
+
+# ---------------------------------------------------------------- rmsnorm/add
+def test_rmsnorm_known_answers(ora):
+    # ops/mod.rs:119-144
+    x = np.float32([3, -4, 12, 0])
+    ora.rmsnorm(x, np.ones(4, np.float32), 0.0)
+    assert close(math.sqrt(float((x * x).sum() / 4)), 1.0)
+    assert x[0] > 0 and x[1] < 0 and x[3] == 0
+    x = np.float32([1, 1])
+    ora.rmsnorm(x, np.float32([2, 3]), 0.0)
+    assert close(x[0], 2.0) and close(x[1], 3.0)
+    x = np.zeros(8, np.float32)
+    ora.rmsnorm(x, np.ones(8, np.float32), 1e-5)
+    assert np.all(np.isfinite(x))
+    with pytest.raises(ora.OracleError):
+        ora.rmsnorm(np.zeros(4, np.float32), np.zeros(3, np.float32), 0.0)
+
+
+def test_sum_sq_and_rmsnorm_vs_float64_closed_form(ora):
+    rng = np.random.default_rng(3)
+    for n in [1, 7, 8, 9, 128, 1024, 5120, 5123]:
+        x = rng.standard_normal(n).astype(np.float32)
+        w = (1 + 0.05 * rng.standard_normal(n)).astype(np.float32)
+        s = ora.sum_sq_f64(x)
+        assert abs(s - math.fsum((x.astype(np.float64) ** 2).tolist())) <= 1e-13 * s
+        dst = np.zeros(n, np.float32)
+        ora.rmsnorm_into(dst, x, w, 1e-6)
+        scale = 1.0 / math.sqrt(s / n + float(np.float32(1e-6)))
+        want = (x.astype(np.float64) * scale).astype(np.float32) * w
+        assert np.array_equal(dst, want)
+        y = x.copy()
+        ora.rmsnorm(y, w, 1e-6)
+        assert np.array_equal(y, dst)
+
+
+def test_sum_sq_uses_the_avx2_lane_order(ora):
+    # two 4-lane accumulators over 8-element steps, (acc0+acc1), lo+hi, then
+    # the two lanes, then the scalar tail: crates/allpaka-backend/src/ops/norm.rs:47-73
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal(8 * 37 + 5) * 1e3).astype(np.float32)
+    d = x.astype(np.float64)
+    acc = np.zeros(8)
+    for i in range(0, 8 * 37, 8):
+        acc = d[i:i + 8] * d[i:i + 8] + acc
+    s = acc[:4] + acc[4:]
+    total = (s[0] + s[2]) + (s[1] + s[3])
+    for v in d[8 * 37:]:
+        total += v * v
+    assert ora.sum_sq_f64(x) == total
+
+
+def test_rmsnorm_rows_into(ora):
+    # ops/mod.rs:412-419 and norm.rs:275-304 (serial and pool-parallel agree)
+    n = 1024
+    with pytest.raises(ora.OracleError, match="dst holds fewer rows than src"):
+        ora.rmsnorm_rows_into(np.zeros(8 * n, np.float32), np.ones(64 * n, np.float32), np.ones(n, np.float32), 1e-6)
+    rng = np.random.default_rng(9)
+    src = rng.standard_normal((37, n)).astype(np.float32)
+    w = rng.standard_normal(n).astype(np.float32)
+    a, b = np.zeros_like(src), np.zeros_like(src)
+    ora.rmsnorm_rows_into(a, src, w, 1e-6, threads=1)
+    ora.rmsnorm_rows_into(b, src, w, 1e-6, threads=8)
+    assert np.array_equal(a, b)
+    for r in range(37):
+        one = np.zeros(n, np.float32)
+        ora.rmsnorm_into(one, src[r].copy(), w, 1e-6)
+        assert np.array_equal(a[r], one)
+
+
+def test_add_assign_rejects_shorter_source(ora):
+    # ops/mod.rs:396-408
+    with pytest.raises(ora.OracleError):
+        ora.add_assign_slice(np.zeros(64, np.float32), np.ones(8, np.float32))
+    with pytest.raises(ora.OracleError):
+        ora.add_scaled_slice(np.zeros(64, np.float32), np.ones(8, np.float32), 2.0)
+    rng = np.random.default_rng(2)
+    a = rng.standard_normal(300000).astype(np.float32)
+    b = rng.standard_normal(300000).astype(np.float32)
+    a1, a2 = a.copy(), a.copy()
+    ora.add_assign_slice(a1, b)
+    ora.add_assign_par(a2, b, 8)
+    assert np.array_equal(a1, a + b) and np.array_equal(a2, a + b)
+
+
+# ----------------------------------------------------------------------- rope
+def test_rope_identity_and_norm_preserving(ora):
+    # ops/mod.rs:188-202
+    for rope in (ora.rope_norm, ora.rope_neox):
+        orig = (np.arange(8) - 3.5).astype(np.float32)
+        x = orig.copy()
+        rope(x, 0, 10000.0)
+        assert np.array_equal(x, orig)
+        rope(x, 17, 10000.0)
+        assert close(float((orig * orig).sum()), float((x * x).sum()))
+        assert not np.array_equal(x, orig)
+
+
+def test_rope_pairing(ora):
+    # ops/mod.rs:206-221
+    x = np.zeros(8, np.float32)
+    x[0] = 1
+    ora.rope_norm(x, 1, 10000.0)
+    assert close(x[1], math.sin(1.0)) and x[4] == 0.0
+    x = np.zeros(8, np.float32)
+    x[0] = 1
+    ora.rope_neox(x, 1, 10000.0)
+    assert close(x[4], math.sin(1.0)) and x[1] == 0.0
+
+
+def test_cached_rope_is_bit_identical_to_naive(ora):
+    # ops/mod.rs:225-245 and :366-391
+    inv = ora.rope_inv_freq(8, 10000.0)
+    for pos in [0, 1, 3, 17, 4097, 5000]:
+        table = ora.rope_sin_cos(pos, inv)
+        orig = (np.arange(8) - 3.5).astype(np.float32)
+        a, b = orig.copy(), orig.copy()
+        ora.rope_neox(a, pos, 10000.0)
+        ora.rope_neox_cached_from_array(b, table)
+        assert np.array_equal(a, b)
+        a, b = orig.copy(), orig.copy()
+        ora.rope_norm(a, pos, 10000.0)
+        ora.rope_norm_cached_from_array(b, table)
+        assert np.array_equal(a, b)
+        # partial rotary: a 12-wide head rotating its first 8 channels
+        wide = np.concatenate([orig * 0.7, np.float32([9, 8, 7, 6])]).astype(np.float32)
+        expect = wide.copy()
+        head = expect[:8].copy()
+        ora.rope_neox_cached_from_array(head, table)
+        expect[:8] = head
+        ora.rope_neox_cached_from_array(wide, table)
+        assert np.array_equal(wide, expect)
+    with pytest.raises(ora.OracleError):
+        ora.rope_neox_cached_from_array(np.zeros(6, np.float32), np.zeros((4, 2), np.float32))
+
+
+def test_rope_frequency_decay_and_relative_position(ora):
+    # ops/mod.rs:249-282
+    x = np.ones(8, np.float32)
+    ora.rope_neox(x, 1, 10000.0)
+    assert abs(x[0] - 1) > 0.3 and abs(x[3] - 1) < 0.01
+    q = np.float32([((i * 7 + 3) % 5) - 2.0 for i in range(8)])
+    k = np.float32([((i * 3 + 1) % 7) - 3.0 for i in range(8)])
+
+    def dot_at(pq, pk):
+        a, b = q.copy(), k.copy()
+        ora.rope_neox(a, pq, 10000.0)
+        ora.rope_neox(b, pk, 10000.0)
+        return float((a * b).sum())
+
+    assert close(dot_at(5, 3), dot_at(102, 100))
+    assert close(dot_at(9, 0), dot_at(59, 50))
+    assert not close(dot_at(5, 3), dot_at(5, 0))
+
+
+def test_rope_tables_vs_closed_form(ora):
+    inv = ora.rope_inv_freq(128, 1e6)
+    want = np.float64(1e6) ** (-2.0 * np.arange(64) / 128.0)
+    assert np.allclose(inv, want, rtol=3e-7, atol=0)
+    assert inv[0] == 1.0
+    for pos in [0, 1, 511, 4095, 32767]:
+        t = ora.rope_sin_cos(pos, inv)
+        ang = (np.float32(pos) * inv).astype(np.float32).astype(np.float64)
+        assert np.allclose(t[:, 0], np.sin(ang), rtol=0, atol=1.2e-7)
+        assert np.allclose(t[:, 1], np.cos(ang), rtol=0, atol=1.2e-7)
+
+
+def test_qknorm_rope_rows_is_rmsnorm_then_rope_per_head(ora):
+    # the reference's own expectation idiom: crates/allpaka-backend/tests/gpu_parity.rs:686-695, 709-723
+    rng = np.random.default_rng(21)
+    rows, nq, nkv, hd = 3, 4, 2, 128
+    q = rng.standard_normal((rows, nq * hd)).astype(np.float32)
+    k = rng.standard_normal((rows, nkv * hd)).astype(np.float32)
+    qw = (0.88 + 0.001 * np.arange(hd)).astype(np.float32)
+    kw = (0.92 + 0.001 * np.arange(hd)).astype(np.float32)
+    inv = ora.rope_inv_freq(hd, 1e6)
+    ropes = ora.rope_table([5, 6, 7], inv)
+    q2, k2 = q.copy(), k.copy()
+    ora.qknorm_rope_rows(q2, k2, nq, nkv, hd, qw, kw, ropes, 1e-6)
+    for arr, got, w, nh in ((q, q2, qw, nq), (k, k2, kw, nkv)):
+        for r in range(rows):
+            for h in range(nh):
+                head = arr[r, h * hd:(h + 1) * hd].copy()
+                ora.rmsnorm(head, w, 1e-6)
+                ora.rope_neox_cached_from_array(head, ropes[r])
+                assert np.array_equal(head, got[r, h * hd:(h + 1) * hd])
+
+
+# ----------------------------------------------------------------- activation
+def test_silu_fixed_points_and_swiglu_sweep(ora):
+    # ops/mod.rs:163-185
+    assert ora.silu(0.0) == 0.0
+    assert close(ora.silu(1.0), 1.0 / (1.0 + math.exp(-1.0)))
+    assert abs(ora.silu(-20.0)) < 1e-7
+    assert close(ora.silu(20.0), 20.0)
+    gate = np.float32([i * 0.7 for i in range(-25, 26)])
+    up = np.float32([i * 0.5 - 3.0 for i in range(51)])
+    orig = gate.copy()
+    ora.swiglu(gate, up)
+    for got, g, u in zip(gate, orig, up):
+        assert close(got, ora.silu(g) * u)
+    want = orig.astype(np.float64) / (1 + np.exp(-orig.astype(np.float64))) * up
+    assert np.allclose(gate, want, rtol=3e-7, atol=1e-30)
+    with pytest.raises(ora.OracleError):
+        ora.swiglu(np.zeros(4, np.float32), np.zeros(3, np.float32))
+
+
+def test_softmax_known_answers(ora):
+    # ops/mod.rs:146-161
+    x = np.float32([1, 3, 2])
+    ora.softmax(x)
+    assert close(float(x.sum()), 1.0) and x[1] > x[2] > x[0]
+    x = np.float32([1000, 999])
+    ora.softmax(x)
+    assert np.all(np.isfinite(x)) and close(float(x[0] + x[1]), 1.0) and x[0] > x[1]
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal(128).astype(np.float32)
+    y = x.copy()
+    ora.softmax(y)
+    e = np.exp(x.astype(np.float64) - x.max())
+    assert np.allclose(y, e / e.sum(), rtol=1e-6)
+
+
+# --------------------------------------------------------------------- router
+def test_route_known_answer(ora):
+    # crates/allpaka-model/tests/gpu_eligible_forward.rs:88-97
+    ids, w = ora.route(np.float32([0.1, 0.5, 0.15, 0.25]), 2)
+    assert list(ids) == [1, 3]
+    assert abs(w[0] - 2.0 / 3.0) < 1e-6 and abs(w[1] - 1.0 / 3.0) < 1e-6
+
+
+def _ref_logits(n):
+    # crates/allpaka-model/src/model/moe.rs:664-669
+    return np.float32([((i * 37 % 331) - 165.0) * 0.03 for i in range(n)])
+
+
+def test_route_stack_heap_boundary_and_wide(ora):
+    # moe.rs:682-726
+    base = _ref_logits(256)
+    wide = np.concatenate([base, np.float32([-np.inf])])
+    for gating, norm in [(ora.SOFTMAX, True), (ora.SOFTMAX, False), (ora.SIGMOID, True)]:
+        for k in (1, 8):
+            a = ora.route_gated(base, k, gating, norm, 1.5)
+            b = ora.route_gated(wide, k, gating, norm, 1.5)
+            assert np.array_equal(a[0], b[0]) and np.all(np.abs(a[1] - b[1]) < 1e-6)
+    bias = np.float32([0.5 + (i % 7) * 0.01 for i in range(256)])
+    a = ora.route_gated(base, 8, ora.SIGMOID, True, 2.5, bias)
+    b = ora.route_gated(wide, 8, ora.SIGMOID, True, 2.5, np.concatenate([bias, np.float32([0])]))
+    assert np.array_equal(a[0], b[0]) and np.all(np.abs(a[1] - b[1]) < 1e-6)
+    probs = ora.route_gated(base, 256, ora.SOFTMAX, False, 1.0)[1]
+    a, b = ora.route(probs, 8), ora.route(np.concatenate([probs, np.float32([0])]), 8)
+    assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
+    w320 = _ref_logits(320)
+    ids, _ = ora.route_gated(w320, 4, ora.SOFTMAX, False, 1.0)
+    assert list(ids) == list(np.argsort(-w320, kind="stable")[:4])
+
+
+def test_route_gated_vs_numpy(ora):
+    rng = np.random.default_rng(13)
+    for _ in range(50):
+        logits = rng.standard_normal(128).astype(np.float32)
+        ids, w = ora.route_gated(logits, 8, ora.SOFTMAX, True, 1.0)
+        order = np.argsort(-logits, kind="stable")[:8]
+        assert list(ids) == list(order)
+        assert np.array_equal(ids, ora.topk_by_logits(logits, 8))
+        p = np.exp(logits.astype(np.float64) - logits.max())
+        p /= p.sum()
+        assert np.allclose(w, p[order] / p[order].sum(), rtol=2e-6)
+        ids2, w2 = ora.route_gated(logits, 8, ora.SOFTMAX, False, 1.5)
+        assert np.allclose(w2, 1.5 * p[order], rtol=2e-6)
+        # k clamps to n; k = 0 returns nothing
+        assert ora.route_gated(logits[:4].copy(), 8)[0].size == 4
+        assert ora.route_gated(logits, 0)[0].size == 0
+
+
+def test_route_ties_take_the_lower_index(ora):
+    logits = np.zeros(16, np.float32)
+    logits[[3, 9, 12]] = 2.0
+    logits[[5, 7]] = 1.0
+    ids, w = ora.route_gated(logits, 4)
+    assert list(ids) == [3, 9, 12, 5]
+    assert abs(float(w.sum()) - 1.0) < 1e-6
+    # all-equal scores: total > 0 so winners share the mass equally
+    ids, w = ora.route_gated(np.zeros(8, np.float32), 2)
+    assert list(ids) == [0, 1] and np.allclose(w, 0.5)
+
+
+def test_moe_group_brute_force(ora):
+    rng = np.random.default_rng(17)
+    for rows, k, ne in [(1, 1, 4), (5, 2, 4), (33, 8, 16), (64, 8, 128), (7, 3, 3)]:
+        logits = rng.standard_normal((rows, ne)).astype(np.float32)
+        ids, w = ora.route_rows(logits, k, threads=3)
+        table, tok, tok_off, hit_row, hit_w = ora.moe_group(ids, w, ne)
+        # brute force, written the way crates/allpaka-model/src/model/moe.rs:229-271 reads
+        groups = [[] for _ in range(ne)]
+        for t in range(rows):
+            for j in range(k):
+                groups[int(ids[t, j])].append((t, float(w[t, j])))
+        used = [e for e in range(ne) if groups[e]]
+        want_table, want_tok, r0 = [], [], 0
+        for e in used:
+            want_table.append([e, r0, len(groups[e])])
+            want_tok += [t for t, _ in groups[e]]
+            r0 += len(groups[e])
+        assert table.tolist() == want_table and tok.tolist() == want_tok and r0 == rows * k
+        hits = [[] for _ in range(rows)]
+        for gi, e in enumerate(used):
+            for ri, (t, wt) in enumerate(groups[e]):
+                hits[t].append((want_table[gi][1] + ri, wt))
+        assert tok_off.tolist() == [t * k for t in range(rows + 1)]
+        for t in range(rows):
+            assert hit_row[t * k:(t + 1) * k].tolist() == [r for r, _ in hits[t]]
+            assert hit_w[t * k:(t + 1) * k].tolist() == [np.float32(x) for _, x in hits[t]]
+            # CSR round trip: every hit row belongs to this token
+            assert all(tok[r] == t for r in hit_row[t * k:(t + 1) * k])
+        # invariants: every token k times, ascending within an expert
+        assert np.array_equal(np.bincount(tok, minlength=rows), np.full(rows, k))
+        for e, a, n in table:
+            seg = tok[a:a + n]
+            assert np.all(np.diff(seg.astype(np.int64)) > 0)
+        src = rng.standard_normal((rows, 24)).astype(np.float32)
+        assert np.array_equal(ora.gather_rows(src, tok), src[tok])
+
+
+# ----------------------------------------------- fp16 variants wrap the f32 ops
+def test_f16_variants_are_widen_op_round_once(ora):
+    rng = np.random.default_rng(23)
+    rows, n = 3, 256
+    x = ora.f32_to_f16_bits(rng.standard_normal((rows, n)).astype(np.float32))
+    d = ora.f32_to_f16_bits(rng.standard_normal((rows, n)).astype(np.float32))
+    g = (1 + 0.05 * rng.standard_normal(n)).astype(np.float32)
+    x2, h2 = x.copy(), np.zeros_like(x)
+    ora.add_rmsnorm_rows(x2, d, h2, g, 1e-6)
+    v = ora.f16_bits_to_f32(x) + ora.f16_bits_to_f32(d)
+    assert np.array_equal(x2, ora.f32_to_f16_bits(v))
+    hv = np.zeros_like(v)
+    for r in range(rows):
+        ora.rmsnorm_into(hv[r], v[r].copy(), g, 1e-6)
+    assert np.array_equal(h2, ora.f32_to_f16_bits(hv))
+    a, b = x.reshape(-1).copy(), d.reshape(-1).copy()
+    ora.swiglu(a, b)
+    gf, uf = ora.f16_bits_to_f32(x.reshape(-1)), ora.f16_bits_to_f32(d.reshape(-1))
+    ora.swiglu(gf, uf)
+    assert np.array_equal(a, ora.f32_to_f16_bits(gf))
