@@ -1,0 +1,264 @@
+"""Host-side mirror of the reference's operator surface over the C ABI.
+
+Names, argument meaning and error behaviour follow `allpaka_backend::ops`
+(crates/allpaka-backend/src/ops/*.rs), `QuantMat` (quantmat/mod.rs:39-89) and
+`model::route_gated` (crates/allpaka-model/src/model/moe.rs:601-616):
+  * where the reference panics on a length mismatch, these raise AssertionError;
+  * where the reference returns Err (QuantMat, dequant), these raise ValueError;
+  * where an accelerator entry would decline (`None`), these raise `Declined`.
+Tensors are torch CUDA tensors (float32, or float16 for the fp16 activation
+form); every op runs in place where the reference's does.
+"""
+import ctypes as C
+import enum
+
+import torch
+
+from . import lib as _l
+from .lib import Declined, check  # noqa: F401
+
+
+class Gating(enum.IntEnum):
+    Softmax = 0
+    Sigmoid = 1
+
+
+class GgmlType(enum.IntEnum):
+    """Values are the unified dequant format codes (gpu/common.rs:47-61)."""
+    Q4K = 0
+    Q5K = 1
+    Q6K = 2
+    Q8_0 = 3
+    Q2K = 4
+    Q3K = 5
+    Q5_0 = 6
+    F16 = 7
+    F32 = 8
+    BF16 = 9
+
+
+def _dt(t):
+    if t.dtype == torch.float32:
+        return _l.F32
+    if t.dtype == torch.float16:
+        return _l.F16
+    raise Declined(_l.DECLINE_UNSUPPORTED, f"activation dtype {t.dtype}")
+
+
+def _ptr(t):
+    if t is None:
+        return None
+    assert t.is_cuda and t.is_contiguous(), "device-resident contiguous tensors only"
+    return t.data_ptr()
+
+
+class Backend:
+    """One device context (`apk_ctx`): the process-wide backend singleton of the
+    reference (`with_gpu`, gpu/cuda/runtime/device.rs:944-948)."""
+
+    def __init__(self, device=0):
+        self.L = _l.load()
+        h = C.c_void_p()
+        check(self.L.apk_init(device, C.byref(h)))
+        self.h = h
+        self.device = torch.device("cuda", device)
+
+    def close(self):
+        if self.h:
+            self.L.apk_shutdown(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    # ---- runtime
+    def sync(self):
+        check(self.L.apk_sync(self.h))
+
+    def stats(self):
+        v = [C.c_uint64() for _ in range(4)]
+        check(self.L.apk_stats(self.h, *[C.byref(x) for x in v]))
+        return tuple(x.value for x in v)
+
+    def take_faults(self):
+        f = C.c_uint32()
+        check(self.L.apk_take_faults(self.h, C.byref(f)))
+        return f.value
+
+    def _enter(self):
+        # torch owns the buffers and fills them on its own stream
+        torch.cuda.current_stream(self.device).synchronize()
+
+    # ---- ops::* (crates/allpaka-backend/src/ops)
+    def rmsnorm(self, x, weight, eps):
+        """ops::rmsnorm (norm.rs:115): in place over ONE row."""
+        assert x.numel() == weight.numel()
+        self._rows(x, None, x, weight, weight.numel(), 1, eps)
+
+    def rmsnorm_into(self, dst, src, weight, eps):
+        """ops::rmsnorm_into (norm.rs:193)."""
+        assert src.numel() == weight.numel()
+        assert dst.numel() == src.numel()
+        self._rows(src, None, dst, weight, weight.numel(), 1, eps)
+
+    def rmsnorm_rows_into(self, dst, src, weight, eps):
+        """ops::rmsnorm_rows_into (norm.rs:275): rows = src.len() / weight.len()."""
+        n = weight.numel()
+        rows = src.numel() // n
+        assert dst.numel() >= rows * n, "dst holds fewer rows than src"
+        self._enter()
+        check(self.L.apk_add_rmsnorm_rows(self.h, _ptr(src), None, _ptr(dst), _ptr(weight), n, rows, eps, _dt(src)))
+        self.sync()
+
+    def add_assign_slice(self, a, b):
+        """ops::add_assign_slice (blas.rs:105) -- on the device this op only exists
+        fused in front of a norm; see add_rmsnorm_rows."""
+        assert a.numel() == b.numel()
+        raise Declined(_l.DECLINE_UNSUPPORTED, "residual add is fused into add_rmsnorm_rows on the device")
+
+    def add_rmsnorm_rows(self, x, delta, h, gamma, eps):
+        """x += delta; h = rmsnorm(x) * gamma, rows = x.len() / gamma.len()
+        (model/decode.rs:584 then :764, one launch)."""
+        n = gamma.numel()
+        assert x.numel() % n == 0
+        rows = x.numel() // n
+        if delta is not None:
+            assert delta.numel() == x.numel()
+            assert delta.dtype == x.dtype
+        assert h.numel() >= rows * n, "dst holds fewer rows than src"
+        assert h.dtype == x.dtype
+        self._rows(x, delta, h, gamma, n, rows, eps)
+
+    def _rows(self, x, delta, h, gamma, n, rows, eps):
+        assert gamma.dtype == torch.float32
+        self._enter()
+        check(self.L.apk_add_rmsnorm_rows(self.h, _ptr(x), _ptr(delta), _ptr(h), _ptr(gamma), n, rows, eps, _dt(x)))
+        self.sync()
+
+    def rope_table(self, positions, inv_freq):
+        """ops::rope_sin_cos per position -> [rows, half, 2] = [sin, cos] (rope.rs:18-22)."""
+        rows, half = positions.numel(), inv_freq.numel()
+        assert positions.dtype in (torch.int32, torch.uint32) and inv_freq.dtype == torch.float32
+        table = torch.empty((rows, half, 2), dtype=torch.float32, device=self.device)
+        self._enter()
+        check(self.L.apk_rope_table(self.h, _ptr(positions), _ptr(inv_freq), rows, half, _ptr(table)))
+        self.sync()
+        return table
+
+    def qknorm_rope_neox(self, q, k, q_norm, k_norm, rope_flat, n_q, n_kv, head_dim, eps, rot_dim=None):
+        """The QK-norm + RoPE loop of run_cpu_attention_from_qkv (attention.rs:131-165):
+        q [rows, n_q*head_dim], k [rows, n_kv*head_dim] in place; rope_flat [rows, half, 2]."""
+        rows = q.numel() // (n_q * head_dim) if n_q else k.numel() // (n_kv * head_dim)
+        assert q.numel() == rows * n_q * head_dim and k.numel() == rows * n_kv * head_dim
+        rot = head_dim if rot_dim is None else rot_dim
+        assert rope_flat.dtype == torch.float32 and rope_flat.numel() == rows * (rot // 2) * 2
+        assert q.dtype == k.dtype
+        for w in (q_norm, k_norm):
+            assert w is None or (w.numel() == head_dim and w.dtype == torch.float32)
+        self._enter()
+        check(self.L.apk_qknorm_rope_neox(self.h, _ptr(q), _ptr(k), _ptr(q_norm), _ptr(k_norm), _ptr(rope_flat), rows,
+                                          n_q, n_kv, head_dim, rot, eps, _dt(q)))
+        self.sync()
+
+    def rope_neox_cached_from_array(self, x, table):
+        """ops::rope_neox_cached_from_array (rope.rs:70) on one head."""
+        assert x.numel() >= table.shape[0] * 2
+        self.qknorm_rope_neox(x, x[:0], None, None, table, 1, 0, x.numel(), 0.0, rot_dim=table.shape[0] * 2)
+
+    def swiglu(self, gate, up):
+        """ops::swiglu (activation.rs:57): gate = silu(gate) * up."""
+        assert gate.numel() == up.numel()
+        assert gate.dtype == up.dtype
+        self._enter()
+        check(self.L.apk_swiglu(self.h, _ptr(gate), _ptr(up), gate.numel(), _dt(gate)))
+        self.sync()
+
+    # ---- model::route_gated (crates/allpaka-model/src/model/moe.rs:601)
+    def route_rows(self, logits, k, gating=Gating.Softmax, norm=True, scale=1.0, bias=None):
+        """route_gated_into_slice for every row of logits [rows, n_expert] -> (ids u32, w f32) [rows, k]."""
+        rows, n = logits.shape
+        k = min(k, n)
+        ids = torch.empty((rows, k), dtype=torch.int32, device=self.device)
+        w = torch.empty((rows, k), dtype=torch.float32, device=self.device)
+        if k == 0:
+            return ids, w
+        assert logits.dtype == torch.float32
+        self._enter()
+        check(self.L.apk_route_topk(self.h, _ptr(logits), _ptr(bias), rows, n, k, int(norm), scale,
+                                    int(gating == Gating.Sigmoid), _ptr(ids), _ptr(w)))
+        self.sync()
+        return ids, w
+
+    def route_gated(self, logits, k, gating=Gating.Softmax, norm=True, scale=1.0, bias=None):
+        """model::route_gated on one row -> list of (expert, weight), best first."""
+        ids, w = self.route_rows(logits.reshape(1, -1), k, gating, norm, scale, bias)
+        return list(zip(ids[0].tolist(), w[0].tolist()))
+
+    def moe_permute(self, ids, w, n_expert):
+        """groups/used/table/tok + CSR of Ffn::moe_batch (moe.rs:229-271, prefill.rs:624-675)."""
+        rows, k = ids.shape
+        dev = self.device
+        table = torch.zeros((n_expert, 3), dtype=torch.int32, device=dev)
+        n_used = torch.zeros(1, dtype=torch.int32, device=dev)
+        tok = torch.empty(rows * k, dtype=torch.int32, device=dev)
+        tok_off = torch.empty(rows + 1, dtype=torch.int32, device=dev)
+        hit_row = torch.empty(rows * k, dtype=torch.int32, device=dev)
+        hit_w = torch.empty(rows * k, dtype=torch.float32, device=dev)
+        self._enter()
+        check(self.L.apk_moe_permute(self.h, _ptr(ids), _ptr(w), rows, k, n_expert, _ptr(table), _ptr(n_used), _ptr(tok),
+                                     _ptr(tok_off), _ptr(hit_row), _ptr(hit_w)))
+        self.sync()
+        return table[: int(n_used.item())], tok, tok_off, hit_row, hit_w
+
+    def gather_rows(self, src, tok):
+        """xe rows in tok order (moe.rs:348-352)."""
+        total = tok.numel()
+        dst = torch.empty((total, src.shape[1]), dtype=src.dtype, device=self.device)
+        self._enter()
+        check(self.L.apk_gather_rows(self.h, _ptr(src), _ptr(tok), src.shape[0], total, src.shape[1], _ptr(dst), _dt(src)))
+        self.sync()
+        return dst
+
+
+class QuantMat:
+    """QuantMat::{new,row,row_into} (quantmat/mod.rs:39-89) over a device-resident table."""
+
+    def __init__(self, backend, data, ty, n_out, n_in):
+        ty = int(ty)
+        rb = backend.L.apk_row_bytes(ty, n_in)
+        if ty < 0 or ty > 9:
+            raise ValueError(f"unsupported ggml type {ty}")
+        if rb == 0:
+            raise ValueError(f"row length {n_in} is not a whole number of blocks")
+        if rb * n_out != data.numel() * data.element_size():
+            raise ValueError(f"{n_out}x{n_in} needs {rb * n_out} bytes, got {data.numel() * data.element_size()}")
+        self.b, self.data, self.ty, self.n_out, self.n_in, self.row_bytes = backend, data, ty, n_out, n_in, rb
+
+    def row(self, j, dtype=torch.float32):
+        out = torch.empty(self.n_in, dtype=dtype, device=self.b.device)
+        self.row_into(j, out)
+        return out
+
+    def row_into(self, j, dst):
+        if j >= self.n_out or j < 0:
+            raise ValueError(f"row {j} out of {self.n_out}")
+        if dst.numel() != self.n_in:
+            raise ValueError(f"row_into destination has {dst.numel()} elements, expected {self.n_in}")
+        ids = (C.c_uint32 * 1)(j)
+        self.b._enter()
+        check(self.b.L.apk_embed_rows_host_ids(self.b.h, self.ty, _ptr(self.data), self.n_out, self.n_in, ids, 1, _ptr(dst), _dt(dst)))
+        self.b.sync()
+
+    def rows_into(self, ids, dst):
+        """The embedding loop of forward_batch (prefill.rs:92-106) as one launch; ids on the device."""
+        t = ids.numel()
+        if dst.numel() != t * self.n_in:
+            raise ValueError("destination size")
+        self.b._enter()
+        check(self.b.L.apk_embed_rows(self.b.h, self.ty, _ptr(self.data), self.n_out, self.n_in, _ptr(ids), t, _ptr(dst), _dt(dst)))
+        self.b.sync()
+        if self.b.take_faults() & _l.FAULT_TOKEN_RANGE:
+            raise ValueError("token id out of vocab")

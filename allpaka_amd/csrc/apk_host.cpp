@@ -1,0 +1,550 @@
+// Host side of libapk_hip.so: the C ABI declared in include/apk_hip.h.
+//
+// A thin runtime: one embedded gfx950 code object loaded with hipModuleLoadData,
+// one hipStream, argument validation that DECLINES (positive status) instead of
+// failing, and hipModuleLaunchKernel.  No device code in this translation unit:
+// it builds with a plain host C++ compiler against the HIP runtime API.
+#include "apk_hip.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <atomic>
+#include <chrono>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <vector>
+
+extern "C" const unsigned char apk_kernels_co[];
+extern "C" const unsigned char apk_kernels_co_end[];
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int status, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+    return status;
+}
+int hip_fail(hipError_t e, const char* what) {
+    return fail(-(int)e, "%s: %s (%d)", what, hipGetErrorString(e), (int)e);
+}
+#define HIP_TRY(expr)                                  \
+    do {                                               \
+        hipError_t e_ = (expr);                        \
+        if (e_ != hipSuccess) return hip_fail(e_, #expr); \
+    } while (0)
+
+uint64_t now_ns() {
+    return (uint64_t)std::chrono::duration_cast<std::chrono::nanoseconds>(
+               std::chrono::steady_clock::now().time_since_epoch())
+        .count();
+}
+
+struct Mapping {
+    void* dev;
+    size_t len;
+};
+
+enum Kernel {
+    K_SWIGLU_F32, K_SWIGLU_F16,
+    K_ADDNORM_F32_C1, K_ADDNORM_F32_C2, K_ADDNORM_F32_C4, K_ADDNORM_F32_C8,
+    K_ADDNORM_F16_C1, K_ADDNORM_F16_C2, K_ADDNORM_F16_C4, K_ADDNORM_F16_C8,
+    K_QKROPE_F32_64, K_QKROPE_F32_128, K_QKROPE_F32_256,
+    K_QKROPE_F16_64, K_QKROPE_F16_128, K_QKROPE_F16_256,
+    K_ROPE_TABLE,
+    K_EMBED_Q4K_F32, K_EMBED_Q4K_F16, K_EMBED_Q8_0_F32, K_EMBED_Q8_0_F16,
+    K_ROUTE_TOPK, K_MOE_PERMUTE, K_GATHER_ROWS, K_COPY,
+    K_COUNT
+};
+const char* const kKernelNames[K_COUNT] = {
+    "apk_swiglu_f32", "apk_swiglu_f16",
+    "apk_add_rmsnorm_f32_c1", "apk_add_rmsnorm_f32_c2", "apk_add_rmsnorm_f32_c4", "apk_add_rmsnorm_f32_c8",
+    "apk_add_rmsnorm_f16_c1", "apk_add_rmsnorm_f16_c2", "apk_add_rmsnorm_f16_c4", "apk_add_rmsnorm_f16_c8",
+    "apk_qknorm_rope_f32_hd64", "apk_qknorm_rope_f32_hd128", "apk_qknorm_rope_f32_hd256",
+    "apk_qknorm_rope_f16_hd64", "apk_qknorm_rope_f16_hd128", "apk_qknorm_rope_f16_hd256",
+    "apk_rope_table",
+    "apk_embed_q4k_f32", "apk_embed_q4k_f16", "apk_embed_q8_0_f32", "apk_embed_q8_0_f16",
+    "apk_route_topk", "apk_moe_permute", "apk_gather_rows", "apk_copy",
+};
+
+}  // namespace
+
+struct apk_ctx {
+    int device = 0;
+    hipModule_t module = nullptr;
+    hipStream_t stream = nullptr;
+    hipFunction_t fn[K_COUNT] = {};
+    uint32_t* fault_dev = nullptr;  // device status word
+    uint32_t* ids_stage_host = nullptr;  // pinned staging for host-side token ids
+    uint32_t* ids_stage_dev = nullptr;
+    size_t ids_stage_cap = 0;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    std::mutex mu;
+    std::map<uintptr_t, Mapping> attached;
+    std::atomic<uint64_t> calls{0}, dispatches{0}, encode_ns{0}, wait_ns{0};
+};
+
+namespace {
+
+struct CallScope {  // counts one ABI call and its host-side encode time
+    apk_ctx* c;
+    uint64_t t0;
+    std::lock_guard<std::mutex> lock;
+    explicit CallScope(apk_ctx* ctx) : c(ctx), t0(now_ns()), lock(ctx->mu) { c->calls++; }
+    ~CallScope() { c->encode_ns += now_ns() - t0; }
+};
+
+int launch(apk_ctx* c, Kernel k, unsigned grid, unsigned block, unsigned shmem, void** args) {
+    if (grid == 0) return APK_OK;
+    hipError_t e = hipModuleLaunchKernel(c->fn[k], grid, 1, 1, block, 1, 1, shmem, c->stream, args, nullptr);
+    if (e != hipSuccess) return hip_fail(e, kKernelNames[k]);
+    c->dispatches++;
+    return APK_OK;
+}
+
+bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+int elem_size(int dtype) { return dtype == APK_F32 ? 4 : (dtype == APK_F16 ? 2 : 0); }
+
+// block geometry: crates/allpaka-dtype/src/lib.rs:79-108
+void block_geom(int fmt, size_t* be, size_t* bb) {
+    static const size_t kBe[10] = {256, 256, 256, 32, 256, 256, 32, 1, 1, 1};
+    static const size_t kBb[10] = {144, 176, 210, 34, 84, 110, 22, 2, 4, 2};
+    if (fmt < 0 || fmt > 9) { *be = *bb = 0; return; }
+    *be = kBe[fmt];
+    *bb = kBb[fmt];
+}
+
+int set_device(apk_ctx* c) {
+    HIP_TRY(hipSetDevice(c->device));
+    return APK_OK;
+}
+
+}  // namespace
+
+#pragma GCC visibility push(default)
+extern "C" {
+
+const char* apk_last_error(void) { return g_err; }
+
+size_t apk_row_bytes(int fmt, size_t n_in) {
+    size_t be, bb;
+    block_geom(fmt, &be, &bb);
+    if (!be || n_in % be) return 0;
+    return n_in / be * bb;
+}
+
+int apk_can_embed(int fmt, size_t n_in) {
+    if (fmt != APK_FMT_Q8_0 && fmt != APK_FMT_Q4K) return 0;
+    return n_in > 0 && apk_row_bytes(fmt, n_in) != 0;
+}
+
+int apk_init(int device, apk_ctx** out) {
+    if (!out) return fail(APK_DECLINE_NULL, "apk_init: out is NULL");
+    *out = nullptr;
+    const char* no_gpu = getenv("ALLPAKA_NO_GPU");
+    if (no_gpu && *no_gpu && strcmp(no_gpu, "0") != 0)
+        return fail(APK_DECLINE_NO_DEVICE, "apk_init: disabled by ALLPAKA_NO_GPU");
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n <= 0 || device < 0 || device >= n)
+        return fail(APK_DECLINE_NO_DEVICE, "apk_init: no usable HIP device %d (count %d, %s)", device, n,
+                    hipGetErrorString(e));
+    apk_ctx* c = new apk_ctx();
+    c->device = device;
+    int rc = [&]() -> int {
+        HIP_TRY(hipSetDevice(device));
+        HIP_TRY(hipModuleLoadData(&c->module, apk_kernels_co));
+        for (int k = 0; k < K_COUNT; k++) HIP_TRY(hipModuleGetFunction(&c->fn[k], c->module, kKernelNames[k]));
+        HIP_TRY(hipStreamCreate(&c->stream));
+        HIP_TRY(hipMalloc((void**)&c->fault_dev, 256));
+        HIP_TRY(hipMemsetAsync(c->fault_dev, 0, 256, c->stream));
+        HIP_TRY(hipEventCreate(&c->ev0));
+        HIP_TRY(hipEventCreate(&c->ev1));
+        HIP_TRY(hipStreamSynchronize(c->stream));
+        return APK_OK;
+    }();
+    if (rc != APK_OK) {
+        apk_shutdown(c);
+        return rc;
+    }
+    *out = c;
+    return APK_OK;
+}
+
+int apk_shutdown(apk_ctx* c) {
+    if (!c) return APK_OK;
+    (void)hipSetDevice(c->device);
+    if (c->stream) (void)hipStreamSynchronize(c->stream);
+    for (auto& kv : c->attached) (void)hipFree(kv.second.dev);
+    if (c->ids_stage_dev) (void)hipFree(c->ids_stage_dev);
+    if (c->ids_stage_host) (void)hipHostFree(c->ids_stage_host);
+    if (c->fault_dev) (void)hipFree(c->fault_dev);
+    if (c->ev0) (void)hipEventDestroy(c->ev0);
+    if (c->ev1) (void)hipEventDestroy(c->ev1);
+    if (c->stream) (void)hipStreamDestroy(c->stream);
+    if (c->module) (void)hipModuleUnload(c->module);
+    delete c;
+    return APK_OK;
+}
+
+int apk_sync(apk_ctx* c) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_sync: ctx is NULL");
+    std::lock_guard<std::mutex> lock(c->mu);
+    uint64_t t0 = now_ns();
+    hipError_t e = hipStreamSynchronize(c->stream);
+    c->wait_ns += now_ns() - t0;
+    if (e != hipSuccess) return hip_fail(e, "hipStreamSynchronize");
+    return APK_OK;
+}
+
+void* apk_stream(apk_ctx* c) { return c ? (void*)c->stream : nullptr; }
+
+int apk_stats(apk_ctx* c, uint64_t* calls, uint64_t* dispatches, uint64_t* encode_ns, uint64_t* wait_ns) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_stats: ctx is NULL");
+    if (calls) *calls = c->calls;
+    if (dispatches) *dispatches = c->dispatches;
+    if (encode_ns) *encode_ns = c->encode_ns;
+    if (wait_ns) *wait_ns = c->wait_ns;
+    return APK_OK;
+}
+
+int apk_take_faults(apk_ctx* c, uint32_t* faults) {
+    if (!c || !faults) return fail(APK_DECLINE_NULL, "apk_take_faults: NULL argument");
+    std::lock_guard<std::mutex> lock(c->mu);
+    if (int rc = set_device(c)) return rc;
+    uint32_t v = 0;
+    HIP_TRY(hipMemcpyAsync(&v, c->fault_dev, 4, hipMemcpyDeviceToHost, c->stream));
+    HIP_TRY(hipStreamSynchronize(c->stream));
+    if (v) {
+        HIP_TRY(hipMemsetAsync(c->fault_dev, 0, 4, c->stream));
+        HIP_TRY(hipStreamSynchronize(c->stream));
+    }
+    *faults = v;
+    return APK_OK;
+}
+
+/* ---------------------------------------------------------------- memory */
+
+int apk_malloc(apk_ctx* c, size_t bytes, void** dev_out) {
+    if (!c || !dev_out) return fail(APK_DECLINE_NULL, "apk_malloc: NULL argument");
+    std::lock_guard<std::mutex> lock(c->mu);
+    if (int rc = set_device(c)) return rc;
+    HIP_TRY(hipMalloc(dev_out, bytes ? bytes : 16));
+    return APK_OK;
+}
+int apk_free(apk_ctx* c, void* dev) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_free: ctx is NULL");
+    std::lock_guard<std::mutex> lock(c->mu);
+    if (int rc = set_device(c)) return rc;
+    HIP_TRY(hipStreamSynchronize(c->stream));
+    HIP_TRY(hipFree(dev));
+    return APK_OK;
+}
+int apk_h2d(apk_ctx* c, void* dev_dst, const void* host_src, size_t bytes) {
+    if (!c || (bytes && (!dev_dst || !host_src))) return fail(APK_DECLINE_NULL, "apk_h2d: NULL argument");
+    CallScope s(c);
+    if (int rc = set_device(c)) return rc;
+    if (bytes) HIP_TRY(hipMemcpyAsync(dev_dst, host_src, bytes, hipMemcpyHostToDevice, c->stream));
+    return APK_OK;
+}
+int apk_d2h(apk_ctx* c, void* host_dst, const void* dev_src, size_t bytes) {
+    if (!c || (bytes && (!host_dst || !dev_src))) return fail(APK_DECLINE_NULL, "apk_d2h: NULL argument");
+    CallScope s(c);
+    if (int rc = set_device(c)) return rc;
+    if (bytes) HIP_TRY(hipMemcpyAsync(host_dst, dev_src, bytes, hipMemcpyDeviceToHost, c->stream));
+    return APK_OK;
+}
+
+int apk_attach(apk_ctx* c, const void* host_base, size_t len) {
+    if (!c || !host_base || !len) return fail(APK_DECLINE_NULL, "apk_attach: NULL or empty mapping");
+    std::lock_guard<std::mutex> lock(c->mu);
+    if (int rc = set_device(c)) return rc;
+    if (c->attached.count((uintptr_t)host_base)) return APK_OK;  // already resident
+    void* dev = nullptr;
+    HIP_TRY(hipMalloc(&dev, len));
+    hipError_t e = hipMemcpy(dev, host_base, len, hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        (void)hipFree(dev);
+        return hip_fail(e, "apk_attach: hipMemcpy");
+    }
+    c->attached[(uintptr_t)host_base] = Mapping{dev, len};
+    return APK_OK;
+}
+int apk_detach(apk_ctx* c, const void* host_base) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_detach: ctx is NULL");
+    std::lock_guard<std::mutex> lock(c->mu);
+    auto it = c->attached.find((uintptr_t)host_base);
+    if (it == c->attached.end()) return fail(APK_DECLINE_NOT_ATTACHED, "apk_detach: mapping is not attached");
+    if (int rc = set_device(c)) return rc;
+    HIP_TRY(hipStreamSynchronize(c->stream));
+    HIP_TRY(hipFree(it->second.dev));
+    c->attached.erase(it);
+    return APK_OK;
+}
+int apk_resolve(apk_ctx* c, const void* host_ptr, size_t len, void** dev_out) {
+    if (!c || !dev_out) return fail(APK_DECLINE_NULL, "apk_resolve: NULL argument");
+    std::lock_guard<std::mutex> lock(c->mu);
+    uintptr_t p = (uintptr_t)host_ptr;
+    auto it = c->attached.upper_bound(p);
+    if (it != c->attached.begin()) {
+        --it;
+        if (p >= it->first && p - it->first <= it->second.len && len <= it->second.len - (p - it->first)) {
+            *dev_out = (char*)it->second.dev + (p - it->first);
+            return APK_OK;
+        }
+    }
+    *dev_out = nullptr;
+    return fail(APK_DECLINE_NOT_ATTACHED, "apk_resolve: foreign memory (not inside an attached mapping)");
+}
+
+int apk_timer_begin(apk_ctx* c) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_timer_begin: ctx is NULL");
+    std::lock_guard<std::mutex> lock(c->mu);
+    HIP_TRY(hipEventRecord(c->ev0, c->stream));
+    return APK_OK;
+}
+int apk_timer_end(apk_ctx* c, float* ms_out) {
+    if (!c || !ms_out) return fail(APK_DECLINE_NULL, "apk_timer_end: NULL argument");
+    std::lock_guard<std::mutex> lock(c->mu);
+    HIP_TRY(hipEventRecord(c->ev1, c->stream));
+    uint64_t t0 = now_ns();
+    HIP_TRY(hipEventSynchronize(c->ev1));
+    c->wait_ns += now_ns() - t0;
+    HIP_TRY(hipEventElapsedTime(ms_out, c->ev0, c->ev1));
+    return APK_OK;
+}
+
+/* ------------------------------------------------------------------- ops */
+
+int apk_swiglu(apk_ctx* c, void* gate, const void* up, size_t n, int dtype) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_swiglu: ctx is NULL");
+    CallScope s(c);
+    const int es = elem_size(dtype);
+    if (!es) return fail(APK_DECLINE_UNSUPPORTED, "apk_swiglu: dtype %d", dtype);
+    if (n == 0) return APK_OK;
+    if (!gate || !up) return fail(APK_DECLINE_NULL, "apk_swiglu: NULL tensor");
+    if (!aligned16(gate) || !aligned16(up)) return fail(APK_DECLINE_SHAPE, "apk_swiglu: tensors must be 16-byte aligned");
+    if (int rc = set_device(c)) return rc;
+    const uint64_t vec = 16 / es, nvec = n / vec;
+    const unsigned block = 256, per_block = block * 4;
+    uint64_t grid = (nvec + per_block - 1) / per_block;
+    if (grid == 0) grid = 1;
+    if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_swiglu: n too large");
+    uint64_t n64 = n;
+    void* args[] = {&gate, &up, &n64};
+    return launch(c, dtype == APK_F32 ? K_SWIGLU_F32 : K_SWIGLU_F16, (unsigned)grid, block, 0, args);
+}
+
+int apk_add_rmsnorm_rows(apk_ctx* c, void* x, const void* delta, void* h, const float* gamma, size_t n, size_t rows,
+                         float eps, int dtype) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_add_rmsnorm_rows: ctx is NULL");
+    CallScope s(c);
+    const int es = elem_size(dtype);
+    if (!es) return fail(APK_DECLINE_UNSUPPORTED, "apk_add_rmsnorm_rows: dtype %d", dtype);
+    if (rows == 0) return APK_OK;
+    if (!x || !h || !gamma) return fail(APK_DECLINE_NULL, "apk_add_rmsnorm_rows: NULL tensor");
+    const size_t vec = 16 / es;
+    if (n == 0 || n % vec) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: n=%zu is not a multiple of %zu", n, vec);
+    if (!aligned16(x) || !aligned16(h) || !aligned16(gamma) || (delta && !aligned16(delta)))
+        return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: tensors must be 16-byte aligned");
+    if (rows > 0x7fffffffu || n > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: too large");
+    const size_t nchunks = n / vec;
+    // fewest tiles per lane that keep the workgroup within 640 lanes (10 waves):
+    // the row stays in registers and several workgroups share a CU.
+    int nch = 1;
+    while (nch < 8 && (nchunks + nch - 1) / nch > 640) nch *= 2;
+    size_t threads = (nchunks + nch - 1) / nch;
+    if (threads > 1024) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: row of %zu elements is too long", n);
+    threads = (threads + 63) / 64 * 64;
+    const int base = dtype == APK_F32 ? K_ADDNORM_F32_C1 : K_ADDNORM_F16_C1;
+    const int which = base + (nch == 1 ? 0 : nch == 2 ? 1 : nch == 4 ? 2 : 3);
+    if (int rc = set_device(c)) return rc;
+    int n_i = (int)n;
+    void* args[] = {&x, &delta, &h, &gamma, &n_i, &eps};
+    return launch(c, (Kernel)which, (unsigned)rows, (unsigned)threads, 0, args);
+}
+
+int apk_qknorm_rope_neox(apk_ctx* c, void* q, void* k, const float* qw, const float* kw, const float* rope,
+                         size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim, float eps, int dtype) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_qknorm_rope_neox: ctx is NULL");
+    CallScope s(c);
+    const int es = elem_size(dtype);
+    if (!es) return fail(APK_DECLINE_UNSUPPORTED, "apk_qknorm_rope_neox: dtype %d", dtype);
+    if (head_dim != 64 && head_dim != 128 && head_dim != 256)
+        return fail(APK_DECLINE_UNSUPPORTED, "apk_qknorm_rope_neox: head_dim %zu", head_dim);
+    if (rot_dim != head_dim)
+        return fail(APK_DECLINE_UNSUPPORTED, "apk_qknorm_rope_neox: partial rotary (rot_dim %zu of %zu)", rot_dim, head_dim);
+    if (rows == 0 || n_q + n_kv == 0) return APK_OK;
+    if ((n_q && !q) || (n_kv && !k) || !rope) return fail(APK_DECLINE_NULL, "apk_qknorm_rope_neox: NULL tensor");
+    if ((q && !aligned16(q)) || (k && !aligned16(k)) || !aligned16(rope) || (qw && !aligned16(qw)) || (kw && !aligned16(kw)))
+        return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_neox: tensors must be 16-byte aligned");
+    if (rows > 0x7fffffffu || n_q > 65535 || n_kv > 65535) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_neox: too large");
+    const uint64_t lanes = (uint64_t)rows * (n_q + n_kv) * (head_dim / 16);
+    const unsigned block = 256;
+    const uint64_t grid = (lanes + block - 1) / block;
+    if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_neox: too large");
+    const int hd_i = head_dim == 64 ? 0 : head_dim == 128 ? 1 : 2;
+    const int which = (dtype == APK_F32 ? K_QKROPE_F32_64 : K_QKROPE_F16_64) + hd_i;
+    if (int rc = set_device(c)) return rc;
+    int rows_i = (int)rows, nq_i = (int)n_q, nkv_i = (int)n_kv;
+    void* args[] = {&q, &k, &qw, &kw, &rope, &rows_i, &nq_i, &nkv_i, &eps};
+    return launch(c, (Kernel)which, (unsigned)grid, block, 0, args);
+}
+
+int apk_rope_table(apk_ctx* c, const uint32_t* positions, const float* inv_freq, size_t rows, size_t half, float* table) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_rope_table: ctx is NULL");
+    CallScope s(c);
+    if (rows == 0 || half == 0) return APK_OK;
+    if (!positions || !inv_freq || !table) return fail(APK_DECLINE_NULL, "apk_rope_table: NULL tensor");
+    if (rows > 0x7fffffffu || half > 0x7fffffffu || rows * half > 0x7fffffffull * 256)
+        return fail(APK_DECLINE_SHAPE, "apk_rope_table: too large");
+    if (int rc = set_device(c)) return rc;
+    int rows_i = (int)rows, half_i = (int)half;
+    const uint64_t grid = ((uint64_t)rows * half + 255) / 256;
+    void* args[] = {&positions, &inv_freq, &rows_i, &half_i, &table};
+    return launch(c, K_ROPE_TABLE, (unsigned)grid, 256, 0, args);
+}
+
+static int embed_common(apk_ctx* c, int fmt, const void* table, size_t vocab, size_t n_in, const uint32_t* ids_dev,
+                        size_t t, void* out, int out_dtype) {
+    if (!apk_can_embed(fmt, n_in)) return fail(APK_DECLINE_UNSUPPORTED, "apk_embed_rows: fmt %d / n_in %zu", fmt, n_in);
+    if (!elem_size(out_dtype)) return fail(APK_DECLINE_UNSUPPORTED, "apk_embed_rows: out_dtype %d", out_dtype);
+    if (t == 0) return APK_OK;
+    if (!table || !ids_dev || !out) return fail(APK_DECLINE_NULL, "apk_embed_rows: NULL tensor");
+    if (!aligned16(table) || !aligned16(out)) return fail(APK_DECLINE_SHAPE, "apk_embed_rows: table/out must be 16-byte aligned");
+    if (vocab == 0 || vocab > 0xffffffffu || n_in > 0x7fffffffu || t > 0x7fffffffu)
+        return fail(APK_DECLINE_SHAPE, "apk_embed_rows: sizes out of range");
+    if (int rc = set_device(c)) return rc;
+    uint32_t vocab32 = (uint32_t)vocab;
+    int n_i = (int)n_in, t_i = (int)t;
+    if (fmt == APK_FMT_Q4K) {
+        const uint64_t lanes = (uint64_t)t * (n_in / 256) * 8;
+        const uint64_t grid = (lanes + 255) / 256;
+        if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_embed_rows: too large");
+        void* args[] = {&table, &vocab32, &n_i, &ids_dev, &t_i, &out, &c->fault_dev};
+        return launch(c, out_dtype == APK_F32 ? K_EMBED_Q4K_F32 : K_EMBED_Q4K_F16, (unsigned)grid, 256, 0, args);
+    }
+    // Q8_0: one workgroup per row, the row staged in LDS
+    const size_t row_bytes = n_in / 32 * 34;
+    const size_t shmem = row_bytes + 32;
+    if (shmem > 64 * 1024) return fail(APK_DECLINE_SHAPE, "apk_embed_rows: Q8_0 row of %zu elements is too long", n_in);
+    size_t threads = (n_in / 8 + 63) / 64 * 64;
+    if (threads > 1024) threads = 1024;
+    uint64_t table_bytes = (uint64_t)vocab * row_bytes;
+    void* args[] = {&table, &table_bytes, &vocab32, &n_i, &ids_dev, &out, &c->fault_dev};
+    return launch(c, out_dtype == APK_F32 ? K_EMBED_Q8_0_F32 : K_EMBED_Q8_0_F16, (unsigned)t, (unsigned)threads,
+                  (unsigned)shmem, args);
+}
+
+int apk_embed_rows(apk_ctx* c, int fmt, const void* table, size_t vocab, size_t n_in, const uint32_t* ids, size_t t,
+                   void* out, int out_dtype) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_embed_rows: ctx is NULL");
+    CallScope s(c);
+    return embed_common(c, fmt, table, vocab, n_in, ids, t, out, out_dtype);
+}
+
+int apk_embed_rows_host_ids(apk_ctx* c, int fmt, const void* table, size_t vocab, size_t n_in,
+                            const uint32_t* ids_host, size_t t, void* out, int out_dtype) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_embed_rows_host_ids: ctx is NULL");
+    CallScope s(c);
+    if (t == 0) return APK_OK;
+    if (!ids_host) return fail(APK_DECLINE_NULL, "apk_embed_rows_host_ids: ids is NULL");
+    for (size_t i = 0; i < t; i++)
+        if (ids_host[i] >= vocab)
+            return fail(APK_DECLINE_RANGE, "apk_embed_rows_host_ids: token %u at %zu >= vocab %zu", ids_host[i], i, vocab);
+    if (int rc = set_device(c)) return rc;
+    if (t > c->ids_stage_cap) {
+        // the previous staging buffer may still be read by an enqueued copy
+        HIP_TRY(hipStreamSynchronize(c->stream));
+        if (c->ids_stage_dev) (void)hipFree(c->ids_stage_dev);
+        if (c->ids_stage_host) (void)hipHostFree(c->ids_stage_host);
+        c->ids_stage_dev = nullptr;
+        c->ids_stage_host = nullptr;
+        c->ids_stage_cap = 0;
+        size_t cap = t < 4096 ? 4096 : t;
+        HIP_TRY(hipHostMalloc((void**)&c->ids_stage_host, cap * 4, hipHostMallocDefault));
+        HIP_TRY(hipMalloc((void**)&c->ids_stage_dev, cap * 4));
+        c->ids_stage_cap = cap;
+    } else {
+        // the pinned buffer is reused: wait until the previous copy out of it has run
+        HIP_TRY(hipStreamSynchronize(c->stream));
+    }
+    memcpy(c->ids_stage_host, ids_host, t * 4);
+    HIP_TRY(hipMemcpyAsync(c->ids_stage_dev, c->ids_stage_host, t * 4, hipMemcpyHostToDevice, c->stream));
+    return embed_common(c, fmt, table, vocab, n_in, c->ids_stage_dev, t, out, out_dtype);
+}
+
+int apk_route_topk(apk_ctx* c, const float* logits, const float* bias, size_t rows, size_t n_expert, size_t k, int norm,
+                   float scale, int sigmoid, uint32_t* ids, float* w) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_route_topk: ctx is NULL");
+    CallScope s(c);
+    if (n_expert == 0 || n_expert > 256) return fail(APK_DECLINE_UNSUPPORTED, "apk_route_topk: n_expert %zu (1..256)", n_expert);
+    if (k == 0 || k > n_expert || k > 64) return fail(APK_DECLINE_UNSUPPORTED, "apk_route_topk: k %zu", k);
+    if (rows == 0) return APK_OK;
+    if (!logits || !ids || !w) return fail(APK_DECLINE_NULL, "apk_route_topk: NULL tensor");
+    if (rows > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_route_topk: too large");
+    if (int rc = set_device(c)) return rc;
+    int rows_i = (int)rows, ne_i = (int)n_expert, k_i = (int)k;
+    const unsigned block = 256, per_block = block / 64;
+    const uint64_t grid = (rows + per_block - 1) / per_block;
+    void* args[] = {&logits, &bias, &rows_i, &ne_i, &k_i, &norm, &scale, &sigmoid, &ids, &w};
+    return launch(c, K_ROUTE_TOPK, (unsigned)grid, block, 0, args);
+}
+
+int apk_moe_permute(apk_ctx* c, const uint32_t* ids, const float* w, size_t rows, size_t k, size_t n_expert,
+                    uint32_t* table, uint32_t* n_used, uint32_t* tok, uint32_t* tok_off, uint32_t* hit_row, float* hit_w) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_moe_permute: ctx is NULL");
+    CallScope s(c);
+    if (n_expert == 0 || n_expert > 1024) return fail(APK_DECLINE_UNSUPPORTED, "apk_moe_permute: n_expert %zu (1..1024)", n_expert);
+    if (k == 0 || k > n_expert) return fail(APK_DECLINE_UNSUPPORTED, "apk_moe_permute: k %zu", k);
+    if (!table || !n_used || !tok_off) return fail(APK_DECLINE_NULL, "apk_moe_permute: NULL tensor");
+    if (rows && (!ids || !w || !tok || !hit_row || !hit_w)) return fail(APK_DECLINE_NULL, "apk_moe_permute: NULL tensor");
+    if (rows * k >= 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_moe_permute: rows*k too large");
+    if (int rc = set_device(c)) return rc;
+    int rows_i = (int)rows, k_i = (int)k, ne_i = (int)n_expert;
+    void* args[] = {&ids, &w, &rows_i, &k_i, &ne_i, &table, &n_used, &tok, &tok_off, &hit_row, &hit_w, &c->fault_dev};
+    return launch(c, K_MOE_PERMUTE, (unsigned)n_expert, 512, 0, args);
+}
+
+int apk_gather_rows(apk_ctx* c, const void* src, const uint32_t* tok, size_t src_rows, size_t total_rows, size_t cols,
+                    void* dst, int dtype) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_gather_rows: ctx is NULL");
+    CallScope s(c);
+    const int es = elem_size(dtype);
+    if (!es) return fail(APK_DECLINE_UNSUPPORTED, "apk_gather_rows: dtype %d", dtype);
+    if (total_rows == 0 || cols == 0) return APK_OK;
+    if (!src || !tok || !dst) return fail(APK_DECLINE_NULL, "apk_gather_rows: NULL tensor");
+    if ((cols * es) % 16 || !aligned16(src) || !aligned16(dst))
+        return fail(APK_DECLINE_SHAPE, "apk_gather_rows: rows must be whole 16-byte tiles");
+    if (total_rows > 0x7fffffffu || src_rows > 0xffffffffu || cols * es / 16 > 0x7fffffffu)
+        return fail(APK_DECLINE_SHAPE, "apk_gather_rows: too large");
+    if (int rc = set_device(c)) return rc;
+    uint32_t src_rows32 = (uint32_t)src_rows;
+    int row_vecs = (int)(cols * es / 16);
+    void* args[] = {&src, &tok, &src_rows32, &row_vecs, &dst, &c->fault_dev};
+    return launch(c, K_GATHER_ROWS, (unsigned)total_rows, 256, 0, args);
+}
+
+int apk_copy(apk_ctx* c, const void* src, void* dst, size_t bytes) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_copy: ctx is NULL");
+    CallScope s(c);
+    if (bytes == 0) return APK_OK;
+    if (!src || !dst) return fail(APK_DECLINE_NULL, "apk_copy: NULL tensor");
+    if (bytes % 16 || !aligned16(src) || !aligned16(dst)) return fail(APK_DECLINE_SHAPE, "apk_copy: whole 16-byte tiles only");
+    if (int rc = set_device(c)) return rc;
+    uint64_t nvec = bytes / 16;
+    const uint64_t grid = (nvec + 1023) / 1024;
+    if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_copy: too large");
+    void* args[] = {&src, &dst, &nvec};
+    return launch(c, K_COPY, (unsigned)grid, 256, 0, args);
+}
+
+}  // extern "C"
+#pragma GCC visibility pop

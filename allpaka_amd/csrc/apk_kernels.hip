@@ -1,0 +1,701 @@
+// gfx950 (CDNA4, MI355X) device code for allpaka's fused per-layer ops.
+//
+// Built with `hipcc --genco --offload-arch=gfx950 -ffp-contract=off` into one
+// code object that the host library embeds and loads with hipModuleLoadData.
+// Every kernel here is HBM-bound: wave64, 128-bit global accesses, DPP/shuffle
+// reductions inside a wave, LDS only for cross-wave sums and byte staging.
+// No MFMA: nothing on this path is a contraction.
+//
+// Arithmetic contract (what the CPU reference computes, op for op):
+//   * -ffp-contract=off for the whole file: a*b-c stays two rounded f32 ops,
+//     as in the reference's Rust (dequant.rs:221-228, rope.rs:75-80).
+//   * RMS statistics are accumulated and applied in f64 (norm.rs:115-187):
+//     out = ((x as f64 * scale) as f32) * w.
+//   * fp16 activations (a storage form the reference does not have) are
+//     widened to f32 on load and rounded once (RNE) on store.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16_t;
+
+#define DEV static __device__ __forceinline__
+
+// Fault bits raised through the context's device status word.
+#define APK_FAULT_TOKEN_RANGE 1u   // embedding id >= vocab
+#define APK_FAULT_EXPERT_RANGE 2u  // routed expert id >= n_expert
+#define APK_FAULT_ROW_RANGE 4u     // gather index >= source rows
+
+DEV float h2f(uint32_t bits16) { return (float)__builtin_bit_cast(f16_t, (uint16_t)bits16); }
+DEV uint32_t f2h(float f) { return (uint32_t)__builtin_bit_cast(uint16_t, (f16_t)f); }
+
+// ----------------------------------------------------------- 16-byte tile IO
+template <typename T> struct io;
+template <> struct io<float> {
+    static constexpr int VEC = 4;
+    DEV void load(const float* p, float* v) {
+        f32x4 t = *(const f32x4*)p;
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    }
+    DEV void load_nt(const float* p, float* v) {
+        f32x4 t = __builtin_nontemporal_load((const f32x4*)p);
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    }
+    DEV void store(float* p, const float* v) {
+        f32x4 t = {v[0], v[1], v[2], v[3]};
+        *(f32x4*)p = t;
+    }
+    DEV void store_nt(float* p, const float* v) {
+        f32x4 t = {v[0], v[1], v[2], v[3]};
+        __builtin_nontemporal_store(t, (f32x4*)p);
+    }
+};
+template <> struct io<f16_t> {
+    static constexpr int VEC = 8;
+    DEV void unpack(u32x4 t, float* v) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            v[2 * i] = h2f(t[i] & 0xffffu);
+            v[2 * i + 1] = h2f(t[i] >> 16);
+        }
+    }
+    DEV u32x4 pack(const float* v) {
+        u32x4 t;
+#pragma unroll
+        for (int i = 0; i < 4; i++) t[i] = f2h(v[2 * i]) | (f2h(v[2 * i + 1]) << 16);
+        return t;
+    }
+    DEV void load(const f16_t* p, float* v) { unpack(*(const u32x4*)p, v); }
+    DEV void load_nt(const f16_t* p, float* v) { unpack(__builtin_nontemporal_load((const u32x4*)p), v); }
+    DEV void store(f16_t* p, const float* v) { *(u32x4*)p = pack(v); }
+    DEV void store_nt(f16_t* p, const float* v) { __builtin_nontemporal_store(pack(v), (u32x4*)p); }
+};
+
+DEV double wave_sum_f64(double v, int width) {
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1)
+        if (o < width) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// =========================================================================
+// SwiGLU: gate[i] = silu(gate[i]) * up[i], silu(x) = x / (1 + exp(-x))
+// (activation.rs:19-22, :116-119).  Pure stream: 2 reads + 1 write / element.
+// =========================================================================
+template <typename T> DEV float silu_mul(float g, float u);
+// f32 activations: accurate expf and IEEE division, same operation order as
+// the reference.
+template <> __device__ __forceinline__ float silu_mul<float>(float g, float u) { return g / (1.0f + expf(-g)) * u; }
+// fp16 activations: the result is rounded to 11 bits, so the hardware exp2 /
+// rcp approximations (about 1 ulp of f32 each) are far inside the 2-ulp-of-fp16
+// budget and keep the kernel under its ALU ceiling.
+template <> __device__ __forceinline__ float silu_mul<f16_t>(float g, float u) {
+    float e = __builtin_amdgcn_exp2f(g * -1.4426950408889634f);
+    return g * __builtin_amdgcn_rcpf(1.0f + e) * u;
+}
+
+template <typename T, int UNR> DEV void swiglu_body(T* gate, const T* up, uint64_t n) {
+    constexpr int VEC = io<T>::VEC;
+    const uint64_t nvec = n / VEC;
+    const uint64_t base = (uint64_t)blockIdx.x * (blockDim.x * UNR) + threadIdx.x;
+    float g[UNR][VEC], u[UNR][VEC];
+#pragma unroll
+    for (int j = 0; j < UNR; j++) {
+        uint64_t c = base + (uint64_t)j * blockDim.x;
+        if (c < nvec) {
+            io<T>::load_nt(gate + c * VEC, g[j]);
+            io<T>::load_nt(up + c * VEC, u[j]);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < UNR; j++) {
+        uint64_t c = base + (uint64_t)j * blockDim.x;
+        if (c < nvec) {
+#pragma unroll
+            for (int i = 0; i < VEC; i++) g[j][i] = silu_mul<T>(g[j][i], u[j][i]);
+            io<T>::store_nt(gate + c * VEC, g[j]);
+        }
+    }
+    // ragged tail (n not a multiple of the 16-byte tile): last block, scalar
+    if (blockIdx.x == gridDim.x - 1) {
+        for (uint64_t i = nvec * VEC + threadIdx.x; i < n; i += blockDim.x)
+            gate[i] = (T)silu_mul<T>((float)gate[i], (float)up[i]);
+    }
+}
+#define APK_SWIGLU_UNR 4
+extern "C" __global__ __launch_bounds__(256) void apk_swiglu_f32(float* gate, const float* up, uint64_t n) {
+    swiglu_body<float, APK_SWIGLU_UNR>(gate, up, n);
+}
+extern "C" __global__ __launch_bounds__(256) void apk_swiglu_f16(f16_t* gate, const f16_t* up, uint64_t n) {
+    swiglu_body<f16_t, APK_SWIGLU_UNR>(gate, up, n);
+}
+
+// =========================================================================
+// Residual add + RMSNorm over rows (blas.rs:105-178 then norm.rs:193-269):
+//   x' = x + delta  (written back when delta != null)
+//   h  = ((x' as f64 * scale) as f32) * gamma,  scale = 1/sqrt(mean(x'^2)+eps)
+// One workgroup per row; each lane keeps its NCH 16-byte tiles of the row in
+// registers between the sum of squares and the scaling pass, so the row is
+// read from HBM once.  Wave sums by shuffle, cross-wave through LDS.
+// =========================================================================
+template <typename T, int NCH>
+DEV void add_rmsnorm_body(T* x, const T* delta, T* h, const float* gamma, int n, float eps) {
+    constexpr int VEC = io<T>::VEC;
+    __shared__ double part[16];
+    const int nchunks = n / VEC;
+    const uint64_t row = blockIdx.x;
+    T* xr = x + row * (uint64_t)n;
+    T* hr = h + row * (uint64_t)n;
+    const T* dr = delta ? delta + row * (uint64_t)n : nullptr;
+
+    float v[NCH][VEC];
+    float d[NCH][VEC];
+#pragma unroll
+    for (int j = 0; j < NCH; j++) {
+        int c = threadIdx.x + j * blockDim.x;
+        if (c < nchunks) {
+            io<T>::load_nt(xr + c * VEC, v[j]);
+            if (dr) io<T>::load_nt(dr + c * VEC, d[j]);
+        }
+    }
+    double ss = 0.0;
+#pragma unroll
+    for (int j = 0; j < NCH; j++) {
+        int c = threadIdx.x + j * blockDim.x;
+        if (c < nchunks) {
+            if (dr) {
+#pragma unroll
+                for (int i = 0; i < VEC; i++) v[j][i] = v[j][i] + d[j][i];
+                io<T>::store(xr + c * VEC, v[j]);
+            }
+#pragma unroll
+            for (int i = 0; i < VEC; i++) ss = __builtin_fma((double)v[j][i], (double)v[j][i], ss);
+        }
+    }
+    ss = wave_sum_f64(ss, 64);
+    const int nwaves = (blockDim.x + 63) >> 6;
+    if (nwaves > 1) {
+        if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+        __syncthreads();
+        ss = 0.0;
+        for (int w = 0; w < nwaves; w++) ss += part[w];
+    }
+    const double scale = 1.0 / sqrt(ss / (double)n + (double)eps);
+#pragma unroll
+    for (int j = 0; j < NCH; j++) {
+        int c = threadIdx.x + j * blockDim.x;
+        if (c < nchunks) {
+            float g[VEC], o[VEC];
+#pragma unroll
+            for (int q = 0; q < VEC; q += 4) io<float>::load(gamma + c * VEC + q, g + q);
+#pragma unroll
+            for (int i = 0; i < VEC; i++) o[i] = (float)((double)v[j][i] * scale) * g[i];
+            io<T>::store_nt(hr + c * VEC, o);
+        }
+    }
+}
+#define APK_ADDNORM(NAME, T, NCH)                                                                                  \
+    extern "C" __global__ __launch_bounds__(1024) void NAME(T* x, const T* delta, T* h, const float* gamma, int n, \
+                                                            float eps) {                                           \
+        add_rmsnorm_body<T, NCH>(x, delta, h, gamma, n, eps);                                                      \
+    }
+APK_ADDNORM(apk_add_rmsnorm_f32_c1, float, 1)
+APK_ADDNORM(apk_add_rmsnorm_f32_c2, float, 2)
+APK_ADDNORM(apk_add_rmsnorm_f32_c4, float, 4)
+APK_ADDNORM(apk_add_rmsnorm_f32_c8, float, 8)
+APK_ADDNORM(apk_add_rmsnorm_f16_c1, f16_t, 1)
+APK_ADDNORM(apk_add_rmsnorm_f16_c2, f16_t, 2)
+APK_ADDNORM(apk_add_rmsnorm_f16_c4, f16_t, 4)
+APK_ADDNORM(apk_add_rmsnorm_f16_c8, f16_t, 8)
+
+// =========================================================================
+// Per-head QK-norm + NeoX RoPE, in place on q [rows, n_q*HD] and k [rows, n_kv*HD]
+// (caller loop attention.rs:131-165: rmsnorm(head, w, eps) then the NeoX
+// rotation with the row's [sin, cos] table, rope.rs:70-81).
+// HD/16 lanes own one head: lane l holds elements [8l, 8l+8) of the first half
+// and their NeoX partners [HD/2+8l, HD/2+8l+8), so the rotation needs no
+// cross-lane traffic and every global access is a 16-byte tile inside a
+// 128-byte run.  The sum of squares crosses only those HD/16 lanes.
+// =========================================================================
+template <typename T, int HD>
+DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv,
+                          float eps) {
+    constexpr int LPH = HD / 16;  // lanes per head
+    constexpr int HALF = HD / 2;
+    const uint64_t gl = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const uint64_t gh = gl / LPH;
+    const int l = (int)(gl % LPH);
+    const int hpr = n_q + n_kv;
+    const uint64_t total = (uint64_t)rows * hpr;
+    const bool live = gh < total;
+    const uint64_t row = live ? gh / hpr : 0;
+    const int hh = live ? (int)(gh % hpr) : 0;
+    const bool is_q = hh < n_q;
+    T* head = is_q ? q + (row * n_q + hh) * HD : k + (row * n_kv + (hh - n_q)) * HD;
+    const float* w = is_q ? qw : kw;
+
+    float a[8], b[8];
+    if (live) {
+        if constexpr (sizeof(T) == 2) {
+            io<T>::load_nt(head + 8 * l, a);
+            io<T>::load_nt(head + HALF + 8 * l, b);
+        } else {
+            io<T>::load_nt(head + 8 * l, a);
+            io<T>::load_nt(head + 8 * l + 4, a + 4);
+            io<T>::load_nt(head + HALF + 8 * l, b);
+            io<T>::load_nt(head + HALF + 8 * l + 4, b + 4);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; i++) a[i] = b[i] = 0.0f;
+    }
+    // [sin, cos] pairs of this row for i in [8l, 8l+8): 16 consecutive floats
+    float sc[16];
+    if (live) {
+        const float* t = rope + (row * HALF + 8 * l) * 2;
+#pragma unroll
+        for (int i = 0; i < 16; i += 4) io<float>::load(t + i, sc + i);
+    }
+    if (w != nullptr) {  // uniform across the lanes of a head (and nearly always the wave)
+        float wa[8], wb[8];
+#pragma unroll
+        for (int i = 0; i < 8; i += 4) {
+            io<float>::load(w + 8 * l + i, wa + i);
+            io<float>::load(w + HALF + 8 * l + i, wb + i);
+        }
+        double ss = 0.0;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            ss = __builtin_fma((double)a[i], (double)a[i], ss);
+            ss = __builtin_fma((double)b[i], (double)b[i], ss);
+        }
+        ss = wave_sum_f64(ss, LPH);
+        const double scale = 1.0 / sqrt(ss / (double)HD + (double)eps);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            a[i] = (float)((double)a[i] * scale) * wa[i];
+            b[i] = (float)((double)b[i] * scale) * wb[i];
+        }
+    }
+    if (live) {
+        float oa[8], ob[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const float s = sc[2 * i], c = sc[2 * i + 1];
+            oa[i] = a[i] * c - b[i] * s;
+            ob[i] = a[i] * s + b[i] * c;
+        }
+        if constexpr (sizeof(T) == 2) {
+            io<T>::store_nt(head + 8 * l, oa);
+            io<T>::store_nt(head + HALF + 8 * l, ob);
+        } else {
+            io<T>::store_nt(head + 8 * l, oa);
+            io<T>::store_nt(head + 8 * l + 4, oa + 4);
+            io<T>::store_nt(head + HALF + 8 * l, ob);
+            io<T>::store_nt(head + HALF + 8 * l + 4, ob + 4);
+        }
+    }
+}
+#define APK_QKROPE(NAME, T, HD)                                                                                        \
+    extern "C" __global__ __launch_bounds__(256) void NAME(T* q, T* k, const float* qw, const float* kw,               \
+                                                           const float* rope, int rows, int n_q, int n_kv, float eps) { \
+        qknorm_rope_body<T, HD>(q, k, qw, kw, rope, rows, n_q, n_kv, eps);                                             \
+    }
+APK_QKROPE(apk_qknorm_rope_f32_hd64, float, 64)
+APK_QKROPE(apk_qknorm_rope_f32_hd128, float, 128)
+APK_QKROPE(apk_qknorm_rope_f32_hd256, float, 256)
+APK_QKROPE(apk_qknorm_rope_f16_hd64, f16_t, 64)
+APK_QKROPE(apk_qknorm_rope_f16_hd128, f16_t, 128)
+APK_QKROPE(apk_qknorm_rope_f16_hd256, f16_t, 256)
+
+// RoPE table rows from per-row positions (rope.rs:18-22, session.rs:34-50):
+// table[r][i] = [sin, cos]((pos[r] as f32) * inv_freq[i]).  One f32 rounding of
+// the angle, then fully range-reduced sincosf (positions reach 32767 rad).
+extern "C" __global__ __launch_bounds__(256) void apk_rope_table(const uint32_t* pos, const float* inv_freq, int rows,
+                                                                int half, float* table) {
+    const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (uint64_t)rows * half) return;
+    const float ang = (float)pos[i / half] * inv_freq[i % half];
+    float s, c;
+    sincosf(ang, &s, &c);
+    table[2 * i] = s;
+    table[2 * i + 1] = c;
+}
+
+// =========================================================================
+// Embedding rows: out[t, :] = dequant(table row ids[t])   (quantmat/mod.rs:75-89)
+// The dequant is fused into the gather; the id is read on the device.
+// An id >= vocab raises APK_FAULT_TOKEN_RANGE and leaves its row untouched.
+// =========================================================================
+template <typename TO> DEV void store8(TO* p, const float* v);
+template <> __device__ __forceinline__ void store8<float>(float* p, const float* v) {
+    io<float>::store_nt(p, v);
+    io<float>::store_nt(p + 4, v + 4);
+}
+template <> __device__ __forceinline__ void store8<f16_t>(f16_t* p, const float* v) { io<f16_t>::store_nt(p, v); }
+
+// Q4_K (dequant.rs:211-231): 144-byte super-block = d, dmin (f16), 12 packed
+// scale bytes, 128 quant bytes.  8 lanes per super-block; lane j owns 16 quant
+// bytes = 16 low-nibble outputs of sub-block 2p and 16 high-nibble outputs of
+// sub-block 2p+1 (p = j/2).  d*sc, dmin*mn, (d*sc)*q and the subtraction are
+// four separately rounded f32 operations.
+template <typename TO>
+DEV void embed_q4k_body(const uint8_t* table, uint32_t vocab, int n_in, const uint32_t* ids, int t_rows, TO* out,
+                        uint32_t* fault) {
+    const int nsb = n_in / 256;
+    const uint64_t gl = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const uint64_t per_row = (uint64_t)nsb * 8;
+    const uint64_t t = gl / per_row;
+    if (t >= (uint64_t)t_rows) return;
+    const int rem = (int)(gl % per_row);
+    const int sb = rem >> 3, j = rem & 7;
+    const uint32_t id = ids[t];
+    if (id >= vocab) {
+        if (rem == 0) atomicOr(fault, APK_FAULT_TOKEN_RANGE);
+        return;
+    }
+    const uint8_t* blk = table + (uint64_t)id * ((uint64_t)nsb * 144) + (uint64_t)sb * 144;
+    const u32x4 hdr = *(const u32x4*)blk;
+    const u32x4 qs = __builtin_nontemporal_load((const u32x4*)(blk + 16 + 16 * j));
+    const float d = h2f(hdr.x & 0xffffu), dmin = h2f(hdr.x >> 16);
+    // the 12 packed bytes are hdr.y, hdr.z, hdr.w (little endian)
+    const int p = j >> 1;
+    uint32_t sc1, mn1, sc2, mn2;
+    auto byte_at = [&](int i) -> uint32_t {
+        uint32_t w = i < 4 ? hdr.y : (i < 8 ? hdr.z : hdr.w);
+        return (w >> (8 * (i & 3))) & 0xffu;
+    };
+    auto scale_min = [&](int s, uint32_t& sc, uint32_t& mn) {
+        if (s < 4) {
+            sc = byte_at(s) & 63u;
+            mn = byte_at(s + 4) & 63u;
+        } else {
+            sc = (byte_at(s + 4) & 0xfu) | ((byte_at(s - 4) >> 6) << 4);
+            mn = (byte_at(s + 4) >> 4) | ((byte_at(s) >> 6) << 4);
+        }
+    };
+    scale_min(2 * p, sc1, mn1);
+    scale_min(2 * p + 1, sc2, mn2);
+    const float d_sc1 = d * (float)sc1, dm1 = dmin * (float)mn1;
+    const float d_sc2 = d * (float)sc2, dm2 = dmin * (float)mn2;
+    float lo[16], hi[16];
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            const uint32_t byte = (qs[w] >> (8 * b)) & 0xffu;
+            lo[4 * w + b] = d_sc1 * (float)(byte & 0xfu) - dm1;
+            hi[4 * w + b] = d_sc2 * (float)(byte >> 4) - dm2;
+        }
+    }
+    TO* o = out + t * (uint64_t)n_in + (uint64_t)sb * 256 + p * 64 + 16 * (j & 1);
+    store8<TO>(o, lo);
+    store8<TO>(o + 8, lo + 8);
+    store8<TO>(o + 32, hi);
+    store8<TO>(o + 40, hi + 8);
+}
+extern "C" __global__ __launch_bounds__(256) void apk_embed_q4k_f32(const uint8_t* table, uint32_t vocab, int n_in,
+                                                                   const uint32_t* ids, int t_rows, float* out,
+                                                                   uint32_t* fault) {
+    embed_q4k_body<float>(table, vocab, n_in, ids, t_rows, out, fault);
+}
+extern "C" __global__ __launch_bounds__(256) void apk_embed_q4k_f16(const uint8_t* table, uint32_t vocab, int n_in,
+                                                                   const uint32_t* ids, int t_rows, f16_t* out,
+                                                                   uint32_t* fault) {
+    embed_q4k_body<f16_t>(table, vocab, n_in, ids, t_rows, out, fault);
+}
+
+// Q8_0 (dequant.rs:94-126): 34-byte block = f16 scale + 32 int8; out = d * q.
+// Blocks are only 2-byte aligned, so one workgroup stages its row in LDS with
+// 16-byte loads (from the 16-byte-aligned address at or below the row start)
+// and each lane then decodes 8 outputs from LDS.  grid = rows, block = n_in/8
+// lanes (rounded up to a wave), looping when the row is longer than the block.
+template <typename TO>
+DEV void embed_q8_0_body(const uint8_t* table, uint64_t table_bytes, uint32_t vocab, int n_in, const uint32_t* ids,
+                         TO* out, uint32_t* fault) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t stage[];
+    const uint64_t t = blockIdx.x;
+    const uint32_t id = ids[t];
+    if (id >= vocab) {
+        if (threadIdx.x == 0) atomicOr(fault, APK_FAULT_TOKEN_RANGE);
+        return;
+    }
+    const uint64_t row_bytes = (uint64_t)(n_in / 32) * 34;
+    const uint64_t start = (uint64_t)id * row_bytes;
+    const uint64_t astart = start & ~(uint64_t)15;  // table base is 16-byte aligned
+    const int mis = (int)(start - astart);
+    const int nvec = (int)((mis + row_bytes + 15) / 16);
+    for (int i = threadIdx.x; i < nvec; i += blockDim.x) {
+        const uint64_t off = astart + (uint64_t)i * 16;
+        u32x4 v;
+        if (off + 16 <= table_bytes) {
+            v = __builtin_nontemporal_load((const u32x4*)(table + off));
+        } else {  // last tile of the last row: stay inside the table
+            uint32_t w[4] = {0, 0, 0, 0};
+            for (int b = 0; b < 16; b++)
+                if (off + b < table_bytes) w[b >> 2] |= (uint32_t)table[off + b] << (8 * (b & 3));
+            v = u32x4{w[0], w[1], w[2], w[3]};
+        }
+        *(u32x4*)(stage + i * 16) = v;
+    }
+    __syncthreads();
+    const int ngroups = n_in / 8;
+    for (int g = threadIdx.x; g < ngroups; g += blockDim.x) {
+        const int blk = g >> 2, qtr = g & 3;
+        const uint8_t* b = stage + mis + blk * 34;  // 2-byte aligned
+        const float d = h2f(*(const uint16_t*)b);
+        const uint16_t* qp = (const uint16_t*)(b + 2 + 8 * qtr);
+        float o[8];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t two = qp[i];
+            o[2 * i] = d * (float)(int8_t)(two & 0xffu);
+            o[2 * i + 1] = d * (float)(int8_t)(two >> 8);
+        }
+        store8<TO>(out + t * (uint64_t)n_in + (uint64_t)g * 8, o);
+    }
+}
+extern "C" __global__ __launch_bounds__(1024) void apk_embed_q8_0_f32(const uint8_t* table, uint64_t table_bytes,
+                                                                     uint32_t vocab, int n_in, const uint32_t* ids,
+                                                                     float* out, uint32_t* fault) {
+    embed_q8_0_body<float>(table, table_bytes, vocab, n_in, ids, out, fault);
+}
+extern "C" __global__ __launch_bounds__(1024) void apk_embed_q8_0_f16(const uint8_t* table, uint64_t table_bytes,
+                                                                     uint32_t vocab, int n_in, const uint32_t* ids,
+                                                                     f16_t* out, uint32_t* fault) {
+    embed_q8_0_body<f16_t>(table, table_bytes, vocab, n_in, ids, out, fault);
+}
+
+// =========================================================================
+// MoE router: per token softmax (or sigmoid) over n_expert <= 256 logits, top-k
+// by descending selection score with the LOWER INDEX winning ties, winners
+// renormalised (moe.rs:524-594).  One wave per token; lane l holds experts
+// l, l+64, l+128, l+192.  For softmax without bias the selection runs on the
+// raw logits (same order as the probabilities, no dependence on exp rounding).
+// =========================================================================
+DEV uint32_t total_order_key(float f) {  // f32::total_cmp as an unsigned key
+    int32_t b = __builtin_bit_cast(int32_t, f);
+    b ^= (int32_t)(((uint32_t)(b >> 31)) >> 1);
+    return (uint32_t)b ^ 0x80000000u;
+}
+DEV float wave_max_f32(float v) {
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+DEV float wave_sum_f32(float v) {
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+DEV uint64_t wave_max_u64(uint64_t v) {
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        uint64_t other = __shfl_xor(v, o, 64);
+        v = other > v ? other : v;
+    }
+    return v;
+}
+
+extern "C" __global__ __launch_bounds__(256) void apk_route_topk(const float* logits, const float* bias, int rows,
+                                                                int n_expert, int k, int norm, float scale,
+                                                                int sigmoid, uint32_t* ids, float* wout) {
+    const int lane = threadIdx.x & 63;
+    const uint64_t t = (uint64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (t >= (uint64_t)rows) return;  // whole wave exits together
+    const float* lr = logits + t * (uint64_t)n_expert;
+    float lg[4], score[4];
+    uint32_t key[4];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int e = lane + 64 * j;
+        lg[j] = e < n_expert ? lr[e] : -INFINITY;
+        if (e < n_expert) mx = fmaxf(mx, lg[j]);
+    }
+    if (!sigmoid) {
+        mx = wave_max_f32(mx);
+        float sum = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int e = lane + 64 * j;
+            score[j] = e < n_expert ? expf(lg[j] - mx) : 0.0f;
+            sum += score[j];
+        }
+        sum = wave_sum_f32(sum);
+        const float inv = 1.0f / sum;
+#pragma unroll
+        for (int j = 0; j < 4; j++) score[j] *= inv;
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; j++) score[j] = 1.0f / (1.0f + expf(-lg[j]));
+    }
+    const bool on_logits = !sigmoid && bias == nullptr;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int e = lane + 64 * j;
+        float sel = on_logits ? lg[j] : (bias != nullptr && e < n_expert ? score[j] + bias[e] : score[j]);
+        key[j] = total_order_key(sel);
+    }
+    uint32_t taken = 0;
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+        if (lane + 64 * j >= n_expert) taken |= 1u << j;
+    uint32_t my_id = 0;
+    float my_score = 0.0f, total = 0.0f;
+    for (int r = 0; r < k; r++) {
+        uint64_t best = 0;  // (key << 32) | ~index; 0 = nothing left on this lane
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            if (!(taken & (1u << j))) {
+                uint64_t cand = ((uint64_t)key[j] << 32) | (uint64_t)(0xffffffffu - (uint32_t)(lane + 64 * j));
+                best = cand > best ? cand : best;
+            }
+        }
+        best = wave_max_u64(best);
+        const uint32_t e = 0xffffffffu - (uint32_t)(best & 0xffffffffu);
+        const int owner = (int)(e & 63u), slot = (int)(e >> 6);
+        float s = 0.0f;
+        if (lane == owner) {
+            taken |= 1u << slot;
+            s = slot == 0 ? score[0] : (slot == 1 ? score[1] : (slot == 2 ? score[2] : score[3]));
+        }
+        s = __shfl(s, owner, 64);
+        total += s;  // best-first sequential f32 sum, as the reference's iterator sum
+        if (lane == r) {
+            my_id = e;
+            my_score = s;
+        }
+    }
+    if (lane < k) {
+        float w = (norm && total > 0.0f) ? my_score / total : (norm ? 1.0f / (float)k : my_score);
+        ids[t * (uint64_t)k + lane] = my_id;
+        wout[t * (uint64_t)k + lane] = w * scale;
+    }
+}
+
+// =========================================================================
+// Token -> expert grouping (moe.rs:229-271, prefill.rs:624-675), deterministic:
+// rows of an expert are in ascending token order, exactly the CPU order.
+// One workgroup per expert, no global atomics and no scratch memory:
+//   pass A  every workgroup histograms all rows*k picks in LDS (integer LDS
+//           atomics: the counts are order-independent) and derives its own
+//           row0 = sum of counts of lower experts and its index among the
+//           non-empty experts;
+//   pass B  walks the tokens in order, ranks the tokens that picked this expert
+//           with a ballot/popcount scan and writes tok[], hit_row[], hit_w[].
+// A token's hit list is ordered by ascending expert id: the slot of this expert
+// in it is the number of the token's picks with a smaller id.
+// =========================================================================
+#define APK_PERMUTE_THREADS 512
+extern "C" __global__ __launch_bounds__(APK_PERMUTE_THREADS) void apk_moe_permute(
+    const uint32_t* ids, const float* w, int rows, int k, int n_expert, uint32_t* table, uint32_t* n_used_out,
+    uint32_t* tok, uint32_t* tok_off, uint32_t* hit_row, float* hit_w, uint32_t* fault) {
+    __shared__ uint32_t hist[1024];
+    __shared__ uint32_t wave_tot[APK_PERMUTE_THREADS / 64];
+    __shared__ uint32_t s_row0, s_used;
+    const int e = blockIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    for (int i = tid; i < n_expert; i += blockDim.x) hist[i] = 0;
+    __syncthreads();
+    const int total = rows * k;
+    for (int i = tid; i < total; i += blockDim.x) {
+        const uint32_t id = ids[i];
+        if (id < (uint32_t)n_expert) atomicAdd(&hist[id], 1u);
+        else if (e == 0) atomicOr(fault, APK_FAULT_EXPERT_RANGE);
+    }
+    __syncthreads();
+    if (tid == 0) {
+        uint32_t r0 = 0, used = 0;
+        for (int i = 0; i < e; i++) {
+            r0 += hist[i];
+            used += hist[i] != 0;
+        }
+        s_row0 = r0;
+        s_used = used;
+    }
+    __syncthreads();
+    const uint32_t row0 = s_row0, mine = hist[e];
+    if (e == 0)
+        for (int t = tid; t <= rows; t += blockDim.x) tok_off[t] = (uint32_t)t * (uint32_t)k;
+    if (tid == 0) {
+        if (mine) {
+            table[3 * s_used] = (uint32_t)e;
+            table[3 * s_used + 1] = row0;
+            table[3 * s_used + 2] = mine;
+        }
+        if (e == n_expert - 1) *n_used_out = s_used + (mine != 0);
+    }
+    if (mine == 0) return;  // uniform for the workgroup
+    uint32_t running = 0;
+    for (int base = 0; base < rows; base += blockDim.x) {
+        const int t = base + tid;
+        int j_hit = -1, slot = 0;
+        if (t < rows) {
+            for (int j = 0; j < k; j++) {
+                const uint32_t id = ids[(uint64_t)t * k + j];
+                if (id == (uint32_t)e && j_hit < 0) j_hit = j;
+                slot += id < (uint32_t)e;
+            }
+        }
+        const bool flag = j_hit >= 0;
+        const uint64_t mask = __ballot(flag);
+        const uint32_t in_wave = (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
+        if (lane == 0) wave_tot[wv] = (uint32_t)__popcll(mask);
+        __syncthreads();
+        uint32_t before = 0, all = 0;
+        for (int i = 0; i < (int)(blockDim.x >> 6); i++) {
+            const uint32_t c = wave_tot[i];
+            before += i < wv ? c : 0;
+            all += c;
+        }
+        if (flag) {
+            const uint32_t r = row0 + running + before + in_wave;
+            tok[r] = (uint32_t)t;
+            hit_row[(uint64_t)t * k + slot] = r;
+            hit_w[(uint64_t)t * k + slot] = w[(uint64_t)t * k + j_hit];
+        }
+        running += all;
+        __syncthreads();
+    }
+}
+
+// Gathered activations in tok order (moe.rs:348-352): dst[r,:] = src[tok[r],:].
+// One workgroup per destination row, 16-byte tiles; row_vecs = row bytes / 16.
+extern "C" __global__ __launch_bounds__(256) void apk_gather_rows(const u32x4* src, const uint32_t* tok,
+                                                                 uint32_t src_rows, int row_vecs, u32x4* dst,
+                                                                 uint32_t* fault) {
+    const uint64_t r = blockIdx.x;
+    const uint32_t s = tok[r];
+    if (s >= src_rows) {
+        if (threadIdx.x == 0) atomicOr(fault, APK_FAULT_ROW_RANGE);
+        return;
+    }
+    const u32x4* sp = src + (uint64_t)s * row_vecs;
+    u32x4* dp = dst + r * row_vecs;
+    for (int c = threadIdx.x; c < row_vecs; c += 2 * blockDim.x) {
+        const int c2 = c + blockDim.x;
+        u32x4 a = sp[c], b;
+        if (c2 < row_vecs) b = sp[c2];
+        __builtin_nontemporal_store(a, dp + c);
+        if (c2 < row_vecs) __builtin_nontemporal_store(b, dp + c2);
+    }
+}
+
+// Reference stream for bandwidth calibration: dst = src, 16-byte tiles.
+extern "C" __global__ __launch_bounds__(256) void apk_copy(const u32x4* src, u32x4* dst, uint64_t nvec) {
+    const uint64_t base = (uint64_t)blockIdx.x * (blockDim.x * 4) + threadIdx.x;
+    u32x4 v[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        uint64_t c = base + (uint64_t)j * blockDim.x;
+        if (c < nvec) v[j] = __builtin_nontemporal_load(src + c);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        uint64_t c = base + (uint64_t)j * blockDim.x;
+        if (c < nvec) __builtin_nontemporal_store(v[j], dst + c);
+    }
+}

@@ -1,0 +1,198 @@
+/*
+ * libapk_hip.so -- C ABI of the MI355X (gfx950) implementation of allpaka's fused
+ * per-layer transformer ops.  This is the boundary an `allpaka_backend::gpu::hip`
+ * module (a sibling of gpu/metal, gpu/cuda and gpu/stub, selected in
+ * crates/allpaka-backend/src/gpu/mod.rs:13-26) binds through `extern "C"`.
+ *
+ * Conventions
+ *   * Every entry returns an int status and never aborts:
+ *       0   APK_OK
+ *       >0  declined (apk_decline): the request is outside what the device path
+ *           takes; nothing was launched, no caller memory was touched, and the
+ *           caller runs its CPU path -- the reference's "decline, never fail"
+ *           rule (gpu/stub.rs:37-217, accel.rs:69-102, gpu/types.rs:243-255).
+ *       <0  -(hipError_t): the HIP runtime failed.
+ *     apk_last_error() returns a thread-local description of the last non-zero
+ *     status.
+ *   * All tensor pointers are DEVICE pointers unless a name ends in `_host`.
+ *     Tensors are dense row-major.  Work is enqueued on the context's single
+ *     stream and is asynchronous; apk_sync() waits for it.  Calls on one context
+ *     serialise on an internal mutex, like the reference's process-wide backend
+ *     (gpu/cuda/runtime/device.rs:267, 944-948).
+ *   * dtype selects the ACTIVATION storage type: APK_F32 is the reference's only
+ *     activation type; APK_F16 stores activations as IEEE half (widen -> the
+ *     same f32/f64 arithmetic -> one round-to-nearest-even).  Norm weights,
+ *     RoPE tables, router logits and router weights are always f32.
+ *   * The device code object is embedded in the library and loaded with
+ *     hipModuleLoadData at apk_init; if that fails apk_init fails -- there is no
+ *     CPU fallback inside this library.
+ */
+#ifndef APK_HIP_H
+#define APK_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct apk_ctx apk_ctx;
+
+enum apk_dtype { APK_F32 = 0, APK_F16 = 1 };
+
+/* Positive statuses: why a request was declined (cf. DeclineReason, accel.rs:9-67). */
+enum apk_decline {
+    APK_OK = 0,
+    APK_DECLINE_UNSUPPORTED = 1, /* format / dtype / head_dim / n_expert the device path does not take */
+    APK_DECLINE_SHAPE = 2,       /* sizes inconsistent or not a whole number of blocks / 16-byte tiles  */
+    APK_DECLINE_NULL = 3,        /* a required pointer is NULL                                         */
+    APK_DECLINE_RANGE = 4,       /* an index is out of range (host-checked ids)                        */
+    APK_DECLINE_NO_DEVICE = 5,   /* no usable GPU / disabled by ALLPAKA_NO_GPU (capability.rs:58-61)   */
+    APK_DECLINE_NOT_ATTACHED = 6 /* host address is not inside an attached mapping                    */
+};
+
+/* Unified dequant format codes -- the exact integers of gpu::common::dq_fmt
+ * (crates/allpaka-backend/src/gpu/common.rs:47-61). */
+enum apk_dq_fmt {
+    APK_FMT_Q4K = 0, APK_FMT_Q5K = 1, APK_FMT_Q6K = 2, APK_FMT_Q8_0 = 3, APK_FMT_Q2K = 4,
+    APK_FMT_Q3K = 5, APK_FMT_Q5_0 = 6, APK_FMT_F16 = 7, APK_FMT_F32 = 8, APK_FMT_BF16 = 9
+};
+
+/* Bits of the device status word (apk_take_faults). */
+enum apk_fault {
+    APK_FAULT_TOKEN_RANGE = 1,  /* an embedding id >= vocab was met on the device  */
+    APK_FAULT_EXPERT_RANGE = 2, /* a routed expert id >= n_expert                  */
+    APK_FAULT_ROW_RANGE = 4     /* a gather index >= source rows                   */
+};
+
+/* ------------------------------------------------------------ life cycle ---- */
+
+/* Creates the backend on `device`: loads the embedded gfx950 code object
+ * (hipModuleLoadData), creates the stream.  Replaces the lazy singleton behind
+ * gpu::attach / init_error (gpu/stub.rs:37-55, gpu/cuda/mod.rs:41-44).
+ * ALLPAKA_NO_GPU set to a non-empty value other than "0" => APK_DECLINE_NO_DEVICE. */
+int apk_init(int device, apk_ctx** out);
+int apk_shutdown(apk_ctx* ctx);
+/* Waits for everything enqueued so far; time spent here is counted as wait_ns. */
+int apk_sync(apk_ctx* ctx);
+/* The raw hipStream_t the context launches on (for callers that record their own
+ * events or order other work against it). */
+void* apk_stream(apk_ctx* ctx);
+const char* apk_last_error(void);
+/* (calls, dispatches, encode_ns, wait_ns) since apk_init -- gpu::stats
+ * (gpu/common.rs:24-31). Any pointer may be NULL. */
+int apk_stats(apk_ctx* ctx, uint64_t* calls, uint64_t* dispatches, uint64_t* encode_ns, uint64_t* wait_ns);
+/* Reads and clears the device status word (synchronises the stream). */
+int apk_take_faults(apk_ctx* ctx, uint32_t* faults);
+
+/* Block geometry of a format: bytes of a row of n_in elements, or 0 when the type
+ * is unknown or n_in is not a whole number of blocks -- gpu::common::row_bytes
+ * (gpu/common.rs:63-68), GgmlType::expected_bytes (allpaka-dtype/src/lib.rs:112-124). */
+size_t apk_row_bytes(int fmt, size_t n_in);
+/* gpu::can_embed_on_gpu(ty, bytes, n_in) (gpu/stub.rs:85-87): 1 when
+ * apk_embed_rows takes this format and row length, else 0. */
+int apk_can_embed(int fmt, size_t n_in);
+
+/* -------------------------------------------------------------- memory ------ */
+
+int apk_malloc(apk_ctx* ctx, size_t bytes, void** dev_out);
+int apk_free(apk_ctx* ctx, void* dev);
+/* Stream-ordered copies; the host buffer must stay valid until apk_sync. */
+int apk_h2d(apk_ctx* ctx, void* dev_dst, const void* host_src, size_t bytes);
+int apk_d2h(apk_ctx* ctx, void* host_dst, const void* dev_src, size_t bytes);
+/* gpu::attach(mapping) / detach (gpu/stub.rs:37-41): copies a host weight mapping
+ * to device memory and keys it by host address, so weights are then named by
+ * their host address inside the mapping (gpu/cuda/runtime/select.rs:80-84). */
+int apk_attach(apk_ctx* ctx, const void* host_base, size_t len);
+int apk_detach(apk_ctx* ctx, const void* host_base);
+/* Device address of a host address inside an attached mapping. */
+int apk_resolve(apk_ctx* ctx, const void* host_ptr, size_t len, void** dev_out);
+
+/* Elapsed device time between two points of the stream (hipEvent based). */
+int apk_timer_begin(apk_ctx* ctx);
+int apk_timer_end(apk_ctx* ctx, float* ms_out);
+
+/* ----------------------------------------------------------------- ops ------ */
+
+/* Embedding gather with the dequant fused in: out[t,:] = dequant(row ids[t]).
+ * Replaces QuantMat::row_into over the token loop (quantmat/mod.rs:75-89; callers
+ * model/prefill.rs:92-106, model/decode.rs:422-431) and the reference's
+ * embed_row_f32_dtoken kernels (token id read on the device).
+ * table: [vocab][apk_row_bytes(fmt,n_in)] bytes, 16-byte aligned; ids: u32[t];
+ * out: [t][n_in] of out_dtype.  An id >= vocab leaves its row untouched and
+ * raises APK_FAULT_TOKEN_RANGE.  Formats taken: APK_FMT_Q8_0, APK_FMT_Q4K. */
+int apk_embed_rows(apk_ctx* ctx, int fmt, const void* table, size_t vocab, size_t n_in, const uint32_t* ids,
+                   size_t t, void* out, int out_dtype);
+/* Same with the ids on the host: range-checked BEFORE anything is enqueued
+ * (APK_DECLINE_RANGE), as the reference's callers reject token >= vocab first. */
+int apk_embed_rows_host_ids(apk_ctx* ctx, int fmt, const void* table, size_t vocab, size_t n_in,
+                            const uint32_t* ids_host, size_t t, void* out, int out_dtype);
+
+/* Residual add + RMSNorm over rows: x += delta (skipped when delta is NULL), then
+ * h = rmsnorm(x) * gamma.  Replaces ops::add_assign_slice followed by
+ * ops::rmsnorm_into / rmsnorm_rows_into (ops/blas.rs:105-178, ops/norm.rs:193-304;
+ * call sites model/decode.rs:584,764, model/prefill.rs:155,308-314).
+ * x, delta, h: [rows][n] of dtype (h may alias x when delta is NULL);
+ * gamma: f32[n].  n must be a multiple of 4 (f32) / 8 (f16). */
+int apk_add_rmsnorm_rows(apk_ctx* ctx, void* x, const void* delta, void* h, const float* gamma, size_t n,
+                         size_t rows, float eps, int dtype);
+
+/* Per-head QK-norm then NeoX RoPE, in place.  Replaces the loop
+ * ops::rmsnorm(head, w, eps); ops::rope_neox_cached_from_array(head, rope_row)
+ * over every q and k head of every row (model/attention.rs:131-165,
+ * ops/norm.rs:115-187, ops/rope.rs:70-81).
+ * q: [rows][n_q*head_dim], k: [rows][n_kv*head_dim] of dtype; qw, kw: f32[head_dim]
+ * or NULL (no norm for that tensor); rope: f32 [rows][head_dim/2][2] = [sin, cos]
+ * per row (the session table rows, model/session.rs:34-50).
+ * head_dim in {64,128,256}; rot_dim must equal head_dim (else declined). */
+int apk_qknorm_rope_neox(apk_ctx* ctx, void* q, void* k, const float* qw, const float* kw, const float* rope,
+                         size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim, float eps,
+                         int dtype);
+
+/* Builds RoPE table rows on the device: table[r][i] = [sin, cos](pos[r] as f32 *
+ * inv_freq[i]).  Replaces ops::rope_sin_cos per position (ops/rope.rs:18-22;
+ * Session::ensure_rope_cache, model/session.rs:34-50; gpu::multi_stage's staging
+ * of positions, gpu/stub.rs:181-183).  positions: u32[rows]; inv_freq: f32[half]. */
+int apk_rope_table(apk_ctx* ctx, const uint32_t* positions, const float* inv_freq, size_t rows, size_t half,
+                   float* table);
+
+/* SwiGLU in place: gate[i] = silu(gate[i]) * up[i].  Replaces ops::swiglu
+ * (ops/activation.rs:57-120, non-aarch64 arm). */
+int apk_swiglu(apk_ctx* ctx, void* gate, const void* up, size_t n, int dtype);
+
+/* MoE router: softmax (sigmoid != 0: sigmoid) over n_expert logits, top-k by
+ * descending selection score (+ bias when given), ties -> lower expert id,
+ * weights renormalised over the winners when norm != 0, then * scale.  Replaces
+ * model::route_gated / route_gated_into_slice per token (model/moe.rs:524-616,
+ * token loop :204-227).  logits: f32[rows][n_expert]; ids: u32[rows][k];
+ * w: f32[rows][k], both best-first.  n_expert <= 256, 1 <= k <= min(n_expert, 64). */
+int apk_route_topk(apk_ctx* ctx, const float* logits, const float* bias, size_t rows, size_t n_expert, size_t k,
+                   int norm, float scale, int sigmoid, uint32_t* ids, float* w);
+
+/* Token -> expert grouping in the CPU order.  Replaces the groups/used/table/tok
+ * construction and the CSR inversion of Ffn::moe_batch (model/moe.rs:229-271,
+ * :298-309; model/prefill.rs:624-675).  ids, w: [rows][k] from apk_route_topk.
+ * table: u32[n_expert][3] = (expert, row0, rows) for the NON-EMPTY experts in
+ * ascending order, *n_used of them (a device u32); tok: u32[rows*k] token of each
+ * flat row (expert-major, token-ascending inside an expert); tok_off: u32[rows+1];
+ * hit_row: u32[rows*k], hit_w: f32[rows*k] per-token hit lists in ascending
+ * expert order.  n_expert <= 1024, rows*k < 2^31. */
+int apk_moe_permute(apk_ctx* ctx, const uint32_t* ids, const float* w, size_t rows, size_t k, size_t n_expert,
+                    uint32_t* table, uint32_t* n_used, uint32_t* tok, uint32_t* tok_off, uint32_t* hit_row,
+                    float* hit_w);
+
+/* dst[r,:] = src[tok[r],:] -- the gathered expert activations (model/moe.rs:348-352).
+ * src: [src_rows][cols], dst: [total_rows][cols] of dtype; cols*sizeof(dtype) must
+ * be a multiple of 16. */
+int apk_gather_rows(apk_ctx* ctx, const void* src, const uint32_t* tok, size_t src_rows, size_t total_rows,
+                    size_t cols, void* dst, int dtype);
+
+/* dst = src, `bytes` a multiple of 16: the plain stream kernel the bandwidth
+ * figures of the other kernels are calibrated against. */
+int apk_copy(apk_ctx* ctx, const void* src, void* dst, size_t bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* APK_HIP_H */

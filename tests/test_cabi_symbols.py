@@ -1,0 +1,91 @@
+"""No-GPU checks of the boundary: the C-ABI library loads, exports every symbol
+include/apk_hip.h declares, embeds a gfx950 code object, and its pure host
+entries (block geometry, declines without a device) behave as the reference's
+(crates/allpaka-backend/src/gpu/common.rs:102-153, gpu/stub.rs)."""
+import ctypes as C
+import os
+import re
+import subprocess
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _lib():
+    import allpaka_amd.lib as lib
+
+    if not os.path.exists(lib.lib_path()):
+        subprocess.check_call(["make", "-s", "-C", os.path.join(ROOT, "allpaka_amd", "csrc")])
+    return lib, lib.load()
+
+
+def test_library_exports_every_declared_symbol():
+    lib, L = _lib()
+    header = open(os.path.join(ROOT, "include", "apk_hip.h")).read()
+    declared = set(re.findall(r"\b(apk_[a-z0-9_]+)\s*\(", header))
+    declared -= {"apk_ctx"}
+    assert declared, "no declarations parsed"
+    assert declared == set(lib.SYMBOLS), declared ^ set(lib.SYMBOLS)
+    for name in declared:
+        assert hasattr(L, name), name
+
+
+def test_code_object_is_gfx950_and_embedded():
+    lib, L = _lib()
+    co = os.path.join(ROOT, "allpaka_amd", "csrc", "apk_kernels.hsaco")
+    blob = open(lib.lib_path(), "rb").read()
+    assert b"\x7fELF" in blob
+    if os.path.exists(co):
+        code = open(co, "rb").read()
+        # hipcc --genco emits a clang offload bundle wrapping the gfx950 ELF; hipModuleLoadData takes both
+        assert code[:4] in (b"\x7fELF", b"__CL") and code in blob, "code object is not embedded verbatim"
+    assert b"gfx950" in blob
+    for k in [b"apk_swiglu_f16", b"apk_add_rmsnorm_f16_c1", b"apk_qknorm_rope_f16_hd128", b"apk_embed_q4k_f16",
+              b"apk_embed_q8_0_f32", b"apk_route_topk", b"apk_moe_permute", b"apk_gather_rows"]:
+        assert k in blob, k
+
+
+def test_row_bytes_and_format_codes_follow_the_reference():
+    lib, L = _lib()
+    # gpu/common.rs:106-115
+    assert L.apk_row_bytes(lib.FMT_Q4K, 512) == 2 * 144
+    assert L.apk_row_bytes(lib.FMT_Q6K, 256) == 210
+    assert L.apk_row_bytes(lib.FMT_Q8_0, 64) == 2 * 34
+    assert L.apk_row_bytes(lib.FMT_F16, 10) == 20
+    assert L.apk_row_bytes(lib.FMT_F32, 3) == 12
+    assert L.apk_row_bytes(lib.FMT_Q4K, 100) == 0
+    assert L.apk_row_bytes(77, 256) == 0
+    assert L.apk_row_bytes(lib.FMT_Q4K, 128) == 0
+    assert L.apk_row_bytes(lib.FMT_Q5_0, 128) == 88
+    # gpu/common.rs:118-134: the ten codes
+    assert [lib.FMT_Q4K, lib.FMT_Q5K, lib.FMT_Q6K, lib.FMT_Q8_0, lib.FMT_Q2K, lib.FMT_Q3K, lib.FMT_Q5_0, lib.FMT_F16,
+            lib.FMT_F32, lib.FMT_BF16] == list(range(10))
+    assert L.apk_can_embed(lib.FMT_Q8_0, 1024) == 1 and L.apk_can_embed(lib.FMT_Q4K, 5120) == 1
+    assert L.apk_can_embed(lib.FMT_Q4K, 100) == 0 and L.apk_can_embed(lib.FMT_Q6K, 256) == 0
+
+
+def test_no_device_declines_instead_of_failing():
+    lib, L = _lib()
+    h = C.c_void_p()
+    env_before = os.environ.get("ALLPAKA_NO_GPU")
+    os.environ["ALLPAKA_NO_GPU"] = "1"  # capability.rs:58-61: the host can force the CPU path
+    try:
+        rc = L.apk_init(0, C.byref(h))
+    finally:
+        if env_before is None:
+            del os.environ["ALLPAKA_NO_GPU"]
+        else:
+            os.environ["ALLPAKA_NO_GPU"] = env_before
+    assert rc == lib.DECLINE_NO_DEVICE and not h.value
+    assert b"ALLPAKA_NO_GPU" in L.apk_last_error()
+    # NULL context: a decline status, never a crash
+    assert L.apk_swiglu(None, None, None, 16, 0) == lib.DECLINE_NULL
+    assert L.apk_sync(None) == lib.DECLINE_NULL
+
+
+def test_package_has_no_cpu_fallback_and_never_touches_the_oracle():
+    pkg = os.path.join(ROOT, "allpaka_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".cpp", ".hip", ".h", ".S")):
+                src = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in src.lower().replace("no oracle", ""), f"{f} mentions the oracle"

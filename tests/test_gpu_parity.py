@@ -1,0 +1,460 @@
+"""GPU parity: every op through the C ABI (libapk_hip.so) against the CPU oracle on
+the same seeded inputs.
+
+Bars (stated per test):
+  * embedding dequant+gather, router ids, grouping tables, gathers: BIT-EXACT;
+  * f32 activations: max relative error <= 1e-5 (util.rel_err_f32) and the
+    reference's own idiom |a-b| < 1e-5(1+|b|);
+  * fp16 activations: <= 2 ulp of fp16.
+Full-size cases that the oracle cannot finish in seconds are covered through
+size-independent properties (row-subset equality, permutation invariants).
+"""
+import numpy as np
+import pytest
+
+from util import close_idiom, f16_ulp_diff, rel_err_f32
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+TOL_F32 = 1e-5
+TOL_F16_ULP = 2
+
+
+@pytest.fixture(scope="module")
+def be():
+    import allpaka_amd
+
+    b = allpaka_amd.Backend(0)
+    yield b
+    b.close()
+
+
+def dev(a):
+    """numpy -> device tensor; uint16 arrays are fp16 bit patterns, uint32 become int32."""
+    if a.dtype == np.uint16:
+        return torch.from_numpy(a.view(np.float16).copy()).cuda()
+    if a.dtype == np.uint32:
+        return torch.from_numpy(a.view(np.int32).copy()).cuda()
+    return torch.from_numpy(a.copy()).cuda()
+
+
+def host(t):
+    a = t.detach().cpu().numpy()
+    if a.dtype == np.float16:
+        return a.view(np.uint16)
+    if a.dtype == np.int32:
+        return a.view(np.uint32)
+    return a
+
+
+def synth():
+    from allpaka_amd import synth as s
+
+    return s
+
+
+# ------------------------------------------------------------------ embedding
+@pytest.mark.parametrize("fmt_name,n_in,vocab,t", [
+    ("Q8_0", 1024, 997, 1), ("Q8_0", 1024, 997, 512), ("Q8_0", 32, 5, 7), ("Q8_0", 96, 33, 40), ("Q8_0", 4096, 64, 9),
+    ("Q4K", 5120, 301, 1), ("Q4K", 5120, 301, 6), ("Q4K", 5120, 301, 300), ("Q4K", 256, 3, 5), ("Q4K", 1024, 17, 33),
+])
+@pytest.mark.parametrize("out_f16", [False, True])
+def test_embed_rows_bit_exact(be, ora, fmt_name, n_in, vocab, t, out_f16):
+    import allpaka_amd as apk
+
+    s = synth()
+    g = s.rng(0 if fmt_name == "Q8_0" else 2, n_in * 7 + vocab)
+    table = (s.q8_0_table if fmt_name == "Q8_0" else s.q4_k_table)(g, vocab, n_in)
+    ids = g.integers(0, vocab, size=t, dtype=np.uint32)
+    ids[0] = vocab - 1  # last row: exercises the end-of-table tile
+    if t > 1:
+        ids[-1] = 0
+    fmt = ora.FMT[fmt_name]
+    want = ora.embed_rows(table, fmt, vocab, n_in, ids, out_f16=out_f16)
+    qm = apk.QuantMat(be, dev(table), fmt, vocab, n_in)
+    out = torch.full((t, n_in), 7.0, dtype=torch.float16 if out_f16 else torch.float32, device="cuda")
+    qm.rows_into(dev(ids), out)
+    got = host(out)
+    assert np.array_equal(got.view(np.uint16 if out_f16 else np.uint32), want.view(np.uint16 if out_f16 else np.uint32))
+    # QuantMat::row / row_into, one row, ids on the host
+    r = qm.row(int(ids[0]), dtype=torch.float16 if out_f16 else torch.float32)
+    assert np.array_equal(host(r), want[0])
+
+
+def test_embed_subnormal_scales_and_reference_vectors(be, ora):
+    import allpaka_amd as apk
+
+    # the reference's Q8_0 known answer (dequant.rs:317-331) and a block of f16-subnormal scales
+    block = np.zeros((4, 34), np.uint8)
+    block[0, 0:2] = np.frombuffer(np.float16(0.5).tobytes(), np.uint8)
+    block[0, 2], block[0, 3], block[0, 33] = 10, np.uint8(236), 127
+    for r, code in enumerate([0x0001, 0x03FF, 0x8001], start=1):
+        block[r, 0:2] = np.frombuffer(np.uint16(code).tobytes(), np.uint8)
+        block[r, 2:] = np.arange(-16, 16, dtype=np.int8).view(np.uint8) * 7
+    qm = apk.QuantMat(be, dev(block.reshape(-1)), ora.FMT["Q8_0"], 4, 32)
+    out = torch.zeros((4, 32), dtype=torch.float32, device="cuda")
+    qm.rows_into(dev(np.arange(4, dtype=np.uint32)), out)
+    got = host(out)
+    assert got[0, 0] == 5.0 and got[0, 1] == -10.0 and got[0, 31] == 63.5 and got[0, 2] == 0.0
+    want = ora.embed_rows(block.reshape(-1), ora.FMT["Q8_0"], 4, 32, np.arange(4, dtype=np.uint32))
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert got[1, 0] == np.float32(-112 * 2.0 ** -24)
+    # Q4_K known answer (dequant.rs:448-468)
+    blk = np.zeros(144, np.uint8)
+    blk[0:2] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    blk[2:4] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    blk[4], blk[5], blk[8], blk[9], blk[16] = 2, 3, 1, 2, 0x75
+    qm = apk.QuantMat(be, dev(blk), ora.FMT["Q4K"], 1, 256)
+    got = host(qm.row(0))
+    assert got[0] == 9.0 and got[1] == -1.0 and got[32] == 19.0 and got[33] == -2.0 and np.all(got[64:] == 0.0)
+
+
+def test_embed_errors_and_declines(be, ora):
+    import allpaka_amd as apk
+
+    data = dev(np.zeros(34 * 2, np.uint8))
+    qm = apk.QuantMat(be, data, ora.FMT["Q8_0"], 1, 64)
+    with pytest.raises(ValueError):  # quantmat/mod.rs:923-937: row(1) of a 1-row matrix
+        qm.row(1)
+    with pytest.raises(ValueError):
+        apk.QuantMat(be, data, ora.FMT["Q8_0"], 1, 48)
+    with pytest.raises(ValueError):
+        apk.QuantMat(be, data[:-1], ora.FMT["Q8_0"], 1, 64)
+    with pytest.raises(ValueError):
+        qm.row_into(0, torch.zeros(32, device="cuda"))
+    # device-side ids out of vocab: no fault, the row is left untouched, the status word says so
+    out = torch.full((2, 64), 3.0, device="cuda")
+    with pytest.raises(ValueError):
+        qm.rows_into(dev(np.array([0, 5], np.uint32)), out)
+    assert np.all(host(out)[1] == 3.0) and np.all(host(out)[0] == 0.0)
+    assert be.take_faults() == 0  # cleared by the read above
+    # a format outside the device path declines, it does not fail
+    q6 = apk.QuantMat(be, dev(np.zeros(210, np.uint8)), ora.FMT["Q6K"], 1, 256)
+    with pytest.raises(apk.Declined):
+        q6.row(0)
+
+
+# ------------------------------------------------------------- add + RMSNorm
+@pytest.mark.parametrize("n,rows", [(1024, 1), (1024, 512), (5120, 1), (5120, 6), (5120, 64), (2048, 33), (128, 5),
+                                    (8, 3), (4096 + 64, 3), (8192, 2), (16384, 2)])
+@pytest.mark.parametrize("f16", [False, True])
+@pytest.mark.parametrize("with_delta", [True, False])
+def test_add_rmsnorm_rows(be, ora, n, rows, f16, with_delta):
+    s = synth()
+    g = s.rng(1, n + rows)
+    x = s.normal_f32(g, (rows, n))
+    d = s.normal_f32(g, (rows, n))
+    gamma = s.normal_f32(g, n, 1.0, 0.05)
+    if f16:
+        x, d = s.to_f16_bits(x), s.to_f16_bits(d)
+    wx, wh = x.copy(), np.zeros_like(x)
+    ora.add_rmsnorm_rows(wx, d if with_delta else None, wh, gamma, 1e-6)
+    tx, th = dev(x), torch.zeros_like(dev(x))
+    be.add_rmsnorm_rows(tx, dev(d) if with_delta else None, th, dev(gamma), 1e-6)
+    gx, gh = host(tx), host(th)
+    if f16:
+        assert np.array_equal(gx, wx)  # the residual sum rounds once: bit-exact
+        assert f16_ulp_diff(gh, wh) <= TOL_F16_ULP
+    else:
+        assert np.array_equal(gx, wx)  # f32 add is exact-same
+        assert rel_err_f32(gh, wh) <= TOL_F32 and close_idiom(gh, wh)
+        assert np.mean(gh.view(np.uint32) == wh.view(np.uint32)) > 0.999  # f64 statistics: bit-equal almost everywhere
+
+
+def test_rmsnorm_reference_vectors_and_asserts(be, ora):
+    # ops/mod.rs:119-144, :412-419
+    x = torch.tensor([3.0, -4.0, 12.0, 0.0], device="cuda")
+    be.rmsnorm(x, torch.ones(4, device="cuda"), 0.0)
+    h = host(x)
+    assert abs(float(np.sqrt((h * h).sum() / 4)) - 1.0) < 1e-5 and h[0] > 0 and h[1] < 0 and h[3] == 0
+    x = torch.zeros(8, device="cuda")
+    be.rmsnorm(x, torch.ones(8, device="cuda"), 1e-5)
+    assert np.all(np.isfinite(host(x)))
+    with pytest.raises(AssertionError, match="dst holds fewer rows than src"):
+        be.rmsnorm_rows_into(torch.zeros(8 * 1024, device="cuda"), torch.ones(64 * 1024, device="cuda"),
+                             torch.ones(1024, device="cuda"), 1e-6)
+    with pytest.raises(AssertionError):
+        be.rmsnorm(torch.zeros(4, device="cuda"), torch.zeros(8, device="cuda"), 0.0)
+    import allpaka_amd as apk
+
+    with pytest.raises(apk.Declined):  # n = 6 is not a whole 16-byte tile: declined, not faulted
+        be.rmsnorm(torch.zeros(6, device="cuda"), torch.zeros(6, device="cuda"), 0.0)
+    src = torch.randn(40, 1024, device="cuda")
+    w = torch.randn(1024, device="cuda")
+    dst = torch.zeros_like(src)
+    be.rmsnorm_rows_into(dst, src, w, 1e-6)
+    want = np.zeros((40, 1024), np.float32)
+    ora.rmsnorm_rows_into(want, host(src), host(w), 1e-6, threads=4)
+    assert rel_err_f32(host(dst), want) <= TOL_F32
+
+
+# ------------------------------------------------------- QK-norm + NeoX RoPE
+def _qk_case(ora, cfg, rows, n_q, n_kv, hd, f16, positions, theta=1e6):
+    s = synth()
+    g = s.rng(cfg, rows * 131 + n_q)
+    q = s.normal_f32(g, (rows, n_q * hd))
+    k = s.normal_f32(g, (rows, n_kv * hd))
+    qw = s.normal_f32(g, hd, 1.0, 0.05)
+    kw = s.normal_f32(g, hd, 1.0, 0.05)
+    if f16:
+        q, k = s.to_f16_bits(q), s.to_f16_bits(k)
+    inv = ora.rope_inv_freq(hd, theta)
+    ropes = ora.rope_table(positions, inv)
+    return q, k, qw, kw, inv, ropes
+
+
+@pytest.mark.parametrize("rows,n_q,n_kv,hd,pos_kind", [
+    (1, 16, 8, 128, "one"), (512, 16, 8, 128, "prefill"), (1, 64, 8, 128, "one"), (6, 64, 8, 128, "verify"),
+    (64, 64, 8, 128, "multi"), (5, 3, 1, 64, "multi"), (3, 2, 2, 256, "multi"), (7, 1, 0, 128, "multi"),
+])
+@pytest.mark.parametrize("f16", [False, True])
+def test_qknorm_rope(be, ora, rows, n_q, n_kv, hd, pos_kind, f16):
+    g = synth().rng(3, rows)
+    positions = {"one": [int(g.integers(0, 4096))], "prefill": list(range(rows)), "verify": list(range(1000, 1000 + rows)),
+                 "multi": [int(p) for p in g.integers(0, 32768, size=rows)]}[pos_kind]
+    q, k, qw, kw, inv, ropes = _qk_case(ora, 3, rows, n_q, n_kv, hd, f16, positions)
+    wq, wk = q.copy(), k.copy()
+    ora.qknorm_rope_rows(wq, wk, n_q, n_kv, hd, qw, kw, ropes, 1e-6)
+    tq, tk = dev(q), dev(k)
+    be.qknorm_rope_neox(tq, tk, dev(qw), dev(kw), dev(ropes), n_q, n_kv, hd, 1e-6)
+    for got, want in ((host(tq), wq), (host(tk), wk)):
+        if f16:
+            assert f16_ulp_diff(got, want) <= TOL_F16_ULP
+        else:
+            assert rel_err_f32(got, want) <= TOL_F32 and close_idiom(got, want)
+
+
+def test_rope_only_and_reference_vectors(be, ora):
+    # no norm weights: rotation only (attention.rs:140-146); bit-exact (same f32 ops, no contraction)
+    rows, n_q, n_kv, hd = 9, 4, 2, 128
+    positions = [0, 1, 17, 5000, 4097, 32767, 3, 511, 12345]
+    q, k, _, _, inv, ropes = _qk_case(ora, 3, rows, n_q, n_kv, hd, False, positions)
+    wq, wk = q.copy(), k.copy()
+    ora.qknorm_rope_rows(wq, wk, n_q, n_kv, hd, None, None, ropes, 1e-6)
+    tq, tk = dev(q), dev(k)
+    be.qknorm_rope_neox(tq, tk, None, None, dev(ropes), n_q, n_kv, hd, 1e-6)
+    assert np.array_equal(host(tq), wq) and np.array_equal(host(tk), wk)
+    assert np.array_equal(host(tq)[0], q[0])  # position 0 is the identity (ops/mod.rs:188-202)
+    # pairing: a one-hot channel 0 moves energy to channel hd/2 (ops/mod.rs:206-221)
+    x = torch.zeros(128, device="cuda")
+    x[0] = 1.0
+    t1 = ora.rope_sin_cos(1, ora.rope_inv_freq(128, 10000.0))
+    be.rope_neox_cached_from_array(x, dev(t1))
+    h = host(x)
+    assert abs(h[64] - np.sin(np.float32(1.0))) < 1e-6 and h[1] == 0.0
+    import allpaka_amd as apk
+
+    with pytest.raises(apk.Declined):  # partial rotary is declined, not mis-rotated
+        be.qknorm_rope_neox(tq, tk, None, None, dev(ropes[:, :32].copy()), n_q, n_kv, hd, 1e-6, rot_dim=64)
+
+
+def test_rope_table_on_device(be, ora):
+    # table rows built on the device vs ops::rope_sin_cos: same f32 angle, device sincosf vs glibc
+    inv = ora.rope_inv_freq(128, 1e6)
+    g = synth().rng(3, 99)
+    positions = np.concatenate([np.arange(0, 512), g.integers(0, 32768, size=64)]).astype(np.uint32)
+    want = ora.rope_table(positions, inv)
+    got = host(be.rope_table(dev(positions), dev(inv)))
+    assert np.max(np.abs(got - want)) <= 2.5e-7  # sin/cos are in [-1,1]: 2 ulp at 1.0
+    # and used end to end on the 64 long-context rows (fp16 config)
+    rows, n_q, n_kv, hd = 64, 64, 8, 128
+    q, k, qw, kw, _, ropes = _qk_case(ora, 3, rows, n_q, n_kv, hd, True, positions[512:])
+    wq, wk = q.copy(), k.copy()
+    ora.qknorm_rope_rows(wq, wk, n_q, n_kv, hd, qw, kw, ropes, 1e-6)
+    tq, tk = dev(q), dev(k)
+    be.qknorm_rope_neox(tq, tk, dev(qw), dev(kw), be.rope_table(dev(positions[512:].copy()), dev(inv)), n_q, n_kv, hd, 1e-6)
+    assert f16_ulp_diff(host(tq), wq) <= TOL_F16_ULP and f16_ulp_diff(host(tk), wk) <= TOL_F16_ULP
+
+
+# --------------------------------------------------------------------- SwiGLU
+@pytest.mark.parametrize("n", [3072, 512 * 3072, 6 * 25600, 64 * 25600, 1, 5, 1031, 8192 * 768 // 16])
+@pytest.mark.parametrize("f16", [False, True])
+def test_swiglu(be, ora, n, f16):
+    s = synth()
+    g = s.rng(4, n)
+    gate, up = s.normal_f32(g, n), s.normal_f32(g, n)
+    gate[: min(n, 8)] = np.float32([0.0, 1.0, -20.0, 20.0, -88.0, 88.0, -0.0, 1e-30])[: min(n, 8)]
+    if f16:
+        gate, up = s.to_f16_bits(gate), s.to_f16_bits(up)
+    want = gate.copy()
+    ora.swiglu(want, up)
+    tg = dev(gate)
+    be.swiglu(tg, dev(up))
+    got = host(tg)
+    if f16:
+        assert f16_ulp_diff(got, want) <= TOL_F16_ULP
+    else:
+        assert rel_err_f32(got, want) <= TOL_F32 and close_idiom(got, want)
+
+
+def test_swiglu_reference_sweep_and_assert(be, ora):
+    # ops/mod.rs:172-185
+    gate = np.float32([i * 0.7 for i in range(-25, 26)])
+    up = np.float32([i * 0.5 - 3.0 for i in range(51)])
+    tg = dev(gate)
+    be.swiglu(tg, dev(up))
+    for got, gg, u in zip(host(tg), gate, up):
+        want = ora.silu(gg) * u
+        assert abs(got - want) < 1e-5 * (1 + abs(want))
+    with pytest.raises(AssertionError):
+        be.swiglu(torch.zeros(4, device="cuda"), torch.zeros(3, device="cuda"))
+
+
+# --------------------------------------------------------------------- router
+def _ref_logits(n):
+    return np.float32([((i * 37 % 331) - 165.0) * 0.03 for i in range(n)])
+
+
+@pytest.mark.parametrize("rows,n_expert,k", [(1024, 128, 8), (1, 128, 8), (7, 64, 4), (33, 256, 8), (5, 60, 6), (3, 4, 4), (9, 200, 1)])
+@pytest.mark.parametrize("norm,scale", [(True, 1.0), (False, 1.5)])
+def test_route_topk(be, ora, rows, n_expert, k, norm, scale):
+    s = synth()
+    logits = s.normal_f32(s.rng(4, rows * n_expert + k), (rows, n_expert))
+    want_ids, want_w = ora.route_rows(logits, k, ora.SOFTMAX, norm, scale, threads=4)
+    # the two selection orders (on probabilities as the CPU does, on raw logits as the device does) agree here
+    for r in range(rows):
+        assert np.array_equal(want_ids[r], ora.topk_by_logits(logits[r], k))
+    ids, w = be.route_rows(dev(logits), k, norm=norm, scale=scale)
+    assert np.array_equal(host(ids), want_ids)  # bit-exact indices
+    assert rel_err_f32(host(w), want_w) <= TOL_F32
+
+
+def test_route_reference_vectors_ties_sigmoid_bias(be, ora):
+    import allpaka_amd as apk
+
+    base = _ref_logits(256)  # moe.rs:664-715
+    for gating, norm in [(apk.Gating.Softmax, True), (apk.Gating.Softmax, False), (apk.Gating.Sigmoid, True)]:
+        for k in (1, 8):
+            wi, ww = ora.route_gated(base, k, int(gating), norm, 1.5)
+            got = be.route_gated(dev(base), k, gating, norm, 1.5)
+            assert [e for e, _ in got] == list(wi)
+            assert np.allclose([x for _, x in got], ww, rtol=1e-5, atol=0)
+    bias = np.float32([0.5 + (i % 7) * 0.01 for i in range(256)])
+    wi, ww = ora.route_gated(base, 8, ora.SIGMOID, True, 2.5, bias)
+    got = be.route_gated(dev(base), 8, apk.Gating.Sigmoid, True, 2.5, dev(bias))
+    assert [e for e, _ in got] == list(wi) and np.allclose([x for _, x in got], ww, rtol=1e-5, atol=0)
+    # softmax with a selection bias: selection on score + bias, weights from the scores
+    lg = synth().normal_f32(synth().rng(4, 5), 128)
+    b2 = synth().normal_f32(synth().rng(4, 6), 128, 0.0, 0.01)
+    wi, ww = ora.route_gated(lg, 8, ora.SOFTMAX, True, 1.0, b2)
+    got = be.route_gated(dev(lg), 8, apk.Gating.Softmax, True, 1.0, dev(b2))
+    assert [e for e, _ in got] == list(wi) and np.allclose([x for _, x in got], ww, rtol=1e-5, atol=0)
+    # exact ties: the lower index wins, inside the top-k and at its boundary
+    t = np.zeros(128, np.float32)
+    t[[3, 9, 12, 100]] = 2.0
+    t[[5, 7, 77]] = 1.0
+    got = be.route_gated(dev(t), 6)
+    assert [e for e, _ in got] == [3, 9, 12, 100, 5, 7] == list(ora.route_gated(t, 6)[0])
+    got = be.route_gated(dev(np.zeros(8, np.float32)), 2)
+    assert [e for e, _ in got] == [0, 1] and np.allclose([x for _, x in got], 0.5)
+    # route(probs, k) of the reference's test (gpu_eligible_forward.rs:88-97) through log-probabilities
+    got = be.route_gated(dev(np.log(np.float32([0.1, 0.5, 0.15, 0.25]))), 2)
+    assert [e for e, _ in got] == [1, 3] and abs(got[0][1] - 2 / 3) < 1e-6 and abs(got[1][1] - 1 / 3) < 1e-6
+    # k clamps to n; more than 256 experts is declined
+    assert len(be.route_gated(dev(t[:4].copy()), 8)) == 4
+    with pytest.raises(apk.Declined):
+        be.route_gated(dev(_ref_logits(320)), 4)
+
+
+# ------------------------------------------------------- grouping and gather
+@pytest.mark.parametrize("rows,k,n_expert", [(1024, 8, 128), (1, 8, 128), (5, 2, 4), (600, 8, 16), (64, 1, 256), (777, 3, 7), (2048, 8, 128)])
+def test_moe_permute_and_gather_bit_exact(be, ora, rows, k, n_expert):
+    s = synth()
+    g = s.rng(4, rows + k)
+    logits = s.normal_f32(g, (rows, n_expert))
+    if rows > 4:
+        logits[:, n_expert // 2] = -50.0  # an expert nobody picks: the table must skip it
+    ids, w = ora.route_rows(logits, k, threads=4)
+    want = ora.moe_group(ids, w, n_expert)
+    got = be.moe_permute(dev(ids), dev(w), n_expert)
+    names = ["table", "tok", "tok_off", "hit_row", "hit_w"]
+    for name, a, b in zip(names, got, want):
+        a = host(a)
+        assert a.shape == b.shape, name
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), name
+    for f16 in (False, True):
+        cols = 2048 if rows <= 1024 else 256
+        hs = s.normal_f32(g, (rows, cols))
+        if f16:
+            hs = s.to_f16_bits(hs)
+        xe = be.gather_rows(dev(hs), got[1])
+        assert np.array_equal(host(xe), ora.gather_rows(hs, want[1]))
+
+
+def test_permute_declines_and_faults(be):
+    import allpaka_amd as apk
+
+    ids = torch.tensor([[0, 9]], dtype=torch.int32, device="cuda")  # expert 9 of 4
+    w = torch.ones((1, 2), device="cuda")
+    be.moe_permute(ids, w, 4)
+    assert be.take_faults() & 2
+    with pytest.raises(apk.Declined):
+        be.moe_permute(ids, w, 2000)
+    src = torch.ones((2, 64), device="cuda")
+    out = be.gather_rows(src, torch.tensor([1, 7], dtype=torch.int32, device="cuda"))
+    assert be.take_faults() & 4 and np.all(host(out)[0] == 1.0)
+    with pytest.raises(apk.Declined):
+        be.gather_rows(torch.ones((2, 3), device="cuda"), torch.tensor([0], dtype=torch.int32, device="cuda"))
+
+
+# ----------------------------------------------- full-size property checks
+def test_full_size_prefill_properties(be, ora):
+    """Qwen3-32B shapes at T=2048 (fp16): the oracle checks a row subset; the rest is
+    covered by row independence (every row of a batched launch equals the same row
+    launched alone, the batch==sequential property of gpu_eligible_forward.rs:33-66)."""
+    s = synth()
+    m = s.MODELS["qwen3-32b"]
+    T, H, F = 2048, m["hidden"], m["ffn"]
+    gen = torch.Generator(device="cuda").manual_seed(1234)
+    x = torch.randn((T, H), generator=gen, device="cuda").half()
+    d = torch.randn((T, H), generator=gen, device="cuda").half()
+    gamma = (1 + 0.05 * torch.randn(H, generator=gen, device="cuda")).float()
+    x0 = x.clone()
+    h = torch.zeros_like(x)
+    be.add_rmsnorm_rows(x, d, h, gamma, 1e-6)
+    pick = [0, 1, 777, 2047]
+    xs, ds = host(x0[pick]).copy(), host(d[pick]).copy()
+    wh = np.zeros_like(xs)
+    ora.add_rmsnorm_rows(xs, ds, wh, host(gamma), 1e-6)
+    assert np.array_equal(host(x[pick]), xs) and f16_ulp_diff(host(h[pick]), wh) <= TOL_F16_ULP
+    x1, h1 = x0[1000:1001].clone(), torch.zeros((1, H), dtype=torch.float16, device="cuda")
+    be.add_rmsnorm_rows(x1, d[1000:1001].clone(), h1, gamma, 1e-6)
+    assert torch.equal(h1[0], h[1000]) and torch.equal(x1[0], x[1000])
+    # SwiGLU over [2048, 25600]: a slice against the oracle, the whole against a row-sliced relaunch
+    gate = torch.randn((T, F), generator=gen, device="cuda").half()
+    up = torch.randn((T, F), generator=gen, device="cuda").half()
+    g0 = gate.clone()
+    be.swiglu(gate, up)
+    wg = host(g0[5]).copy()
+    ora.swiglu(wg, host(up[5]).copy())
+    assert f16_ulp_diff(host(gate[5]), wg) <= TOL_F16_ULP
+    part = g0[1024:1030].clone()
+    be.swiglu(part, up[1024:1030].clone())
+    assert torch.equal(part, gate[1024:1030])
+    # embedding gather of 2048 rows from a Q4_K table: every output row equals the single-row gather of its id
+    import allpaka_amd as apk
+
+    vocab = 4096
+    table = s.q4_k_table(s.rng(2, 1), vocab, H)
+    qm = apk.QuantMat(be, dev(table.reshape(-1)), ora.FMT["Q4K"], vocab, H)
+    ids = s.rng(2, 2).integers(0, vocab, size=T, dtype=np.uint32)
+    out = torch.zeros((T, H), dtype=torch.float16, device="cuda")
+    qm.rows_into(dev(ids), out)
+    sub = [0, 5, 2047]
+    want = ora.embed_rows(table.reshape(-1), ora.FMT["Q4K"], vocab, H, ids[sub], out_f16=True)
+    assert np.array_equal(host(out[sub]), want)
+    # rows with equal ids are equal (gather idempotence)
+    order = np.argsort(ids, kind="stable")
+    same = [(order[i], order[i + 1]) for i in range(T - 1) if ids[order[i]] == ids[order[i + 1]]][:50]
+    for a, b in same:
+        assert torch.equal(out[a], out[b])
+
+
+def test_stats_count_calls_and_dispatches(be):
+    c0, d0, _, _ = be.stats()
+    a = torch.ones(4096, device="cuda")
+    be.swiglu(a, torch.ones(4096, device="cuda"))
+    c1, d1, enc, wait = be.stats()
+    assert c1 == c0 + 1 and d1 == d0 + 1 and enc > 0 and wait > 0
