@@ -16,6 +16,8 @@
 #include <cstring>
 #include <map>
 #include <mutex>
+#include <string>
+#include <unordered_map>
 #include <vector>
 
 extern "C" const unsigned char apk_kernels_co[];
@@ -52,27 +54,25 @@ struct Mapping {
     size_t len;
 };
 
-enum Kernel {
-    K_SWIGLU_F32, K_SWIGLU_F16,
-    K_ADDNORM_F32_C1, K_ADDNORM_F32_C2, K_ADDNORM_F32_C4, K_ADDNORM_F32_C8,
-    K_ADDNORM_F16_C1, K_ADDNORM_F16_C2, K_ADDNORM_F16_C4, K_ADDNORM_F16_C8,
-    K_QKROPE_F32_64, K_QKROPE_F32_128, K_QKROPE_F32_256,
-    K_QKROPE_F16_64, K_QKROPE_F16_128, K_QKROPE_F16_256,
-    K_ROPE_TABLE,
-    K_EMBED_Q4K_F32, K_EMBED_Q4K_F16, K_EMBED_Q8_0_F32, K_EMBED_Q8_0_F16,
-    K_ROUTE_TOPK, K_MOE_PERMUTE, K_GATHER_ROWS, K_COPY,
-    K_COUNT
-};
-const char* const kKernelNames[K_COUNT] = {
-    "apk_swiglu_f32", "apk_swiglu_f16",
-    "apk_add_rmsnorm_f32_c1", "apk_add_rmsnorm_f32_c2", "apk_add_rmsnorm_f32_c4", "apk_add_rmsnorm_f32_c8",
-    "apk_add_rmsnorm_f16_c1", "apk_add_rmsnorm_f16_c2", "apk_add_rmsnorm_f16_c4", "apk_add_rmsnorm_f16_c8",
-    "apk_qknorm_rope_f32_hd64", "apk_qknorm_rope_f32_hd128", "apk_qknorm_rope_f32_hd256",
-    "apk_qknorm_rope_f16_hd64", "apk_qknorm_rope_f16_hd128", "apk_qknorm_rope_f16_hd256",
-    "apk_rope_table",
-    "apk_embed_q4k_f32", "apk_embed_q4k_f16", "apk_embed_q8_0_f32", "apk_embed_q8_0_f16",
-    "apk_route_topk", "apk_moe_permute", "apk_gather_rows", "apk_copy",
-};
+// Every kernel of the embedded code object, resolved once at apk_init so that a
+// missing symbol fails there and not at the first launch.
+const int kAddnormTiles[] = {1, 2, 3, 4, 5, 6, 8, 10, 12, 16, 20};  // 16-byte tiles per lane
+const int kAddnormBound[] = {1024, 1024, 512, 512, 256, 256, 256, 256, 256, 256, 256};  // launch bound of each
+const int kQkIters[] = {1, 3, 9};
+const int kQkHeadDims[] = {64, 128, 256};
+
+std::vector<std::string> all_kernel_names() {
+    std::vector<std::string> v = {"apk_swiglu_f32", "apk_swiglu_f16", "apk_rope_table", "apk_embed_q4k_f32",
+                                  "apk_embed_q4k_f16", "apk_embed_q8_0_f32", "apk_embed_q8_0_f16", "apk_route_topk",
+                                  "apk_moe_permute", "apk_gather_rows", "apk_copy"};
+    for (const char* t : {"f32", "f16"}) {
+        for (int c : kAddnormTiles) v.push_back(std::string("apk_add_rmsnorm_") + t + "_c" + std::to_string(c));
+        for (int hd : kQkHeadDims)
+            for (int it : kQkIters)
+                v.push_back(std::string("apk_qknorm_rope_") + t + "_hd" + std::to_string(hd) + "_i" + std::to_string(it));
+    }
+    return v;
+}
 
 }  // namespace
 
@@ -80,7 +80,7 @@ struct apk_ctx {
     int device = 0;
     hipModule_t module = nullptr;
     hipStream_t stream = nullptr;
-    hipFunction_t fn[K_COUNT] = {};
+    std::unordered_map<std::string, hipFunction_t> fn;
     uint32_t* fault_dev = nullptr;  // device status word
     uint32_t* ids_stage_host = nullptr;  // pinned staging for host-side token ids
     uint32_t* ids_stage_dev = nullptr;
@@ -101,10 +101,12 @@ struct CallScope {  // counts one ABI call and its host-side encode time
     ~CallScope() { c->encode_ns += now_ns() - t0; }
 };
 
-int launch(apk_ctx* c, Kernel k, unsigned grid, unsigned block, unsigned shmem, void** args) {
+int launch(apk_ctx* c, const std::string& k, unsigned grid, unsigned block, unsigned shmem, void** args) {
     if (grid == 0) return APK_OK;
-    hipError_t e = hipModuleLaunchKernel(c->fn[k], grid, 1, 1, block, 1, 1, shmem, c->stream, args, nullptr);
-    if (e != hipSuccess) return hip_fail(e, kKernelNames[k]);
+    auto it = c->fn.find(k);
+    if (it == c->fn.end()) return fail(APK_DECLINE_UNSUPPORTED, "no kernel %s in the code object", k.c_str());
+    hipError_t e = hipModuleLaunchKernel(it->second, grid, 1, 1, block, 1, 1, shmem, c->stream, args, nullptr);
+    if (e != hipSuccess) return hip_fail(e, k.c_str());
     c->dispatches++;
     return APK_OK;
 }
@@ -161,7 +163,11 @@ int apk_init(int device, apk_ctx** out) {
     int rc = [&]() -> int {
         HIP_TRY(hipSetDevice(device));
         HIP_TRY(hipModuleLoadData(&c->module, apk_kernels_co));
-        for (int k = 0; k < K_COUNT; k++) HIP_TRY(hipModuleGetFunction(&c->fn[k], c->module, kKernelNames[k]));
+        for (const std::string& name : all_kernel_names()) {
+            hipFunction_t f = nullptr;
+            HIP_TRY(hipModuleGetFunction(&f, c->module, name.c_str()));
+            c->fn[name] = f;
+        }
         HIP_TRY(hipStreamCreate(&c->stream));
         HIP_TRY(hipMalloc((void**)&c->fault_dev, 256));
         HIP_TRY(hipMemsetAsync(c->fault_dev, 0, 256, c->stream));
@@ -333,13 +339,13 @@ int apk_swiglu(apk_ctx* c, void* gate, const void* up, size_t n, int dtype) {
     if (!aligned16(gate) || !aligned16(up)) return fail(APK_DECLINE_SHAPE, "apk_swiglu: tensors must be 16-byte aligned");
     if (int rc = set_device(c)) return rc;
     const uint64_t vec = 16 / es, nvec = n / vec;
-    const unsigned block = 256, per_block = block * 4;
+    const unsigned block = 256, per_block = block;  // one 16-byte tile per lane
     uint64_t grid = (nvec + per_block - 1) / per_block;
     if (grid == 0) grid = 1;
     if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_swiglu: n too large");
     uint64_t n64 = n;
     void* args[] = {&gate, &up, &n64};
-    return launch(c, dtype == APK_F32 ? K_SWIGLU_F32 : K_SWIGLU_F16, (unsigned)grid, block, 0, args);
+    return launch(c, dtype == APK_F32 ? "apk_swiglu_f32" : "apk_swiglu_f16", (unsigned)grid, block, 0, args);
 }
 
 int apk_add_rmsnorm_rows(apk_ctx* c, void* x, const void* delta, void* h, const float* gamma, size_t n, size_t rows,
@@ -356,19 +362,29 @@ int apk_add_rmsnorm_rows(apk_ctx* c, void* x, const void* delta, void* h, const 
         return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: tensors must be 16-byte aligned");
     if (rows > 0x7fffffffu || n > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: too large");
     const size_t nchunks = n / vec;
-    // fewest tiles per lane that keep the workgroup within 640 lanes (10 waves):
-    // the row stays in registers and several workgroups share a CU.
-    int nch = 1;
-    while (nch < 8 && (nchunks + nch - 1) / nch > 640) nch *= 2;
-    size_t threads = (nchunks + nch - 1) / nch;
-    if (threads > 1024) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: row of %zu elements is too long", n);
-    threads = (threads + 63) / 64 * 64;
-    const int base = dtype == APK_F32 ? K_ADDNORM_F32_C1 : K_ADDNORM_F16_C1;
-    const int which = base + (nch == 1 ? 0 : nch == 2 ? 1 : nch == 4 ? 2 : 3);
+    // Tiles per lane (NCH) and waves per row (W = ceil(nchunks / (64*NCH))): the first
+    // choice that keeps the whole batch resident in one round (rows * W <= 2048 waves,
+    // 8 per CU) -- a wave per row for prefill batches, many waves per row for a few
+    // decode rows -- else the fewest waves per row the register budget allows.
+    const int max_nch = dtype == APK_F16 ? 10 : 20;
+    int nch = 0;
+    size_t waves = 0;
+    for (size_t i = 0; i < sizeof kAddnormTiles / sizeof kAddnormTiles[0]; i++) {
+        const int cand = kAddnormTiles[i];
+        if (cand > max_nch) break;
+        const size_t w = (nchunks + 64 * (size_t)cand - 1) / (64 * (size_t)cand);
+        if (w * 64 > (size_t)kAddnormBound[i]) continue;
+        nch = cand;
+        waves = w;
+        if (rows * w <= 2048) break;
+    }
+    if (!nch) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: row of %zu elements is too long", n);
+    const size_t threads = waves * 64;
+    const std::string which = std::string("apk_add_rmsnorm_") + (dtype == APK_F32 ? "f32" : "f16") + "_c" + std::to_string(nch);
     if (int rc = set_device(c)) return rc;
     int n_i = (int)n;
     void* args[] = {&x, &delta, &h, &gamma, &n_i, &eps};
-    return launch(c, (Kernel)which, (unsigned)rows, (unsigned)threads, 0, args);
+    return launch(c, which, (unsigned)rows, (unsigned)threads, 0, args);
 }
 
 int apk_qknorm_rope_neox(apk_ctx* c, void* q, void* k, const float* qw, const float* kw, const float* rope,
@@ -386,16 +402,26 @@ int apk_qknorm_rope_neox(apk_ctx* c, void* q, void* k, const float* qw, const fl
     if ((q && !aligned16(q)) || (k && !aligned16(k)) || !aligned16(rope) || (qw && !aligned16(qw)) || (kw && !aligned16(kw)))
         return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_neox: tensors must be 16-byte aligned");
     if (rows > 0x7fffffffu || n_q > 65535 || n_kv > 65535) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_neox: too large");
-    const uint64_t lanes = (uint64_t)rows * (n_q + n_kv) * (head_dim / 16);
-    const unsigned block = 256;
-    const uint64_t grid = (lanes + block - 1) / block;
+    // A wave owns (row, group of HPW*ITER heads); HPW = heads per wave pass.  The largest
+    // ITER that still leaves >= 1536 waves (6 per CU) amortises the row's [sin, cos] tile
+    // and the norm weights over the most heads; small batches take ITER = 1.
+    const size_t epl = 16 / es, lph = head_dim / 2 / epl, hpw = 64 / lph, hpr = n_q + n_kv;
+    int iter = 1;
+    for (int cand : {9, 3}) {
+        if ((size_t)cand > (hpr + hpw - 1) / hpw) continue;
+        const size_t groups = (hpr + hpw * cand - 1) / (hpw * cand);
+        if (rows * groups >= 1536) { iter = cand; break; }
+    }
+    const uint64_t waves = (uint64_t)rows * ((hpr + hpw * iter - 1) / (hpw * iter));
+    const unsigned block = iter == 9 ? 64 : 256;
+    const uint64_t grid = (waves * 64 + block - 1) / block;
     if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_neox: too large");
-    const int hd_i = head_dim == 64 ? 0 : head_dim == 128 ? 1 : 2;
-    const int which = (dtype == APK_F32 ? K_QKROPE_F32_64 : K_QKROPE_F16_64) + hd_i;
+    const std::string which = std::string("apk_qknorm_rope_") + (dtype == APK_F32 ? "f32" : "f16") + "_hd" +
+                              std::to_string(head_dim) + "_i" + std::to_string(iter);
     if (int rc = set_device(c)) return rc;
     int rows_i = (int)rows, nq_i = (int)n_q, nkv_i = (int)n_kv;
     void* args[] = {&q, &k, &qw, &kw, &rope, &rows_i, &nq_i, &nkv_i, &eps};
-    return launch(c, (Kernel)which, (unsigned)grid, block, 0, args);
+    return launch(c, which, (unsigned)grid, block, 0, args);
 }
 
 int apk_rope_table(apk_ctx* c, const uint32_t* positions, const float* inv_freq, size_t rows, size_t half, float* table) {
@@ -409,7 +435,7 @@ int apk_rope_table(apk_ctx* c, const uint32_t* positions, const float* inv_freq,
     int rows_i = (int)rows, half_i = (int)half;
     const uint64_t grid = ((uint64_t)rows * half + 255) / 256;
     void* args[] = {&positions, &inv_freq, &rows_i, &half_i, &table};
-    return launch(c, K_ROPE_TABLE, (unsigned)grid, 256, 0, args);
+    return launch(c, "apk_rope_table", (unsigned)grid, 256, 0, args);
 }
 
 static int embed_common(apk_ctx* c, int fmt, const void* table, size_t vocab, size_t n_in, const uint32_t* ids_dev,
@@ -423,23 +449,23 @@ static int embed_common(apk_ctx* c, int fmt, const void* table, size_t vocab, si
         return fail(APK_DECLINE_SHAPE, "apk_embed_rows: sizes out of range");
     if (int rc = set_device(c)) return rc;
     uint32_t vocab32 = (uint32_t)vocab;
-    int n_i = (int)n_in, t_i = (int)t;
+    int n_i = (int)n_in;
     if (fmt == APK_FMT_Q4K) {
-        const uint64_t lanes = (uint64_t)t * (n_in / 256) * 8;
-        const uint64_t grid = (lanes + 255) / 256;
-        if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_embed_rows: too large");
-        void* args[] = {&table, &vocab32, &n_i, &ids_dev, &t_i, &out, &c->fault_dev};
-        return launch(c, out_dtype == APK_F32 ? K_EMBED_Q4K_F32 : K_EMBED_Q4K_F16, (unsigned)grid, 256, 0, args);
+        // one workgroup per row, 8 lanes per 256-element super-block
+        size_t threads = (n_in / 256 * 8 + 63) / 64 * 64;
+        if (threads > 256) threads = 256;
+        void* args[] = {&table, &vocab32, &n_i, &ids_dev, &out, &c->fault_dev};
+        return launch(c, out_dtype == APK_F32 ? "apk_embed_q4k_f32" : "apk_embed_q4k_f16", (unsigned)t, (unsigned)threads, 0, args);
     }
     // Q8_0: one workgroup per row, the row staged in LDS
     const size_t row_bytes = n_in / 32 * 34;
     const size_t shmem = row_bytes + 32;
     if (shmem > 64 * 1024) return fail(APK_DECLINE_SHAPE, "apk_embed_rows: Q8_0 row of %zu elements is too long", n_in);
-    size_t threads = (n_in / 8 + 63) / 64 * 64;
+    size_t threads = (n_in / (16 / elem_size(out_dtype)) + 63) / 64 * 64;  // one output tile per lane
     if (threads > 1024) threads = 1024;
     uint64_t table_bytes = (uint64_t)vocab * row_bytes;
     void* args[] = {&table, &table_bytes, &vocab32, &n_i, &ids_dev, &out, &c->fault_dev};
-    return launch(c, out_dtype == APK_F32 ? K_EMBED_Q8_0_F32 : K_EMBED_Q8_0_F16, (unsigned)t, (unsigned)threads,
+    return launch(c, out_dtype == APK_F32 ? "apk_embed_q8_0_f32" : "apk_embed_q8_0_f16", (unsigned)t, (unsigned)threads,
                   (unsigned)shmem, args);
 }
 
@@ -495,7 +521,7 @@ int apk_route_topk(apk_ctx* c, const float* logits, const float* bias, size_t ro
     const unsigned block = 256, per_block = block / 64;
     const uint64_t grid = (rows + per_block - 1) / per_block;
     void* args[] = {&logits, &bias, &rows_i, &ne_i, &k_i, &norm, &scale, &sigmoid, &ids, &w};
-    return launch(c, K_ROUTE_TOPK, (unsigned)grid, block, 0, args);
+    return launch(c, "apk_route_topk", (unsigned)grid, block, 0, args);
 }
 
 int apk_moe_permute(apk_ctx* c, const uint32_t* ids, const float* w, size_t rows, size_t k, size_t n_expert,
@@ -510,7 +536,7 @@ int apk_moe_permute(apk_ctx* c, const uint32_t* ids, const float* w, size_t rows
     if (int rc = set_device(c)) return rc;
     int rows_i = (int)rows, k_i = (int)k, ne_i = (int)n_expert;
     void* args[] = {&ids, &w, &rows_i, &k_i, &ne_i, &table, &n_used, &tok, &tok_off, &hit_row, &hit_w, &c->fault_dev};
-    return launch(c, K_MOE_PERMUTE, (unsigned)n_expert, 512, 0, args);
+    return launch(c, "apk_moe_permute", (unsigned)n_expert, 512, 0, args);
 }
 
 int apk_gather_rows(apk_ctx* c, const void* src, const uint32_t* tok, size_t src_rows, size_t total_rows, size_t cols,
@@ -529,7 +555,7 @@ int apk_gather_rows(apk_ctx* c, const void* src, const uint32_t* tok, size_t src
     uint32_t src_rows32 = (uint32_t)src_rows;
     int row_vecs = (int)(cols * es / 16);
     void* args[] = {&src, &tok, &src_rows32, &row_vecs, &dst, &c->fault_dev};
-    return launch(c, K_GATHER_ROWS, (unsigned)total_rows, 256, 0, args);
+    return launch(c, "apk_gather_rows", (unsigned)total_rows, 256, 0, args);
 }
 
 int apk_copy(apk_ctx* c, const void* src, void* dst, size_t bytes) {
@@ -540,10 +566,10 @@ int apk_copy(apk_ctx* c, const void* src, void* dst, size_t bytes) {
     if (bytes % 16 || !aligned16(src) || !aligned16(dst)) return fail(APK_DECLINE_SHAPE, "apk_copy: whole 16-byte tiles only");
     if (int rc = set_device(c)) return rc;
     uint64_t nvec = bytes / 16;
-    const uint64_t grid = (nvec + 1023) / 1024;
+    const uint64_t grid = (nvec + 255) / 256;
     if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_copy: too large");
     void* args[] = {&src, &dst, &nvec};
-    return launch(c, K_COPY, (unsigned)grid, 256, 0, args);
+    return launch(c, "apk_copy", (unsigned)grid, 256, 0, args);
 }
 
 }  // extern "C"

@@ -35,6 +35,10 @@ DEV uint32_t f2h(float f) { return (uint32_t)__builtin_bit_cast(uint16_t, (f16_t
 template <typename T> struct io;
 template <> struct io<float> {
     static constexpr int VEC = 4;
+    typedef f32x4 raw_t;  // a tile as loaded: kept raw until all loads of a lane are in flight
+    DEV raw_t ldraw_nt(const float* p) { return __builtin_nontemporal_load((const f32x4*)p); }
+    DEV raw_t zero() { return f32x4{0.f, 0.f, 0.f, 0.f}; }
+    DEV void widen(raw_t t, float* v) { v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w; }
     DEV void load(const float* p, float* v) {
         f32x4 t = *(const f32x4*)p;
         v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
@@ -54,6 +58,10 @@ template <> struct io<float> {
 };
 template <> struct io<f16_t> {
     static constexpr int VEC = 8;
+    typedef u32x4 raw_t;
+    DEV raw_t ldraw_nt(const f16_t* p) { return __builtin_nontemporal_load((const u32x4*)p); }
+    DEV raw_t zero() { return u32x4{0u, 0u, 0u, 0u}; }
+    DEV void widen(raw_t t, float* v) { unpack(t, v); }
     DEV void unpack(u32x4 t, float* v) {
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -124,7 +132,7 @@ template <typename T, int UNR> DEV void swiglu_body(T* gate, const T* up, uint64
             gate[i] = (T)silu_mul<T>((float)gate[i], (float)up[i]);
     }
 }
-#define APK_SWIGLU_UNR 4
+#define APK_SWIGLU_UNR 1  // measured: 1 tile per lane streams best (most waves in flight)
 extern "C" __global__ __launch_bounds__(256) void apk_swiglu_f32(float* gate, const float* up, uint64_t n) {
     swiglu_body<float, APK_SWIGLU_UNR>(gate, up, n);
 }
@@ -136,179 +144,223 @@ extern "C" __global__ __launch_bounds__(256) void apk_swiglu_f16(f16_t* gate, co
 // Residual add + RMSNorm over rows (blas.rs:105-178 then norm.rs:193-269):
 //   x' = x + delta  (written back when delta != null)
 //   h  = ((x' as f64 * scale) as f32) * gamma,  scale = 1/sqrt(mean(x'^2)+eps)
-// One workgroup per row; each lane keeps its NCH 16-byte tiles of the row in
-// registers between the sum of squares and the scaling pass, so the row is
-// read from HBM once.  Wave sums by shuffle, cross-wave through LDS.
+// One workgroup of W waves per row; each lane keeps its NCH 16-byte tiles of
+// the row in registers between the sum of squares and the scaling pass, so the
+// row is read from HBM once.  The host picks W so that every row of a large
+// batch is resident at once (W = 1: a wave per row, no LDS, no barrier).
+// f32 activations: statistics and scaling in f64, exactly the reference's
+// operations.  fp16 activations: the output keeps 11 bits, so the statistics
+// are f32 (8-element partial sums, then a tree) and the scaling is two f32
+// multiplies; the result stays within 1 ulp of fp16 of the f64 form.
 // =========================================================================
-template <typename T, int NCH>
-DEV void add_rmsnorm_body(T* x, const T* delta, T* h, const float* gamma, int n, float eps) {
+template <typename T> struct stat;
+template <> struct stat<float> {
+    typedef double acc_t;
+    DEV double sq(double a, float v) { return __builtin_fma((double)v, (double)v, a); }
+    DEV double wave_sum(double v) { return wave_sum_f64(v, 64); }
+    DEV double rscale(double ss, int n, float eps) { return 1.0 / sqrt(ss / (double)n + (double)eps); }
+    DEV float apply(float v, double scale, float g) { return (float)((double)v * scale) * g; }
+};
+template <> struct stat<f16_t> {
+    typedef float acc_t;
+    DEV float sq(float a, float v) { return __builtin_fmaf(v, v, a); }
+    DEV float wave_sum(float v) {
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) v += __shfl_xor(v, o, 64);
+        return v;
+    }
+    DEV float rscale(float ss, int n, float eps) { return __builtin_amdgcn_rsqf(ss * (1.0f / (float)n) + eps); }
+    DEV float apply(float v, float scale, float g) { return v * scale * g; }
+};
+
+template <typename T, int NCH, bool HAS_DELTA>
+DEV void add_rmsnorm_impl(T* x, const T* delta, T* h, const float* gamma, int n, float eps) {
     constexpr int VEC = io<T>::VEC;
-    __shared__ double part[16];
+    typedef typename stat<T>::acc_t acc_t;
+    __shared__ acc_t part[16];
     const int nchunks = n / VEC;
     const uint64_t row = blockIdx.x;
     T* xr = x + row * (uint64_t)n;
     T* hr = h + row * (uint64_t)n;
-    const T* dr = delta ? delta + row * (uint64_t)n : nullptr;
+    const T* dr = HAS_DELTA ? delta + row * (uint64_t)n : nullptr;
 
+    // Every load of the lane is issued before the first use: no branch and no
+    // conversion in this loop (a lane past the end of the row re-reads the last tile).
+    typename io<T>::raw_t xraw[NCH], draw[NCH];
+#pragma unroll
+    for (int j = 0; j < NCH; j++) {
+        const int c = min((int)(threadIdx.x + j * blockDim.x), nchunks - 1);
+        xraw[j] = io<T>::ldraw_nt(xr + c * VEC);
+        if constexpr (HAS_DELTA) draw[j] = io<T>::ldraw_nt(dr + c * VEC);
+    }
     float v[NCH][VEC];
-    float d[NCH][VEC];
+    acc_t ss = 0;
 #pragma unroll
     for (int j = 0; j < NCH; j++) {
-        int c = threadIdx.x + j * blockDim.x;
-        if (c < nchunks) {
-            io<T>::load_nt(xr + c * VEC, v[j]);
-            if (dr) io<T>::load_nt(dr + c * VEC, d[j]);
+        const int c = threadIdx.x + j * blockDim.x;
+        io<T>::widen(xraw[j], v[j]);
+        if constexpr (HAS_DELTA) {
+            float d[VEC];
+            io<T>::widen(draw[j], d);
+#pragma unroll
+            for (int i = 0; i < VEC; i++) v[j][i] = v[j][i] + d[i];
+            if (c < nchunks) io<T>::store(xr + c * VEC, v[j]);
         }
+        acc_t s8 = 0;
+#pragma unroll
+        for (int i = 0; i < VEC; i++) s8 = stat<T>::sq(s8, v[j][i]);
+        ss += c < nchunks ? s8 : (acc_t)0;
     }
-    double ss = 0.0;
-#pragma unroll
-    for (int j = 0; j < NCH; j++) {
-        int c = threadIdx.x + j * blockDim.x;
-        if (c < nchunks) {
-            if (dr) {
-#pragma unroll
-                for (int i = 0; i < VEC; i++) v[j][i] = v[j][i] + d[j][i];
-                io<T>::store(xr + c * VEC, v[j]);
-            }
-#pragma unroll
-            for (int i = 0; i < VEC; i++) ss = __builtin_fma((double)v[j][i], (double)v[j][i], ss);
-        }
-    }
-    ss = wave_sum_f64(ss, 64);
+    ss = stat<T>::wave_sum(ss);
     const int nwaves = (blockDim.x + 63) >> 6;
     if (nwaves > 1) {
         if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
         __syncthreads();
-        ss = 0.0;
+        ss = 0;
         for (int w = 0; w < nwaves; w++) ss += part[w];
     }
-    const double scale = 1.0 / sqrt(ss / (double)n + (double)eps);
+    const acc_t scale = stat<T>::rscale(ss, n, eps);
 #pragma unroll
     for (int j = 0; j < NCH; j++) {
-        int c = threadIdx.x + j * blockDim.x;
+        const int c = threadIdx.x + j * blockDim.x;
         if (c < nchunks) {
             float g[VEC], o[VEC];
 #pragma unroll
             for (int q = 0; q < VEC; q += 4) io<float>::load(gamma + c * VEC + q, g + q);
 #pragma unroll
-            for (int i = 0; i < VEC; i++) o[i] = (float)((double)v[j][i] * scale) * g[i];
+            for (int i = 0; i < VEC; i++) o[i] = stat<T>::apply(v[j][i], scale, g[i]);
             io<T>::store_nt(hr + c * VEC, o);
         }
     }
 }
-#define APK_ADDNORM(NAME, T, NCH)                                                                                  \
-    extern "C" __global__ __launch_bounds__(1024) void NAME(T* x, const T* delta, T* h, const float* gamma, int n, \
-                                                            float eps) {                                           \
-        add_rmsnorm_body<T, NCH>(x, delta, h, gamma, n, eps);                                                      \
+template <typename T, int NCH>
+DEV void add_rmsnorm_body(T* x, const T* delta, T* h, const float* gamma, int n, float eps) {
+    if (delta) add_rmsnorm_impl<T, NCH, true>(x, delta, h, gamma, n, eps);   // uniform for the launch
+    else add_rmsnorm_impl<T, NCH, false>(x, delta, h, gamma, n, eps);
+}
+// The launch bound is the largest workgroup the host uses with that tile count
+// (it also caps the registers the compiler may take: 512 / (bound/64/4) per lane).
+#define APK_ADDNORM(T, TN, NCH, MAXT)                                                                        \
+    extern "C" __global__ __launch_bounds__(MAXT) void apk_add_rmsnorm_##TN##_c##NCH(                        \
+        T* x, const T* delta, T* h, const float* gamma, int n, float eps) {                                  \
+        add_rmsnorm_body<T, NCH>(x, delta, h, gamma, n, eps);                                                \
     }
-APK_ADDNORM(apk_add_rmsnorm_f32_c1, float, 1)
-APK_ADDNORM(apk_add_rmsnorm_f32_c2, float, 2)
-APK_ADDNORM(apk_add_rmsnorm_f32_c4, float, 4)
-APK_ADDNORM(apk_add_rmsnorm_f32_c8, float, 8)
-APK_ADDNORM(apk_add_rmsnorm_f16_c1, f16_t, 1)
-APK_ADDNORM(apk_add_rmsnorm_f16_c2, f16_t, 2)
-APK_ADDNORM(apk_add_rmsnorm_f16_c4, f16_t, 4)
-APK_ADDNORM(apk_add_rmsnorm_f16_c8, f16_t, 8)
+#define APK_ADDNORM_ALL(T, TN)                                                                                   \
+    APK_ADDNORM(T, TN, 1, 1024) APK_ADDNORM(T, TN, 2, 1024) APK_ADDNORM(T, TN, 3, 512) APK_ADDNORM(T, TN, 4, 512) \
+    APK_ADDNORM(T, TN, 5, 256) APK_ADDNORM(T, TN, 6, 256) APK_ADDNORM(T, TN, 8, 256) APK_ADDNORM(T, TN, 10, 256)  \
+    APK_ADDNORM(T, TN, 12, 256) APK_ADDNORM(T, TN, 16, 256) APK_ADDNORM(T, TN, 20, 256)
+APK_ADDNORM_ALL(float, f32)
+APK_ADDNORM_ALL(f16_t, f16)
 
 // =========================================================================
 // Per-head QK-norm + NeoX RoPE, in place on q [rows, n_q*HD] and k [rows, n_kv*HD]
 // (caller loop attention.rs:131-165: rmsnorm(head, w, eps) then the NeoX
 // rotation with the row's [sin, cos] table, rope.rs:70-81).
-// HD/16 lanes own one head: lane l holds elements [8l, 8l+8) of the first half
-// and their NeoX partners [HD/2+8l, HD/2+8l+8), so the rotation needs no
-// cross-lane traffic and every global access is a 16-byte tile inside a
-// 128-byte run.  The sum of squares crosses only those HD/16 lanes.
+// Lane mapping: a lane holds one 16-byte tile of the first half of a head and
+// the tile of its NeoX partners in the second half (EPL = 8 fp16 / 4 f32
+// elements each), so the rotation needs no cross-lane traffic, every global
+// access is a full 16-byte tile and the LPH = HD/2/EPL lanes of a head cover
+// contiguous runs.  A wave owns (row, group of HPW*ITER consecutive heads),
+// HPW = 64/LPH heads per pass: the row's [sin, cos] tile and both norm weights
+// are loaded once per wave and reused over ITER passes.  The host picks ITER so
+// that a large batch is one resident round of waves.
+// f32 activations: f64 statistics and scaling, no contraction: the reference's
+// operations.  fp16 activations: f32 statistics (the output keeps 11 bits).
 // =========================================================================
-template <typename T, int HD>
+template <typename T, int HD, int ITER>
 DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv,
                           float eps) {
-    constexpr int LPH = HD / 16;  // lanes per head
+    constexpr int EPL = io<T>::VEC;       // elements per lane per half
     constexpr int HALF = HD / 2;
-    const uint64_t gl = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const uint64_t gh = gl / LPH;
-    const int l = (int)(gl % LPH);
+    constexpr int LPH = HALF / EPL;       // lanes per head
+    constexpr int HPW = 64 / LPH;         // heads per wave pass
+    typedef typename stat<T>::acc_t acc_t;
+    const int lane = threadIdx.x & 63;
+    const int l = lane % LPH, sub = lane / LPH;
     const int hpr = n_q + n_kv;
-    const uint64_t total = (uint64_t)rows * hpr;
-    const bool live = gh < total;
-    const uint64_t row = live ? gh / hpr : 0;
-    const int hh = live ? (int)(gh % hpr) : 0;
-    const bool is_q = hh < n_q;
-    T* head = is_q ? q + (row * n_q + hh) * HD : k + (row * n_kv + (hh - n_q)) * HD;
-    const float* w = is_q ? qw : kw;
+    const int groups = (hpr + HPW * ITER - 1) / (HPW * ITER);
+    const uint64_t wid = ((uint64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    if (wid >= (uint64_t)rows * groups) return;  // whole wave
+    const uint64_t row = wid / groups;
+    const int g = (int)(wid % groups);
 
-    float a[8], b[8];
-    if (live) {
-        if constexpr (sizeof(T) == 2) {
-            io<T>::load_nt(head + 8 * l, a);
-            io<T>::load_nt(head + HALF + 8 * l, b);
-        } else {
-            io<T>::load_nt(head + 8 * l, a);
-            io<T>::load_nt(head + 8 * l + 4, a + 4);
-            io<T>::load_nt(head + HALF + 8 * l, b);
-            io<T>::load_nt(head + HALF + 8 * l + 4, b + 4);
-        }
-    } else {
+    // Loads return in issue order, so the small cached ones go first: the first pass can
+    // start as soon as its own two tiles arrive.
+    // [sin, cos] of pairs [EPL*l, EPL*l+EPL): 2*EPL consecutive floats of the row's table
+    const float* trow = rope + row * HD;
+    float sc[2 * EPL];
 #pragma unroll
-        for (int i = 0; i < 8; i++) a[i] = b[i] = 0.0f;
+    for (int i = 0; i < 2 * EPL; i += 4) io<float>::load(trow + 2 * EPL * l + i, sc + i);
+    const float* qwp = qw ? qw : trow;
+    const float* kwp = kw ? kw : trow;
+    float wqa[EPL], wqb[EPL], wka[EPL], wkb[EPL];
+#pragma unroll
+    for (int i = 0; i < EPL; i += 4) {
+        io<float>::load(qwp + EPL * l + i, wqa + i);
+        io<float>::load(qwp + HALF + EPL * l + i, wqb + i);
+        io<float>::load(kwp + EPL * l + i, wka + i);
+        io<float>::load(kwp + HALF + EPL * l + i, wkb + i);
     }
-    // [sin, cos] pairs of this row for i in [8l, 8l+8): 16 consecutive floats
-    float sc[16];
-    if (live) {
-        const float* t = rope + (row * HALF + 8 * l) * 2;
+    // Every load of the wave is issued before the first use, without branches: a lane
+    // of a pass beyond the last head re-reads the row's last head and stores nothing;
+    // a missing norm weight is read from the [sin, cos] tile instead and never used.
+    typename io<T>::raw_t araw[ITER], braw[ITER];
+    T* hp[ITER];
+    bool live[ITER], isq[ITER];
 #pragma unroll
-        for (int i = 0; i < 16; i += 4) io<float>::load(t + i, sc + i);
+    for (int it = 0; it < ITER; it++) {
+        const int hh0 = (g * ITER + it) * HPW + sub;
+        live[it] = hh0 < hpr;
+        const int hh = min(hh0, hpr - 1);
+        isq[it] = hh < n_q;
+        hp[it] = isq[it] ? q + (row * n_q + hh) * HD : k + (row * n_kv + (hh - n_q)) * HD;
+        araw[it] = io<T>::ldraw_nt(hp[it] + EPL * l);
+        braw[it] = io<T>::ldraw_nt(hp[it] + HALF + EPL * l);
     }
-    if (w != nullptr) {  // uniform across the lanes of a head (and nearly always the wave)
-        float wa[8], wb[8];
 #pragma unroll
-        for (int i = 0; i < 8; i += 4) {
-            io<float>::load(w + 8 * l + i, wa + i);
-            io<float>::load(w + HALF + 8 * l + i, wb + i);
+    for (int it = 0; it < ITER; it++) {
+        const bool normed = isq[it] ? (qw != nullptr) : (kw != nullptr);  // uniform over the lanes of a head
+        float a[EPL], b[EPL];
+        io<T>::widen(araw[it], a);
+        io<T>::widen(braw[it], b);
+        acc_t ss = 0;
+#pragma unroll
+        for (int i = 0; i < EPL; i++) {
+            ss = stat<T>::sq(ss, a[i]);
+            ss = stat<T>::sq(ss, b[i]);
         }
-        double ss = 0.0;
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            ss = __builtin_fma((double)a[i], (double)a[i], ss);
-            ss = __builtin_fma((double)b[i], (double)b[i], ss);
-        }
-        ss = wave_sum_f64(ss, LPH);
-        const double scale = 1.0 / sqrt(ss / (double)HD + (double)eps);
+        for (int o = 1; o < LPH; o <<= 1) ss += __shfl_xor(ss, o, 64);
+        const acc_t scale = stat<T>::rscale(ss, HD, eps);
+        float oa[EPL], ob[EPL];
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            a[i] = (float)((double)a[i] * scale) * wa[i];
-            b[i] = (float)((double)b[i] * scale) * wb[i];
-        }
-    }
-    if (live) {
-        float oa[8], ob[8];
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
+        for (int i = 0; i < EPL; i++) {
+            float x = a[i], y = b[i];
+            if (normed) {
+                x = stat<T>::apply(x, scale, isq[it] ? wqa[i] : wka[i]);
+                y = stat<T>::apply(y, scale, isq[it] ? wqb[i] : wkb[i]);
+            }
             const float s = sc[2 * i], c = sc[2 * i + 1];
-            oa[i] = a[i] * c - b[i] * s;
-            ob[i] = a[i] * s + b[i] * c;
+            oa[i] = x * c - y * s;
+            ob[i] = x * s + y * c;
         }
-        if constexpr (sizeof(T) == 2) {
-            io<T>::store_nt(head + 8 * l, oa);
-            io<T>::store_nt(head + HALF + 8 * l, ob);
-        } else {
-            io<T>::store_nt(head + 8 * l, oa);
-            io<T>::store_nt(head + 8 * l + 4, oa + 4);
-            io<T>::store_nt(head + HALF + 8 * l, ob);
-            io<T>::store_nt(head + HALF + 8 * l + 4, ob + 4);
+        if (live[it]) {
+            io<T>::store_nt(hp[it] + EPL * l, oa);
+            io<T>::store_nt(hp[it] + HALF + EPL * l, ob);
         }
     }
 }
-#define APK_QKROPE(NAME, T, HD)                                                                                        \
-    extern "C" __global__ __launch_bounds__(256) void NAME(T* q, T* k, const float* qw, const float* kw,               \
-                                                           const float* rope, int rows, int n_q, int n_kv, float eps) { \
-        qknorm_rope_body<T, HD>(q, k, qw, kw, rope, rows, n_q, n_kv, eps);                                             \
+#define APK_QKROPE(T, TN, HD, ITER)                                                                          \
+    extern "C" __global__ __launch_bounds__(256) void apk_qknorm_rope_##TN##_hd##HD##_i##ITER(              \
+        T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv, float eps) { \
+        qknorm_rope_body<T, HD, ITER>(q, k, qw, kw, rope, rows, n_q, n_kv, eps);                              \
     }
-APK_QKROPE(apk_qknorm_rope_f32_hd64, float, 64)
-APK_QKROPE(apk_qknorm_rope_f32_hd128, float, 128)
-APK_QKROPE(apk_qknorm_rope_f32_hd256, float, 256)
-APK_QKROPE(apk_qknorm_rope_f16_hd64, f16_t, 64)
-APK_QKROPE(apk_qknorm_rope_f16_hd128, f16_t, 128)
-APK_QKROPE(apk_qknorm_rope_f16_hd256, f16_t, 256)
+#define APK_QKROPE_ALL(T, TN)                                                                           \
+    APK_QKROPE(T, TN, 64, 1) APK_QKROPE(T, TN, 64, 3) APK_QKROPE(T, TN, 64, 9)                          \
+    APK_QKROPE(T, TN, 128, 1) APK_QKROPE(T, TN, 128, 3) APK_QKROPE(T, TN, 128, 9)                       \
+    APK_QKROPE(T, TN, 256, 1) APK_QKROPE(T, TN, 256, 3) APK_QKROPE(T, TN, 256, 9)
+APK_QKROPE_ALL(float, f32)
+APK_QKROPE_ALL(f16_t, f16)
 
 // RoPE table rows from per-row positions (rope.rs:18-22, session.rs:34-50):
 // table[r][i] = [sin, cos]((pos[r] as f32) * inv_freq[i]).  One f32 rounding of
@@ -329,93 +381,112 @@ extern "C" __global__ __launch_bounds__(256) void apk_rope_table(const uint32_t*
 // The dequant is fused into the gather; the id is read on the device.
 // An id >= vocab raises APK_FAULT_TOKEN_RANGE and leaves its row untouched.
 // =========================================================================
-template <typename TO> DEV void store8(TO* p, const float* v);
-template <> __device__ __forceinline__ void store8<float>(float* p, const float* v) {
-    io<float>::store_nt(p, v);
-    io<float>::store_nt(p + 4, v + 4);
-}
-template <> __device__ __forceinline__ void store8<f16_t>(f16_t* p, const float* v) { io<f16_t>::store_nt(p, v); }
-
 // Q4_K (dequant.rs:211-231): 144-byte super-block = d, dmin (f16), 12 packed
-// scale bytes, 128 quant bytes.  8 lanes per super-block; lane j owns 16 quant
-// bytes = 16 low-nibble outputs of sub-block 2p and 16 high-nibble outputs of
-// sub-block 2p+1 (p = j/2).  d*sc, dmin*mn, (d*sc)*q and the subtraction are
-// four separately rounded f32 operations.
-template <typename TO>
-DEV void embed_q4k_body(const uint8_t* table, uint32_t vocab, int n_in, const uint32_t* ids, int t_rows, TO* out,
-                        uint32_t* fault) {
-    const int nsb = n_in / 256;
-    const uint64_t gl = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const uint64_t per_row = (uint64_t)nsb * 8;
-    const uint64_t t = gl / per_row;
-    if (t >= (uint64_t)t_rows) return;
-    const int rem = (int)(gl % per_row);
-    const int sb = rem >> 3, j = rem & 7;
-    const uint32_t id = ids[t];
-    if (id >= vocab) {
-        if (rem == 0) atomicOr(fault, APK_FAULT_TOKEN_RANGE);
-        return;
-    }
-    const uint8_t* blk = table + (uint64_t)id * ((uint64_t)nsb * 144) + (uint64_t)sb * 144;
-    const u32x4 hdr = *(const u32x4*)blk;
-    const u32x4 qs = __builtin_nontemporal_load((const u32x4*)(blk + 16 + 16 * j));
-    const float d = h2f(hdr.x & 0xffffu), dmin = h2f(hdr.x >> 16);
-    // the 12 packed bytes are hdr.y, hdr.z, hdr.w (little endian)
-    const int p = j >> 1;
-    uint32_t sc1, mn1, sc2, mn2;
+// scale bytes, 128 quant bytes -> 256 outputs.  d*sc, dmin*mn, (d*sc)*q and the
+// subtraction are four separately rounded f32 operations.
+// One workgroup per output row; 8 lanes share a super-block and are laid out so
+// that EVERY store instruction writes one full, contiguous 128-byte line per
+// super-block (partial-line streaming stores cost more than 2x here):
+//   fp16 out: store k (0..3) of lane L covers outputs [64k + 8L, +8): sub-block
+//             2k + L/4, i.e. quant bytes qs[32k + 8(L%4), +8), low nibbles for
+//             L < 4 and high nibbles for L >= 4;
+//   f32 out : store k (0..7) of lane L covers outputs [32k + 4L, +4): sub-block k,
+//             quant bytes qs[32(k/2) + 4L, +4), low nibbles for even k.
+DEV void k4_scale_min(const u32x4 hdr, int s, float& sc, float& mn) {
+    // the 12 packed bytes are hdr.y, hdr.z, hdr.w (little endian); scale_min_k4, allpaka-dtype lib.rs:382-390
     auto byte_at = [&](int i) -> uint32_t {
         uint32_t w = i < 4 ? hdr.y : (i < 8 ? hdr.z : hdr.w);
         return (w >> (8 * (i & 3))) & 0xffu;
     };
-    auto scale_min = [&](int s, uint32_t& sc, uint32_t& mn) {
-        if (s < 4) {
-            sc = byte_at(s) & 63u;
-            mn = byte_at(s + 4) & 63u;
+    uint32_t a, b;
+    if (s < 4) {
+        a = byte_at(s) & 63u;
+        b = byte_at(s + 4) & 63u;
+    } else {
+        a = (byte_at(s + 4) & 0xfu) | ((byte_at(s - 4) >> 6) << 4);
+        b = (byte_at(s + 4) >> 4) | ((byte_at(s) >> 6) << 4);
+    }
+    sc = (float)a;
+    mn = (float)b;
+}
+
+template <typename TO>
+DEV void embed_q4k_body(const uint8_t* table, uint32_t vocab, int n_in, const uint32_t* ids, TO* out, uint32_t* fault) {
+    const int nsb = n_in / 256;
+    const uint64_t t = blockIdx.x;
+    const uint32_t id = ids[t];
+    if (id >= vocab) {
+        if (threadIdx.x == 0) atomicOr(fault, APK_FAULT_TOKEN_RANGE);
+        return;
+    }
+    const uint8_t* row = table + (uint64_t)id * ((uint64_t)nsb * 144);
+    TO* orow = out + t * (uint64_t)n_in;
+    for (int rem = threadIdx.x; rem < nsb * 8; rem += blockDim.x) {
+        const int sb = rem >> 3, L = rem & 7;
+        const uint8_t* blk = row + (uint64_t)sb * 144;
+        const u32x4 hdr = *(const u32x4*)blk;
+        const float d = h2f(hdr.x & 0xffffu), dmin = h2f(hdr.x >> 16);
+        if constexpr (sizeof(TO) == 2) {
+            u32x2 qs[4];
+#pragma unroll
+            for (int k = 0; k < 4; k++) qs[k] = *(const u32x2*)(blk + 16 + k * 32 + (L & 3) * 8);
+            const int hi = L >> 2;
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                float sc, mn;
+                k4_scale_min(hdr, 2 * k + hi, sc, mn);
+                const float dl = d * sc, ml = dmin * mn;
+                float v[8];
+#pragma unroll
+                for (int w = 0; w < 2; w++)
+#pragma unroll
+                    for (int b = 0; b < 4; b++) {
+                        const uint32_t byte = (qs[k][w] >> (8 * b)) & 0xffu;
+                        const uint32_t qv = hi ? (byte >> 4) : (byte & 0xfu);
+                        v[4 * w + b] = dl * (float)qv - ml;
+                    }
+                io<f16_t>::store_nt((f16_t*)orow + (uint64_t)sb * 256 + k * 64 + L * 8, v);
+            }
         } else {
-            sc = (byte_at(s + 4) & 0xfu) | ((byte_at(s - 4) >> 6) << 4);
-            mn = (byte_at(s + 4) >> 4) | ((byte_at(s) >> 6) << 4);
-        }
-    };
-    scale_min(2 * p, sc1, mn1);
-    scale_min(2 * p + 1, sc2, mn2);
-    const float d_sc1 = d * (float)sc1, dm1 = dmin * (float)mn1;
-    const float d_sc2 = d * (float)sc2, dm2 = dmin * (float)mn2;
-    float lo[16], hi[16];
+            uint32_t qs[4];
 #pragma unroll
-    for (int w = 0; w < 4; w++) {
+            for (int pr = 0; pr < 4; pr++) qs[pr] = *(const uint32_t*)(blk + 16 + pr * 32 + L * 4);
 #pragma unroll
-        for (int b = 0; b < 4; b++) {
-            const uint32_t byte = (qs[w] >> (8 * b)) & 0xffu;
-            lo[4 * w + b] = d_sc1 * (float)(byte & 0xfu) - dm1;
-            hi[4 * w + b] = d_sc2 * (float)(byte >> 4) - dm2;
+            for (int k = 0; k < 8; k++) {
+                float sc, mn;
+                k4_scale_min(hdr, k, sc, mn);
+                const float dl = d * sc, ml = dmin * mn;
+                float v[4];
+#pragma unroll
+                for (int b = 0; b < 4; b++) {
+                    const uint32_t byte = (qs[k >> 1] >> (8 * b)) & 0xffu;
+                    const uint32_t qv = (k & 1) ? (byte >> 4) : (byte & 0xfu);
+                    v[b] = dl * (float)qv - ml;
+                }
+                io<float>::store_nt((float*)orow + (uint64_t)sb * 256 + k * 32 + L * 4, v);
+            }
         }
     }
-    TO* o = out + t * (uint64_t)n_in + (uint64_t)sb * 256 + p * 64 + 16 * (j & 1);
-    store8<TO>(o, lo);
-    store8<TO>(o + 8, lo + 8);
-    store8<TO>(o + 32, hi);
-    store8<TO>(o + 40, hi + 8);
 }
 extern "C" __global__ __launch_bounds__(256) void apk_embed_q4k_f32(const uint8_t* table, uint32_t vocab, int n_in,
-                                                                   const uint32_t* ids, int t_rows, float* out,
-                                                                   uint32_t* fault) {
-    embed_q4k_body<float>(table, vocab, n_in, ids, t_rows, out, fault);
+                                                                   const uint32_t* ids, float* out, uint32_t* fault) {
+    embed_q4k_body<float>(table, vocab, n_in, ids, out, fault);
 }
 extern "C" __global__ __launch_bounds__(256) void apk_embed_q4k_f16(const uint8_t* table, uint32_t vocab, int n_in,
-                                                                   const uint32_t* ids, int t_rows, f16_t* out,
-                                                                   uint32_t* fault) {
-    embed_q4k_body<f16_t>(table, vocab, n_in, ids, t_rows, out, fault);
+                                                                   const uint32_t* ids, f16_t* out, uint32_t* fault) {
+    embed_q4k_body<f16_t>(table, vocab, n_in, ids, out, fault);
 }
 
 // Q8_0 (dequant.rs:94-126): 34-byte block = f16 scale + 32 int8; out = d * q.
 // Blocks are only 2-byte aligned, so one workgroup stages its row in LDS with
 // 16-byte loads (from the 16-byte-aligned address at or below the row start)
-// and each lane then decodes 8 outputs from LDS.  grid = rows, block = n_in/8
-// lanes (rounded up to a wave), looping when the row is longer than the block.
+// and each lane then decodes one 16-byte output tile (8 fp16 / 4 f32) per pass
+// from LDS, consecutive lanes writing consecutive tiles.
 template <typename TO>
 DEV void embed_q8_0_body(const uint8_t* table, uint64_t table_bytes, uint32_t vocab, int n_in, const uint32_t* ids,
                          TO* out, uint32_t* fault) {
     extern __shared__ __attribute__((aligned(16))) uint8_t stage[];
+    constexpr int OPT = io<TO>::VEC;  // outputs per tile
     const uint64_t t = blockIdx.x;
     const uint32_t id = ids[t];
     if (id >= vocab) {
@@ -441,20 +512,21 @@ DEV void embed_q8_0_body(const uint8_t* table, uint64_t table_bytes, uint32_t vo
         *(u32x4*)(stage + i * 16) = v;
     }
     __syncthreads();
-    const int ngroups = n_in / 8;
-    for (int g = threadIdx.x; g < ngroups; g += blockDim.x) {
-        const int blk = g >> 2, qtr = g & 3;
+    const int ntiles = n_in / OPT;
+    constexpr int TPB = 32 / OPT;  // tiles per 32-element block
+    for (int g = threadIdx.x; g < ntiles; g += blockDim.x) {
+        const int blk = g / TPB, part = g % TPB;
         const uint8_t* b = stage + mis + blk * 34;  // 2-byte aligned
         const float d = h2f(*(const uint16_t*)b);
-        const uint16_t* qp = (const uint16_t*)(b + 2 + 8 * qtr);
-        float o[8];
+        const uint16_t* qp = (const uint16_t*)(b + 2 + OPT * part);
+        float o[OPT];
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
+        for (int i = 0; i < OPT / 2; i++) {
             const uint32_t two = qp[i];
             o[2 * i] = d * (float)(int8_t)(two & 0xffu);
             o[2 * i + 1] = d * (float)(int8_t)(two >> 8);
         }
-        store8<TO>(out + t * (uint64_t)n_in + (uint64_t)g * 8, o);
+        io<TO>::store_nt(out + t * (uint64_t)n_in + (uint64_t)g * OPT, o);
     }
 }
 extern "C" __global__ __launch_bounds__(1024) void apk_embed_q8_0_f32(const uint8_t* table, uint64_t table_bytes,
@@ -684,18 +756,8 @@ extern "C" __global__ __launch_bounds__(256) void apk_gather_rows(const u32x4* s
     }
 }
 
-// Reference stream for bandwidth calibration: dst = src, 16-byte tiles.
+// Reference stream for bandwidth calibration: dst = src, one 16-byte tile per lane.
 extern "C" __global__ __launch_bounds__(256) void apk_copy(const u32x4* src, u32x4* dst, uint64_t nvec) {
-    const uint64_t base = (uint64_t)blockIdx.x * (blockDim.x * 4) + threadIdx.x;
-    u32x4 v[4];
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        uint64_t c = base + (uint64_t)j * blockDim.x;
-        if (c < nvec) v[j] = __builtin_nontemporal_load(src + c);
-    }
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        uint64_t c = base + (uint64_t)j * blockDim.x;
-        if (c < nvec) __builtin_nontemporal_store(v[j], dst + c);
-    }
+    const uint64_t c = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c < nvec) __builtin_nontemporal_store(__builtin_nontemporal_load(src + c), dst + c);
 }

@@ -1,0 +1,346 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused per-layer ops on ONE MI355X.
+
+A "step" is one decoder layer's worth of the hot path at Qwen3-32B shapes,
+T=2048 prefill rows, fp16 activations (BASELINE configs[2]):
+    add+RMSNorm (attention norm) -> per-head QK-norm + NeoX RoPE ->
+    add+RMSNorm (FFN norm) -> SwiGLU
+i.e. 4 launches per layer, inputs resident in HBM.  Every op cycles through its
+own pool of distinct buffer sets of more than 640 MB, so no launch is served
+from the 256 MB last-level cache ("cold" = HBM numbers).  Every op is also
+timed on its own, at every BASELINE shape, with HIP events on the library's
+stream (3 untimed launches first).  The JSON line carries
+    value     = microseconds per layer (lower is better),
+    roofline  = the dominant kernel (SwiGLU, 300 MiB per launch) against 8 TB/s,
+    per_op    = us / GB/s / fraction of peak / launches for every op and shape,
+    cpu_baseline = the CPU oracle (a C restatement of the reference's CPU path with
+                   the reference's threading rules) timed on this box's host cores.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_GBS = 8000.0  # MI355X HBM3E peak
+COLD_BYTES = 640e6  # every op rotates through at least this many distinct bytes
+
+# FETCH_SIZE / WRITE_SIZE of the dominant kernel (rocprofv3 --pmc, KiB per dispatch,
+# scaled by the same counters on apk_copy of a known size); see profiles/.
+TRAFFIC_BYTES_PER_LAUNCH = None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=60)
+    ap.add_argument("--warmup", type=int, default=12)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--rows", type=int, default=2048, help="prefill rows T of the timed step")
+    ap.add_argument("--shapes", choices=["all", "headline"], default="all",
+                    help="headline: only the timed layer chain and its per-op timings (what the rocprof summaries are made from)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the path is row-parallel and shards by rows with no "
+              f"communication); --gpus {args.gpus} is not run", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    import allpaka_amd.lib as apklib
+    from allpaka_amd import synth
+
+    L = apklib.load()  # raises if libapk_hip.so is not built: no fallback
+    h = C.c_void_p()
+    apklib.check(L.apk_init(0, C.byref(h)))
+    dev = torch.device("cuda", 0)
+    F16, F32 = apklib.F16, apklib.F32
+    gen = torch.Generator(device=dev).manual_seed(0xA11A)
+
+    def randn(shape, dtype=torch.float16):
+        return torch.randn(shape, generator=gen, device=dev, dtype=torch.float32).to(dtype)
+
+    def pool(set_bytes, make):
+        """enough distinct sets that one cycle touches more than COLD_BYTES"""
+        return [make() for _ in range(max(3, int(COLD_BYTES // set_bytes) + 1))]
+
+    def p(t):
+        return t.data_ptr()
+
+    def sync():
+        apklib.check(L.apk_sync(h))
+
+    def timed(fn, reps):
+        """avg microseconds per call of fn(i): HIP events on the library's stream, after 3 untimed calls"""
+        for i in range(3):
+            fn(i)
+        ms = C.c_float()
+        apklib.check(L.apk_timer_begin(h))
+        for i in range(reps):
+            fn(i + 3)
+        apklib.check(L.apk_timer_end(h, C.byref(ms)))
+        return ms.value * 1000.0 / reps
+
+    per_op = []
+
+    def record(op, shape, us, nbytes, launches=1, note=None):
+        gbs = nbytes / us / 1e3
+        e = {"op": op, "shape": shape, "us": round(us, 3), "bytes": int(nbytes), "GBps": round(gbs, 1),
+             "frac_of_peak": round(gbs / PEAK_GBS, 4), "launches": launches}
+        if note:
+            e["note"] = note
+        per_op.append(e)
+        return e
+
+    # ------------------------------------------------ Qwen3-32B, fp16 (configs 2, 3)
+    m = synth.MODELS["qwen3-32b"]
+    H, NQ, NKV, HD, FF, EPS = m["hidden"], m["n_q"], m["n_kv"], m["head_dim"], m["ffn"], m["eps"]
+    T = args.rows
+    b = 2
+    gamma1 = 1 + 0.05 * randn(H, torch.float32)
+    gamma2 = 1 + 0.05 * randn(H, torch.float32)
+    qw = 1 + 0.05 * randn(HD, torch.float32)
+    kw = 1 + 0.05 * randn(HD, torch.float32)
+    inv = torch.tensor(np.float32(m["theta"]) ** (-2.0 * np.arange(HD // 2, dtype=np.float32) / np.float32(HD)), device=dev)
+    pos = torch.arange(T, dtype=torch.int32, device=dev)
+    rope = torch.empty((T, HD // 2, 2), dtype=torch.float32, device=dev)
+    torch.cuda.synchronize()
+    apklib.check(L.apk_rope_table(h, p(pos), p(inv), T, HD // 2, p(rope)))
+    sync()
+    an = pool(3 * T * H * b, lambda: dict(x=randn((T, H)), d=randn((T, H)), h=torch.empty((T, H), dtype=torch.float16, device=dev)))
+    qk = pool(T * (NQ + NKV) * HD * b, lambda: dict(q=randn((T, NQ * HD)), k=randn((T, NKV * HD))))
+    sw = pool(2 * T * FF * b, lambda: dict(gate=randn((T, FF)), up=randn((T, FF))))
+    torch.cuda.synchronize()
+
+    def op_addnorm(i, gamma=gamma1, rows=T):
+        s = an[i % len(an)]
+        apklib.check(L.apk_add_rmsnorm_rows(h, p(s["x"]), p(s["d"]), p(s["h"]), p(gamma), H, rows, EPS, F16))
+
+    def op_qkrope(i, rows=T):
+        s = qk[i % len(qk)]
+        apklib.check(L.apk_qknorm_rope_neox(h, p(s["q"]), p(s["k"]), p(qw), p(kw), p(rope), rows, NQ, NKV, HD, HD, EPS, F16))
+
+    def op_swiglu(i, rows=T):
+        s = sw[i % len(sw)]
+        apklib.check(L.apk_swiglu(h, p(s["gate"]), p(s["up"]), rows * FF, F16))
+
+    def layer(i):
+        op_addnorm(2 * i)
+        op_qkrope(i)
+        op_addnorm(2 * i + 1, gamma2)
+        op_swiglu(i)
+
+    # ------------------------------------------------------------ timed steps
+    for i in range(args.warmup):
+        layer(i)
+    sync()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ms = C.c_float()
+    apklib.check(L.apk_timer_begin(h))
+    for i in range(args.steps):
+        layer(i + args.warmup)
+    apklib.check(L.apk_timer_end(h, C.byref(ms)))
+    sync()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1000.0
+    ms_per_step = wall_ms / args.steps
+    us_layer_events = ms.value * 1000.0 / args.steps
+
+    # ---------------------------------------------- per-op timings, headline shape
+    reps = max(20, args.steps)
+    tag = f"qwen3-32b T={T} f16"
+    bytes_addnorm = 4 * T * H * b + 4 * H
+    bytes_qkrope = 2 * T * (NQ + NKV) * HD * b + T * (HD // 2) * 8 + 2 * HD * 4
+    bytes_swiglu = 3 * T * FF * b
+    record("add_rmsnorm", tag, timed(op_addnorm, reps), bytes_addnorm)
+    record("qknorm_rope_neox", tag, timed(op_qkrope, reps), bytes_qkrope)
+    dom = record("swiglu", tag, timed(op_swiglu, reps), bytes_swiglu)
+    cp_bytes = T * FF * b
+    record("copy (plain stream)", f"{cp_bytes >> 20} MiB -> {cp_bytes >> 20} MiB",
+           timed(lambda i: apklib.check(L.apk_copy(h, p(sw[i % len(sw)]["up"]), p(sw[i % len(sw)]["gate"]), cp_bytes)), reps), 2 * cp_bytes)
+
+    if args.shapes == "all":
+        # small-T shapes of the same model: launch-latency bound, reported as us/launch
+        for rows, label in ((1, "decode T=1"), (6, "verify T=6"), (64, "batched decode, 64 rows with own positions")):
+            sh = f"qwen3-32b {label} f16"
+            record("add_rmsnorm", sh, timed(lambda i: op_addnorm(i, rows=rows), 200), 4 * rows * H * b + 4 * H, note="launch-bound")
+            record("qknorm_rope_neox", sh, timed(lambda i: op_qkrope(i, rows=rows), 200),
+                   2 * rows * (NQ + NKV) * HD * b + rows * (HD // 2) * 8 + 2 * HD * 4, note="launch-bound")
+            record("swiglu", sh, timed(lambda i: op_swiglu(i, rows=rows), 200), 3 * rows * FF * b, note="launch-bound")
+        del an, qk, sw
+        other_shapes(args, L, h, apklib, synth, torch, gen, dev, randn, pool, p, timed, record, reps, m, qw, kw, rope)
+    sync()
+
+    faults = C.c_uint32()
+    apklib.check(L.apk_take_faults(h, C.byref(faults)))
+    stats = [C.c_uint64() for _ in range(4)]
+    L.apk_stats(h, *[C.byref(v) for v in stats])
+
+    # ------------------------------------------------------------ cpu baseline
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_baseline(np, T, H, NQ, NKV, HD, FF, EPS)
+
+    layer_bytes = 2 * bytes_addnorm + bytes_qkrope + bytes_swiglu
+    out = {
+        "metric": "us/layer, fused layer ops (2x add+RMSNorm, QK-norm+RoPE, SwiGLU), Qwen3-32B shape",
+        "value": round(us_layer_events, 3),
+        "unit": "us/layer",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 6),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": f"BASELINE configs[2]: Qwen3-32B fused layer ops, T={T} prefill rows, fp16 activations, "
+                               f"hidden {H}, {NQ}q/{NKV}kv heads x {HD}, ffn {FF}; every op rotates through >= 640 MB of "
+                               "distinct buffers so every launch streams from HBM",
+                   "launches_per_layer": 4, "rows": T},
+        "roofline": {"bound": "hbm", "kernel": "apk_swiglu_f16", "achieved": dom["GBps"], "peak": PEAK_GBS, "unit": "GB/s",
+                     "frac": round(dom["GBps"] / PEAK_GBS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH,
+                     "algorithmic_bytes_per_launch": dom["bytes"], "avg_launch_us": dom["us"]},
+        "layer_algorithmic_bytes": int(layer_bytes),
+        "layer_GBps": round(layer_bytes / us_layer_events / 1e3, 1),
+        "layer_frac_of_peak": round(layer_bytes / us_layer_events / 1e3 / PEAK_GBS, 4),
+        "cpu_baseline": cpu,
+        "per_op": per_op,
+        "device_faults": faults.value,
+        "stats": {"calls": stats[0].value, "dispatches": stats[1].value, "encode_ns": stats[2].value, "wait_ns": stats[3].value},
+    }
+    L.apk_shutdown(h)
+    print(json.dumps(out))
+
+
+def other_shapes(args, L, h, apklib, synth, torch, gen, dev, randn, pool, p, timed, record, reps, m, qw, kw, rope):
+    """Embedding gathers, the Qwen3-0.6B f32 shapes and the MoE layer ops."""
+    F16, F32 = apklib.F16, apklib.F32
+    H, HD, EPS, T = m["hidden"], m["head_dim"], m["eps"], args.rows
+    check = apklib.check
+
+    # embedding gather, Q4_K table [151936 x 5120] -> fp16 rows (config 2)
+    vocab = m["vocab"]
+    rb = L.apk_row_bytes(apklib.FMT_Q4K, H)
+    table = torch.randint(0, 256, (vocab, H // 256, 144), generator=gen, device=dev, dtype=torch.uint8)
+    dd = (torch.randn((vocab, H // 256, 2), generator=gen, device=dev).abs() * (0.02 / 63.0)).half()
+    table[:, :, 0:4] = dd.view(torch.uint8).reshape(vocab, H // 256, 4)
+    ids = torch.randint(0, vocab, (8, T), generator=gen, device=dev, dtype=torch.int32)
+    outs = pool(T * H * 2, lambda: torch.empty((T, H), dtype=torch.float16, device=dev))
+    torch.cuda.synchronize()
+    for rows in (1, 6, T):
+        us = timed(lambda i: check(L.apk_embed_rows(h, apklib.FMT_Q4K, p(table), vocab, H, p(ids[i % 8]), rows,
+                                                    p(outs[i % len(outs)]), F16)), 200 if rows < T else reps)
+        record("embed_rows Q4_K->f16", f"qwen3-32b T={rows}", us, rows * (rb + 4 + H * 2), note=None if rows == T else "launch-bound")
+    del table, outs
+
+    # Qwen3-0.6B shapes, f32 activations (configs 0 and 1)
+    m0 = synth.MODELS["qwen3-0.6b"]
+    H0, NQ0, NKV0, FF0, V0 = m0["hidden"], m0["n_q"], m0["n_kv"], m0["ffn"], m0["vocab"]
+    T0 = 512
+    f32 = torch.float32
+    an0 = pool(3 * T0 * H0 * 4, lambda: dict(x=randn((T0, H0), f32), d=randn((T0, H0), f32), h=torch.empty((T0, H0), dtype=f32, device=dev)))
+    qk0 = pool(T0 * (NQ0 + NKV0) * HD * 4, lambda: dict(q=randn((T0, NQ0 * HD), f32), k=randn((T0, NKV0 * HD), f32)))
+    sw0 = pool(2 * T0 * FF0 * 4, lambda: dict(gate=randn((T0, FF0), f32), up=randn((T0, FF0), f32)))
+    g0 = 1 + 0.05 * randn(H0, f32)
+    q8 = torch.randint(0, 256, (V0, H0 // 32, 34), generator=gen, device=dev, dtype=torch.uint8)
+    sc = (torch.randn((V0, H0 // 32, 1), generator=gen, device=dev).abs() * (0.02 / 127.0)).half()
+    q8[:, :, 0:2] = sc.view(torch.uint8).reshape(V0, H0 // 32, 2)
+    ids0 = torch.randint(0, V0, (8, T0), generator=gen, device=dev, dtype=torch.int32)
+    torch.cuda.synchronize()
+    for rows, label in ((1, "T=1"), (T0, f"T={T0}")):
+        note = "launch-bound" if rows == 1 else None
+        us = timed(lambda i: check(L.apk_embed_rows(h, apklib.FMT_Q8_0, p(q8), V0, H0, p(ids0[i % 8]), rows,
+                                                    p(an0[i % len(an0)]["d"]), F32)), 200)
+        record("embed_rows Q8_0->f32", f"qwen3-0.6b {label}", us, rows * (1088 + 4 + H0 * 4), note=note)
+        us = timed(lambda i: check(L.apk_add_rmsnorm_rows(h, p(an0[i % len(an0)]["x"]), p(an0[i % len(an0)]["d"]),
+                                                          p(an0[i % len(an0)]["h"]), p(g0), H0, rows, EPS, F32)), 200)
+        record("add_rmsnorm", f"qwen3-0.6b {label} f32", us, 4 * rows * H0 * 4 + 4 * H0, note=note)
+        us = timed(lambda i: check(L.apk_qknorm_rope_neox(h, p(qk0[i % len(qk0)]["q"]), p(qk0[i % len(qk0)]["k"]), p(qw), p(kw),
+                                                          p(rope), rows, NQ0, NKV0, HD, HD, EPS, F32)), 200)
+        record("qknorm_rope_neox", f"qwen3-0.6b {label} f32", us, 2 * rows * (NQ0 + NKV0) * HD * 4 + rows * (HD // 2) * 8 + 2 * HD * 4, note=note)
+        us = timed(lambda i: check(L.apk_swiglu(h, p(sw0[i % len(sw0)]["gate"]), p(sw0[i % len(sw0)]["up"]), rows * FF0, F32)), 200)
+        record("swiglu", f"qwen3-0.6b {label} f32", us, 3 * rows * FF0 * 4, note=note)
+    del q8, an0, qk0, sw0
+
+    # Qwen3-30B-A3B MoE layer ops, T=1024 tokens, f32 (config 4)
+    mm = synth.MODELS["qwen3-30b-a3b"]
+    TM, HM, NE, K, FM = 1024, mm["hidden"], mm["n_expert"], mm["top_k"], mm["moe_ffn"]
+    logits = [randn((TM, NE), f32) for _ in range(8)]
+    ga = pool(TM * HM * 4 + TM * K * HM * 4, lambda: dict(hs=randn((TM, HM), f32), xe=torch.empty((TM * K, HM), dtype=f32, device=dev)))
+    se = pool(2 * TM * K * FM * 4, lambda: dict(gate=randn((TM * K, FM), f32), up=randn((TM * K, FM), f32)))
+    i32 = torch.int32
+    ids_m = torch.empty((TM, K), dtype=i32, device=dev)
+    w_m = torch.empty((TM, K), dtype=f32, device=dev)
+    tbl = torch.zeros((NE, 3), dtype=i32, device=dev)
+    n_used = torch.zeros(1, dtype=i32, device=dev)
+    tok = torch.empty(TM * K, dtype=i32, device=dev)
+    tok_off = torch.empty(TM + 1, dtype=i32, device=dev)
+    hit_row = torch.empty(TM * K, dtype=i32, device=dev)
+    hit_w = torch.empty(TM * K, dtype=f32, device=dev)
+    torch.cuda.synchronize()
+    tagm = f"qwen3-30b-a3b T={TM} f32"
+    us = timed(lambda i: check(L.apk_route_topk(h, p(logits[i % 8]), None, TM, NE, K, 1, 1.0, 0, p(ids_m), p(w_m))), 200)
+    record("route_topk", tagm, us, TM * NE * 4 + TM * K * 8, note="launch-bound")
+    us = timed(lambda i: check(L.apk_moe_permute(h, p(ids_m), p(w_m), TM, K, NE, p(tbl), p(n_used), p(tok), p(tok_off),
+                                                 p(hit_row), p(hit_w))), 200)
+    record("moe_permute (tables)", tagm, us, TM * K * 8 + TM * K * 12 + TM * 4, note="launch-bound")
+    us = timed(lambda i: check(L.apk_gather_rows(h, p(ga[i % len(ga)]["hs"]), p(tok), TM, TM * K, HM, p(ga[i % len(ga)]["xe"]), F32)), reps)
+    record("gather_rows (permute)", tagm, us, TM * HM * 4 + TM * K * HM * 4 + TM * K * 4)
+    us = timed(lambda i: check(L.apk_swiglu(h, p(se[i % len(se)]["gate"]), p(se[i % len(se)]["up"]), TM * K * FM, F32)), reps)
+    record("swiglu", f"qwen3-30b-a3b [{TM * K}x{FM}] f32", us, 3 * TM * K * FM * 4)
+
+
+def cpu_baseline(np, T, H, NQ, NKV, HD, FF, EPS):
+    """The CPU oracle on the same layer chain (f32 activations: the reference's
+    CPU path has no other), whole T rows, a few repetitions (~10-20 s)."""
+    import oracle as ora
+
+    ora.build()
+    cores = os.cpu_count() or 1
+    g = np.random.default_rng(7)
+    x = g.standard_normal((T, H), dtype=np.float32)
+    d = g.standard_normal((T, H), dtype=np.float32)
+    hbuf = np.empty_like(x)
+    gamma = (1 + 0.05 * g.standard_normal(H)).astype(np.float32)
+    q = g.standard_normal((T, NQ * HD), dtype=np.float32)
+    k = g.standard_normal((T, NKV * HD), dtype=np.float32)
+    qw = (1 + 0.05 * g.standard_normal(HD)).astype(np.float32)
+    kw = (1 + 0.05 * g.standard_normal(HD)).astype(np.float32)
+    inv = ora.rope_inv_freq(HD, 1e6)
+    ropes = ora.rope_table(list(range(T)), inv)
+    gate = g.standard_normal((T, FF), dtype=np.float32)
+    up = g.standard_normal((T, FF), dtype=np.float32)
+
+    def layer():
+        ora.add_assign_par(x.reshape(-1), d.reshape(-1), cores)          # prefill.rs:246
+        ora.rmsnorm_rows_into(hbuf.reshape(-1), x.reshape(-1), gamma, EPS, threads=cores)  # prefill.rs:155
+        ora.qknorm_rope_rows(q, k, NQ, NKV, HD, qw, kw, ropes, EPS)      # attention.rs:131-165, serial
+        ora.add_assign_par(x.reshape(-1), d.reshape(-1), cores)
+        ora.rmsnorm_rows_into(hbuf.reshape(-1), x.reshape(-1), gamma, EPS, threads=cores)
+        ora.swiglu(gate.reshape(-1), up.reshape(-1))                     # moe.rs:126, serial
+
+    layer()  # warm-up
+    times = []
+    t_end = time.perf_counter() + 12.0
+    while len(times) < 5 or (time.perf_counter() < t_end and len(times) < 40):
+        gate[:] = up  # keep SwiGLU inputs in a sane range across repetitions
+        t0 = time.perf_counter()
+        layer()
+        times.append(time.perf_counter() - t0)
+    med = sorted(times)[len(times) // 2]
+    return {"value": round(med * 1e6, 1), "unit": "us/layer", "cores": cores, "kind": "port",
+            "sample": f"median of {len(times)} repetitions of the whole T={T} layer chain in f32 (the reference's CPU activations are f32); "
+                      "C restatement of the reference CPU path, not the reference binary; residual add and row norms "
+                      "pool-parallel, QK-norm+RoPE and SwiGLU serial, as the reference runs them"}
+
+
+if __name__ == "__main__":
+    main()

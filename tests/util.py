@@ -8,6 +8,8 @@ def rel_err_f32(got, want):
     measured against a thousandth of the tensor's scale instead of themselves."""
     got = np.asarray(got, np.float64).ravel()
     want = np.asarray(want, np.float64).ravel()
+    if got.size == 0:
+        return 0.0
     floor = 1e-3 * float(np.sqrt(np.mean(want * want))) + 1e-30
     return float(np.max(np.abs(got - want) / np.maximum(np.abs(want), floor))) if got.size else 0.0
 
