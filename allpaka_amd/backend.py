@@ -163,6 +163,19 @@ class Backend:
                                           n_q, n_kv, head_dim, rot, eps, _dt(q)))
         self.sync()
 
+    def layer_prologue(self, x, delta, h, gamma, q, k, q_norm, k_norm, rope_flat, n_q, n_kv, head_dim, eps):
+        """add_rmsnorm_rows(x, delta, h, gamma) and qknorm_rope_neox(q, k, ...) as one launch
+        (small decode batches; larger ones run as the two launches)."""
+        n = gamma.numel()
+        rows = x.numel() // n
+        assert x.numel() == rows * n and h.numel() >= rows * n and (delta is None or delta.numel() == x.numel())
+        assert q.numel() == rows * n_q * head_dim and k.numel() == rows * n_kv * head_dim
+        assert rope_flat.numel() == rows * head_dim and q.dtype == k.dtype == x.dtype
+        self._enter()
+        check(self.L.apk_layer_prologue(self.h, _ptr(x), _ptr(delta), _ptr(h), _ptr(gamma), n, _ptr(q), _ptr(k), _ptr(q_norm),
+                                        _ptr(k_norm), _ptr(rope_flat), rows, n_q, n_kv, head_dim, head_dim, eps, _dt(x)))
+        self.sync()
+
     def rope_neox_cached_from_array(self, x, table):
         """ops::rope_neox_cached_from_array (rope.rs:70) on one head."""
         assert x.numel() >= table.shape[0] * 2

@@ -67,6 +67,7 @@ std::vector<std::string> all_kernel_names() {
                                   "apk_moe_permute", "apk_gather_rows", "apk_copy"};
     for (const char* t : {"f32", "f16"}) {
         for (int c : kAddnormTiles) v.push_back(std::string("apk_add_rmsnorm_") + t + "_c" + std::to_string(c));
+        for (int hd : kQkHeadDims) v.push_back(std::string("apk_layer_prologue_") + t + "_hd" + std::to_string(hd));
         for (int hd : kQkHeadDims)
             for (int it : kQkIters)
                 v.push_back(std::string("apk_qknorm_rope_") + t + "_hd" + std::to_string(hd) + "_i" + std::to_string(it));
@@ -422,6 +423,41 @@ int apk_qknorm_rope_neox(apk_ctx* c, void* q, void* k, const float* qw, const fl
     int rows_i = (int)rows, nq_i = (int)n_q, nkv_i = (int)n_kv;
     void* args[] = {&q, &k, &qw, &kw, &rope, &rows_i, &nq_i, &nkv_i, &eps};
     return launch(c, which, (unsigned)grid, block, 0, args);
+}
+
+int apk_layer_prologue(apk_ctx* c, void* x, const void* delta, void* h, const float* gamma, size_t n, void* q, void* k,
+                       const float* qw, const float* kw, const float* rope, size_t rows, size_t n_q, size_t n_kv,
+                       size_t head_dim, size_t rot_dim, float eps, int dtype) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_layer_prologue: ctx is NULL");
+    const int es = elem_size(dtype);
+    bool fused = es != 0 && rows > 0 && n_q + n_kv > 0 && n > 0 && x && h && gamma && rope && (!n_q || q) && (!n_kv || k) &&
+                 (head_dim == 64 || head_dim == 128 || head_dim == 256) && rot_dim == head_dim;
+    size_t threads = 0;
+    if (fused) {
+        const size_t vec = 16 / es, nchunks = n / vec;
+        threads = (nchunks + 63) / 64 * 64;  // one 16-byte tile per lane
+        fused = n % vec == 0 && threads <= 1024 && rows * (threads / 64) <= 2048 && rows <= 0x7fffffffu &&
+                aligned16(x) && aligned16(h) && aligned16(gamma) && (!delta || aligned16(delta)) && (!q || aligned16(q)) &&
+                (!k || aligned16(k)) && aligned16(rope) && (!qw || aligned16(qw)) && (!kw || aligned16(kw)) &&
+                n_q <= 65535 && n_kv <= 65535;
+    }
+    if (!fused) {
+        // outside the single-launch shape (large batches are bandwidth-bound, not launch-bound):
+        // the same result as two launches; every check and decline is theirs
+        if (int rc = apk_add_rmsnorm_rows(c, x, delta, h, gamma, n, rows, eps, dtype)) return rc;
+        return apk_qknorm_rope_neox(c, q, k, qw, kw, rope, rows, n_q, n_kv, head_dim, rot_dim, eps, dtype);
+    }
+    CallScope s(c);
+    if (int rc = set_device(c)) return rc;
+    const size_t epl = 16 / es, lph = head_dim / 2 / epl, hpw = 64 / lph, hpr = n_q + n_kv;
+    const uint64_t qk_waves = (uint64_t)rows * ((hpr + hpw - 1) / hpw);
+    const uint64_t wpb = threads / 64;
+    const uint64_t grid = rows + (qk_waves + wpb - 1) / wpb;
+    if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_layer_prologue: too large");
+    const std::string which = std::string("apk_layer_prologue_") + (dtype == APK_F32 ? "f32" : "f16") + "_hd" + std::to_string(head_dim);
+    int n_i = (int)n, rows_i = (int)rows, nq_i = (int)n_q, nkv_i = (int)n_kv;
+    void* args[] = {&x, &delta, &h, &gamma, &n_i, &q, &k, &qw, &kw, &rope, &rows_i, &nq_i, &nkv_i, &eps};
+    return launch(c, which, (unsigned)grid, (unsigned)threads, 0, args);
 }
 
 int apk_rope_table(apk_ctx* c, const uint32_t* positions, const float* inv_freq, size_t rows, size_t half, float* table) {

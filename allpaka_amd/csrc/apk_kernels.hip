@@ -174,12 +174,12 @@ template <> struct stat<f16_t> {
 };
 
 template <typename T, int NCH, bool HAS_DELTA>
-DEV void add_rmsnorm_impl(T* x, const T* delta, T* h, const float* gamma, int n, float eps) {
+DEV void add_rmsnorm_impl(T* x, const T* delta, T* h, const float* gamma, int n, float eps, uint32_t vblock) {
     constexpr int VEC = io<T>::VEC;
     typedef typename stat<T>::acc_t acc_t;
     __shared__ acc_t part[16];
     const int nchunks = n / VEC;
-    const uint64_t row = blockIdx.x;
+    const uint64_t row = vblock;
     T* xr = x + row * (uint64_t)n;
     T* hr = h + row * (uint64_t)n;
     const T* dr = HAS_DELTA ? delta + row * (uint64_t)n : nullptr;
@@ -234,16 +234,16 @@ DEV void add_rmsnorm_impl(T* x, const T* delta, T* h, const float* gamma, int n,
     }
 }
 template <typename T, int NCH>
-DEV void add_rmsnorm_body(T* x, const T* delta, T* h, const float* gamma, int n, float eps) {
-    if (delta) add_rmsnorm_impl<T, NCH, true>(x, delta, h, gamma, n, eps);   // uniform for the launch
-    else add_rmsnorm_impl<T, NCH, false>(x, delta, h, gamma, n, eps);
+DEV void add_rmsnorm_body(T* x, const T* delta, T* h, const float* gamma, int n, float eps, uint32_t vblock) {
+    if (delta) add_rmsnorm_impl<T, NCH, true>(x, delta, h, gamma, n, eps, vblock);   // uniform for the launch
+    else add_rmsnorm_impl<T, NCH, false>(x, delta, h, gamma, n, eps, vblock);
 }
 // The launch bound is the largest workgroup the host uses with that tile count
 // (it also caps the registers the compiler may take: 512 / (bound/64/4) per lane).
 #define APK_ADDNORM(T, TN, NCH, MAXT)                                                                        \
     extern "C" __global__ __launch_bounds__(MAXT) void apk_add_rmsnorm_##TN##_c##NCH(                        \
         T* x, const T* delta, T* h, const float* gamma, int n, float eps) {                                  \
-        add_rmsnorm_body<T, NCH>(x, delta, h, gamma, n, eps);                                                \
+        add_rmsnorm_body<T, NCH>(x, delta, h, gamma, n, eps, blockIdx.x);                                    \
     }
 #define APK_ADDNORM_ALL(T, TN)                                                                                   \
     APK_ADDNORM(T, TN, 1, 1024) APK_ADDNORM(T, TN, 2, 1024) APK_ADDNORM(T, TN, 3, 512) APK_ADDNORM(T, TN, 4, 512) \
@@ -269,7 +269,7 @@ APK_ADDNORM_ALL(f16_t, f16)
 // =========================================================================
 template <typename T, int HD, int ITER>
 DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv,
-                          float eps) {
+                          float eps, uint32_t vblock) {
     constexpr int EPL = io<T>::VEC;       // elements per lane per half
     constexpr int HALF = HD / 2;
     constexpr int LPH = HALF / EPL;       // lanes per head
@@ -279,7 +279,7 @@ DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const fl
     const int l = lane % LPH, sub = lane / LPH;
     const int hpr = n_q + n_kv;
     const int groups = (hpr + HPW * ITER - 1) / (HPW * ITER);
-    const uint64_t wid = ((uint64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const uint64_t wid = ((uint64_t)vblock * blockDim.x + threadIdx.x) >> 6;
     if (wid >= (uint64_t)rows * groups) return;  // whole wave
     const uint64_t row = wid / groups;
     const int g = (int)(wid % groups);
@@ -353,7 +353,7 @@ DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const fl
 #define APK_QKROPE(T, TN, HD, ITER)                                                                          \
     extern "C" __global__ __launch_bounds__(256) void apk_qknorm_rope_##TN##_hd##HD##_i##ITER(              \
         T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv, float eps) { \
-        qknorm_rope_body<T, HD, ITER>(q, k, qw, kw, rope, rows, n_q, n_kv, eps);                              \
+        qknorm_rope_body<T, HD, ITER>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, blockIdx.x);                  \
     }
 #define APK_QKROPE_ALL(T, TN)                                                                           \
     APK_QKROPE(T, TN, 64, 1) APK_QKROPE(T, TN, 64, 3) APK_QKROPE(T, TN, 64, 9)                          \
@@ -361,6 +361,22 @@ DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const fl
     APK_QKROPE(T, TN, 256, 1) APK_QKROPE(T, TN, 256, 3) APK_QKROPE(T, TN, 256, 9)
 APK_QKROPE_ALL(float, f32)
 APK_QKROPE_ALL(f16_t, f16)
+
+// Layer prologue for small decode batches: the residual add + RMSNorm of the hidden
+// rows and the QK-norm + RoPE of the q/k rows as ONE launch.  They are two independent
+// jobs sharing a grid (workgroups [0, rows) normalise one hidden row each, the rest
+// own 8-head groups of q/k); in a layer a QKV projection sits between them, so this
+// removes a launch, not a pass over memory.  One tile per lane (NCH = 1), one pass per
+// wave (ITER = 1): the shapes where launch latency, not bandwidth, is the cost.
+#define APK_PROLOGUE(T, TN, HD)                                                                                   \
+    extern "C" __global__ __launch_bounds__(1024) void apk_layer_prologue_##TN##_hd##HD(                         \
+        T* x, const T* delta, T* h, const float* gamma, int n, T* q, T* k, const float* qw, const float* kw,     \
+        const float* rope, int rows, int n_q, int n_kv, float eps) {                                             \
+        if (blockIdx.x < (uint32_t)rows) add_rmsnorm_body<T, 1>(x, delta, h, gamma, n, eps, blockIdx.x);         \
+        else qknorm_rope_body<T, HD, 1>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, blockIdx.x - (uint32_t)rows);  \
+    }
+APK_PROLOGUE(float, f32, 64) APK_PROLOGUE(float, f32, 128) APK_PROLOGUE(float, f32, 256)
+APK_PROLOGUE(f16_t, f16, 64) APK_PROLOGUE(f16_t, f16, 128) APK_PROLOGUE(f16_t, f16, 256)
 
 // RoPE table rows from per-row positions (rope.rs:18-22, session.rs:34-50):
 // table[r][i] = [sin, cos]((pos[r] as f32) * inv_freq[i]).  One f32 rounding of

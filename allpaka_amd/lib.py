@@ -36,6 +36,7 @@ SYMBOLS = {
     "apk_embed_rows_host_ids": (_i, [_vp, _i, _vp, _sz, _sz, _vp, _sz, _vp, _i]),
     "apk_add_rmsnorm_rows": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _f, _i]),
     "apk_qknorm_rope_neox": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _f, _i]),
+    "apk_layer_prologue": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _f, _i]),
     "apk_rope_table": (_i, [_vp, _vp, _vp, _sz, _sz, _vp]),
     "apk_swiglu": (_i, [_vp, _vp, _vp, _sz, _i]),
     "apk_route_topk": (_i, [_vp, _vp, _vp, _sz, _sz, _sz, _i, _f, _i, _vp, _vp]),

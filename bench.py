@@ -173,6 +173,11 @@ def main():
             record("qknorm_rope_neox", sh, timed(lambda i: op_qkrope(i, rows=rows), 200),
                    2 * rows * (NQ + NKV) * HD * b + rows * (HD // 2) * 8 + 2 * HD * 4, note="launch-bound")
             record("swiglu", sh, timed(lambda i: op_swiglu(i, rows=rows), 200), 3 * rows * FF * b, note="launch-bound")
+            us = timed(lambda i: apklib.check(L.apk_layer_prologue(
+                h, p(an[i % len(an)]["x"]), p(an[i % len(an)]["d"]), p(an[i % len(an)]["h"]), p(gamma1), H,
+                p(qk[i % len(qk)]["q"]), p(qk[i % len(qk)]["k"]), p(qw), p(kw), p(rope), rows, NQ, NKV, HD, HD, EPS, F16)), 200)
+            record("layer_prologue (add_rmsnorm || qknorm_rope, one launch)", sh, us,
+                   4 * rows * H * b + 4 * H + 2 * rows * (NQ + NKV) * HD * b + rows * (HD // 2) * 8 + 2 * HD * 4, note="launch-bound")
         del an, qk, sw
         other_shapes(args, L, h, apklib, synth, torch, gen, dev, randn, pool, p, timed, record, reps, m, qw, kw, rope)
     sync()

@@ -150,6 +150,18 @@ int apk_qknorm_rope_neox(apk_ctx* ctx, void* q, void* k, const float* qw, const 
                          size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim, float eps,
                          int dtype);
 
+/* Layer prologue as ONE launch: apk_add_rmsnorm_rows(x, delta, h, gamma, n, rows) and
+ * apk_qknorm_rope_neox(q, k, qw, kw, rope, rows, ...) with the same arguments and the
+ * same results, as two independent jobs in one grid (the reference's accelerators fuse
+ * the same pair of ops into their per-token command buffer, e.g. residual_norm + qk_prep,
+ * crates/allpaka-backend/src/gpu/metal/decode.rs:670; here q/k are inputs, a QKV
+ * projection sits between the two in a real layer).  Single launch when a row is at most
+ * 1024 16-byte tiles and rows * ceil(tiles/64) <= 2048 (decode and batched-decode
+ * shapes); otherwise it runs the two launches itself. */
+int apk_layer_prologue(apk_ctx* ctx, void* x, const void* delta, void* h, const float* gamma, size_t n, void* q,
+                       void* k, const float* qw, const float* kw, const float* rope, size_t rows, size_t n_q,
+                       size_t n_kv, size_t head_dim, size_t rot_dim, float eps, int dtype);
+
 /* Builds RoPE table rows on the device: table[r][i] = [sin, cos](pos[r] as f32 *
  * inv_freq[i]).  Replaces ops::rope_sin_cos per position (ops/rope.rs:18-22;
  * Session::ensure_rope_cache, model/session.rs:34-50; gpu::multi_stage's staging

@@ -268,6 +268,39 @@ def test_rope_table_on_device(be, ora):
     assert f16_ulp_diff(host(tq), wq) <= TOL_F16_ULP and f16_ulp_diff(host(tk), wk) <= TOL_F16_ULP
 
 
+# ------------------------------------------- single-launch layer prologue
+@pytest.mark.parametrize("rows,n,n_q,n_kv,hd,f16", [
+    (64, 5120, 64, 8, 128, True), (1, 5120, 64, 8, 128, True), (6, 5120, 64, 8, 128, True),
+    (1, 1024, 16, 8, 128, False), (8, 2048, 4, 4, 64, False), (3, 1024, 2, 1, 256, True),
+    (300, 5120, 64, 8, 128, True),  # beyond the single-launch shape: runs as two launches, same result
+])
+def test_layer_prologue_matches_the_two_ops(be, ora, rows, n, n_q, n_kv, hd, f16):
+    """Continuous-batching decode: every row has its own position; residual add + RMSNorm and
+    QK-norm + RoPE go out as one launch and must equal the two reference ops."""
+    s = synth()
+    g = s.rng(3, rows * 7 + n)
+    positions = [int(p) for p in g.integers(0, 32768, size=rows)]
+    q, k, qw, kw, inv, ropes = _qk_case(ora, 3, rows, n_q, n_kv, hd, f16, positions)
+    x, d = s.normal_f32(g, (rows, n)), s.normal_f32(g, (rows, n))
+    gamma = s.normal_f32(g, n, 1.0, 0.05)
+    if f16:
+        x, d = s.to_f16_bits(x), s.to_f16_bits(d)
+    wx, wh, wq, wk = x.copy(), np.zeros_like(x), q.copy(), k.copy()
+    ora.add_rmsnorm_rows(wx, d, wh, gamma, 1e-6)
+    ora.qknorm_rope_rows(wq, wk, n_q, n_kv, hd, qw, kw, ropes, 1e-6)
+    tx, th, tq, tk = dev(x), torch.zeros_like(dev(x)), dev(q), dev(k)
+    _, d0, _, _ = be.stats()
+    be.layer_prologue(tx, dev(d), th, dev(gamma), tq, tk, dev(qw), dev(kw), dev(ropes), n_q, n_kv, hd, 1e-6)
+    _, d1, _, _ = be.stats()
+    assert d1 - d0 == (1 if rows <= 64 else 2)  # one dispatch for decode batches
+    assert np.array_equal(host(tx), wx)
+    for got, want in ((host(th), wh), (host(tq), wq), (host(tk), wk)):
+        if f16:
+            assert f16_ulp_diff(got, want) <= TOL_F16_ULP
+        else:
+            assert rel_err_f32(got, want) <= TOL_F32 and close_idiom(got, want)
+
+
 # --------------------------------------------------------------------- SwiGLU
 @pytest.mark.parametrize("n", [3072, 512 * 3072, 6 * 25600, 64 * 25600, 1, 5, 1031, 8192 * 768 // 16])
 @pytest.mark.parametrize("f16", [False, True])
