@@ -58,7 +58,7 @@ struct Mapping {
 // missing symbol fails there and not at the first launch.
 const int kAddnormTiles[] = {1, 2, 3, 4, 5, 6, 8, 10, 12, 16, 20};  // 16-byte tiles per lane
 const int kAddnormBound[] = {1024, 1024, 512, 512, 256, 256, 256, 256, 256, 256, 256};  // launch bound of each
-const int kQkIters[] = {1, 3, 9};
+const int kQkIters[] = {1, 2, 4, 8};
 const int kQkHeadDims[] = {64, 128, 256};
 
 std::vector<std::string> all_kernel_names() {
@@ -403,18 +403,20 @@ int apk_qknorm_rope_neox(apk_ctx* c, void* q, void* k, const float* qw, const fl
     if ((q && !aligned16(q)) || (k && !aligned16(k)) || !aligned16(rope) || (qw && !aligned16(qw)) || (kw && !aligned16(kw)))
         return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_neox: tensors must be 16-byte aligned");
     if (rows > 0x7fffffffu || n_q > 65535 || n_kv > 65535) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_neox: too large");
-    // A wave owns (row, group of HPW*ITER heads); HPW = heads per wave pass.  The largest
-    // ITER that still leaves >= 1536 waves (6 per CU) amortises the row's [sin, cos] tile
-    // and the norm weights over the most heads; small batches take ITER = 1.
-    const size_t epl = 16 / es, lph = head_dim / 2 / epl, hpw = 64 / lph, hpr = n_q + n_kv;
+    // A wave owns (row, q or k, group of HPW*ITER heads), HPW = heads per wave pass; k waves
+    // take one pass.  The largest ITER for q that still leaves >= 1536 waves (6 per CU)
+    // amortises the row's [sin, cos] tile and the norm weight over the most heads; small
+    // batches take ITER = 1.
+    const size_t epl = 16 / es, lph = head_dim / 2 / epl, hpw = 64 / lph;
+    const size_t gk = (n_kv + hpw - 1) / hpw;
     int iter = 1;
-    for (int cand : {9, 3}) {
-        if ((size_t)cand > (hpr + hpw - 1) / hpw) continue;
-        const size_t groups = (hpr + hpw * cand - 1) / (hpw * cand);
-        if (rows * groups >= 1536) { iter = cand; break; }
+    for (int cand : {8, 4, 2}) {
+        if ((size_t)cand > (n_q + hpw - 1) / hpw) continue;
+        const size_t gq = (n_q + hpw * cand - 1) / (hpw * cand);
+        if (rows * (gq + gk) >= 1536) { iter = cand; break; }
     }
-    const uint64_t waves = (uint64_t)rows * ((hpr + hpw * iter - 1) / (hpw * iter));
-    const unsigned block = iter == 9 ? 64 : 256;
+    const uint64_t waves = (uint64_t)rows * ((n_q + hpw * iter - 1) / (hpw * iter) + gk);
+    const unsigned block = iter >= 4 ? 64 : 256;
     const uint64_t grid = (waves * 64 + block - 1) / block;
     if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_neox: too large");
     const std::string which = std::string("apk_qknorm_rope_") + (dtype == APK_F32 ? "f32" : "f16") + "_hd" +
@@ -449,8 +451,8 @@ int apk_layer_prologue(apk_ctx* c, void* x, const void* delta, void* h, const fl
     }
     CallScope s(c);
     if (int rc = set_device(c)) return rc;
-    const size_t epl = 16 / es, lph = head_dim / 2 / epl, hpw = 64 / lph, hpr = n_q + n_kv;
-    const uint64_t qk_waves = (uint64_t)rows * ((hpr + hpw - 1) / hpw);
+    const size_t epl = 16 / es, lph = head_dim / 2 / epl, hpw = 64 / lph;
+    const uint64_t qk_waves = (uint64_t)rows * ((n_q + hpw - 1) / hpw + (n_kv + hpw - 1) / hpw);
     const uint64_t wpb = threads / 64;
     const uint64_t grid = rows + (qk_waves + wpb - 1) / wpb;
     if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_layer_prologue: too large");
