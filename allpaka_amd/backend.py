@@ -235,6 +235,16 @@ class Backend:
         self.sync()
         return dst
 
+    def scatter_rows(self, src, hit_row, k):
+        """The same xe rows from the token side: xe[hit_row[t*k+j]] = src[t] (each row read once)."""
+        rows = src.shape[0]
+        total = rows * k
+        dst = torch.empty((total, src.shape[1]), dtype=src.dtype, device=self.device)
+        self._enter()
+        check(self.L.apk_scatter_rows(self.h, _ptr(src), _ptr(hit_row), rows, k, total, src.shape[1], _ptr(dst), _dt(src)))
+        self.sync()
+        return dst
+
 
 class QuantMat:
     """QuantMat::{new,row,row_into} (quantmat/mod.rs:39-89) over a device-resident table."""
@@ -275,3 +285,4 @@ class QuantMat:
         self.b.sync()
         if self.b.take_faults() & _l.FAULT_TOKEN_RANGE:
             raise ValueError("token id out of vocab")
+

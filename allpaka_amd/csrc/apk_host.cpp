@@ -64,7 +64,7 @@ const int kQkHeadDims[] = {64, 128, 256};
 std::vector<std::string> all_kernel_names() {
     std::vector<std::string> v = {"apk_swiglu_f32", "apk_swiglu_f16", "apk_rope_table", "apk_embed_q4k_f32",
                                   "apk_embed_q4k_f16", "apk_embed_q8_0_f32", "apk_embed_q8_0_f16", "apk_route_topk",
-                                  "apk_moe_permute", "apk_gather_rows", "apk_copy"};
+                                  "apk_moe_permute", "apk_gather_rows", "apk_scatter_rows", "apk_copy"};
     for (const char* t : {"f32", "f16"}) {
         for (int c : kAddnormTiles) v.push_back(std::string("apk_add_rmsnorm_") + t + "_c" + std::to_string(c));
         for (int hd : kQkHeadDims) v.push_back(std::string("apk_layer_prologue_") + t + "_hd" + std::to_string(hd));
@@ -594,6 +594,25 @@ int apk_gather_rows(apk_ctx* c, const void* src, const uint32_t* tok, size_t src
     int row_vecs = (int)(cols * es / 16);
     void* args[] = {&src, &tok, &src_rows32, &row_vecs, &dst, &c->fault_dev};
     return launch(c, "apk_gather_rows", (unsigned)total_rows, 256, 0, args);
+}
+
+int apk_scatter_rows(apk_ctx* c, const void* src, const uint32_t* hit_row, size_t rows, size_t k, size_t total_rows,
+                     size_t cols, void* dst, int dtype) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_scatter_rows: ctx is NULL");
+    CallScope s(c);
+    const int es = elem_size(dtype);
+    if (!es) return fail(APK_DECLINE_UNSUPPORTED, "apk_scatter_rows: dtype %d", dtype);
+    if (rows == 0 || k == 0 || cols == 0) return APK_OK;
+    if (!src || !hit_row || !dst) return fail(APK_DECLINE_NULL, "apk_scatter_rows: NULL tensor");
+    if ((cols * es) % 16 || !aligned16(src) || !aligned16(dst))
+        return fail(APK_DECLINE_SHAPE, "apk_scatter_rows: rows must be whole 16-byte tiles");
+    if (rows > 0x7fffffffu || total_rows > 0xffffffffu || k > 0x7fffffffu || cols * es / 16 > 0x7fffffffu)
+        return fail(APK_DECLINE_SHAPE, "apk_scatter_rows: too large");
+    if (int rc = set_device(c)) return rc;
+    int k_i = (int)k, row_vecs = (int)(cols * es / 16);
+    uint32_t total32 = (uint32_t)total_rows;
+    void* args[] = {&src, &hit_row, &k_i, &total32, &row_vecs, &dst, &c->fault_dev};
+    return launch(c, "apk_scatter_rows", (unsigned)rows, 256, 0, args);
 }
 
 int apk_copy(apk_ctx* c, const void* src, void* dst, size_t bytes) {

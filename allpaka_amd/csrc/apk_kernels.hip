@@ -803,6 +803,34 @@ extern "C" __global__ __launch_bounds__(256) void apk_gather_rows(const u32x4* s
     }
 }
 
+// The same permutation driven from the token side: dst[hit_row[t*k + j], :] = src[t, :]
+// for the k hits of token t (the CSR lists of apk_moe_permute).  Each source row is read
+// from HBM once and written k times; the gather form above re-reads it from every XCD's
+// own L2 (8 XCDs, 8 fills of the same row through the fabric).  One workgroup per token.
+extern "C" __global__ __launch_bounds__(256) void apk_scatter_rows(const u32x4* src, const uint32_t* hit_row, int k,
+                                                                  uint32_t total_rows, int row_vecs, u32x4* dst,
+                                                                  uint32_t* fault) {
+    const uint64_t t = blockIdx.x;
+    const u32x4* sp = src + t * row_vecs;
+    const uint32_t* hits = hit_row + t * k;
+    for (int c = threadIdx.x; c < row_vecs; c += 2 * blockDim.x) {
+        const int c2 = c + blockDim.x;
+        const bool two = c2 < row_vecs;
+        const u32x4 a = __builtin_nontemporal_load(sp + c);
+        const u32x4 b = __builtin_nontemporal_load(sp + (two ? c2 : c));
+        for (int j = 0; j < k; j++) {
+            const uint32_t r = hits[j];
+            if (r >= total_rows) {
+                if (c == 0) atomicOr(fault, APK_FAULT_ROW_RANGE);
+                continue;
+            }
+            u32x4* dp = dst + (uint64_t)r * row_vecs;
+            __builtin_nontemporal_store(a, dp + c);
+            if (two) __builtin_nontemporal_store(b, dp + c2);
+        }
+    }
+}
+
 // Reference stream for bandwidth calibration: dst = src, one 16-byte tile per lane.
 extern "C" __global__ __launch_bounds__(256) void apk_copy(const u32x4* src, u32x4* dst, uint64_t nvec) {
     const uint64_t c = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;

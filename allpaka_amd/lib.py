@@ -42,6 +42,7 @@ SYMBOLS = {
     "apk_route_topk": (_i, [_vp, _vp, _vp, _sz, _sz, _sz, _i, _f, _i, _vp, _vp]),
     "apk_moe_permute": (_i, [_vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp]),
     "apk_gather_rows": (_i, [_vp, _vp, _vp, _sz, _sz, _sz, _vp, _i]),
+    "apk_scatter_rows": (_i, [_vp, _vp, _vp, _sz, _sz, _sz, _sz, _vp, _i]),
     "apk_copy": (_i, [_vp, _vp, _vp, _sz]),
 }
 

@@ -298,7 +298,9 @@ def other_shapes(args, L, h, apklib, synth, torch, gen, dev, randn, pool, p, tim
                                                  p(hit_row), p(hit_w))), 200)
     record("moe_permute (tables)", tagm, us, TM * K * 8 + TM * K * 12 + TM * 4, note="launch-bound")
     us = timed(lambda i: check(L.apk_gather_rows(h, p(ga[i % len(ga)]["hs"]), p(tok), TM, TM * K, HM, p(ga[i % len(ga)]["xe"]), F32)), reps)
-    record("gather_rows (permute)", tagm, us, TM * HM * 4 + TM * K * HM * 4 + TM * K * 4)
+    record("gather_rows (permute, row-side)", tagm, us, TM * HM * 4 + TM * K * HM * 4 + TM * K * 4)
+    us = timed(lambda i: check(L.apk_scatter_rows(h, p(ga[i % len(ga)]["hs"]), p(hit_row), TM, K, TM * K, HM, p(ga[i % len(ga)]["xe"]), F32)), reps)
+    record("scatter_rows (permute, token-side)", tagm, us, TM * HM * 4 + TM * K * HM * 4 + TM * K * 4)
     us = timed(lambda i: check(L.apk_swiglu(h, p(se[i % len(se)]["gate"]), p(se[i % len(se)]["up"]), TM * K * FM, F32)), reps)
     record("swiglu", f"qwen3-30b-a3b [{TM * K}x{FM}] f32", us, 3 * TM * K * FM * 4)
 

@@ -200,6 +200,15 @@ int apk_moe_permute(apk_ctx* ctx, const uint32_t* ids, const float* w, size_t ro
 int apk_gather_rows(apk_ctx* ctx, const void* src, const uint32_t* tok, size_t src_rows, size_t total_rows,
                     size_t cols, void* dst, int dtype);
 
+/* The same expert-grouped rows produced from the token side with the CSR lists of
+ * apk_moe_permute: dst[hit_row[t*k + j], :] = src[t, :] for j < k.  Equal to
+ * apk_gather_rows(src, tok, ...) when (tok, hit_row) come from one apk_moe_permute call
+ * (model/moe.rs:298-309 builds hit_row as the inverse of tok), and the faster form:
+ * each source row is read once.  A hit >= total_rows is skipped and raises
+ * APK_FAULT_ROW_RANGE. */
+int apk_scatter_rows(apk_ctx* ctx, const void* src, const uint32_t* hit_row, size_t rows, size_t k, size_t total_rows,
+                     size_t cols, void* dst, int dtype);
+
 /* dst = src, `bytes` a multiple of 16: the plain stream kernel the bandwidth
  * figures of the other kernels are calibrated against. */
 int apk_copy(apk_ctx* ctx, const void* src, void* dst, size_t bytes);

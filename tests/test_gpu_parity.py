@@ -414,6 +414,8 @@ def test_moe_permute_and_gather_bit_exact(be, ora, rows, k, n_expert):
             hs = s.to_f16_bits(hs)
         xe = be.gather_rows(dev(hs), got[1])
         assert np.array_equal(host(xe), ora.gather_rows(hs, want[1]))
+        xs = be.scatter_rows(dev(hs), got[3], k)  # token-side form of the same permutation
+        assert torch.equal(xs, xe)
 
 
 def test_permute_declines_and_faults(be):
@@ -430,6 +432,8 @@ def test_permute_declines_and_faults(be):
     assert be.take_faults() & 4 and np.all(host(out)[0] == 1.0)
     with pytest.raises(apk.Declined):
         be.gather_rows(torch.ones((2, 3), device="cuda"), torch.tensor([0], dtype=torch.int32, device="cuda"))
+    out = be.scatter_rows(src, torch.tensor([1, 9, 0, 3], dtype=torch.int32, device="cuda"), 2)
+    assert be.take_faults() & 4 and np.all(host(out)[[0, 1, 3]] == 1.0)
 
 
 # ----------------------------------------------- full-size property checks
