@@ -69,8 +69,10 @@ std::vector<std::string> all_kernel_names() {
         for (int c : kAddnormTiles) v.push_back(std::string("apk_add_rmsnorm_") + t + "_c" + std::to_string(c));
         for (int hd : kQkHeadDims) v.push_back(std::string("apk_layer_prologue_") + t + "_hd" + std::to_string(hd));
         for (int hd : kQkHeadDims)
-            for (int it : kQkIters)
+            for (int it : kQkIters) {
                 v.push_back(std::string("apk_qknorm_rope_") + t + "_hd" + std::to_string(hd) + "_i" + std::to_string(it));
+                v.push_back(std::string("apk_qknorm_rope_kv_") + t + "_hd" + std::to_string(hd) + "_i" + std::to_string(it));
+            }
     }
     return v;
 }
@@ -388,10 +390,17 @@ int apk_add_rmsnorm_rows(apk_ctx* c, void* x, const void* delta, void* h, const 
     return launch(c, which, (unsigned)rows, (unsigned)threads, 0, args);
 }
 
-int apk_qknorm_rope_neox(apk_ctx* c, void* q, void* k, const float* qw, const float* kw, const float* rope,
-                         size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim, float eps, int dtype) {
-    if (!c) return fail(APK_DECLINE_NULL, "apk_qknorm_rope_neox: ctx is NULL");
-    CallScope s(c);
+struct KvStore {  // the fused K/V cache store of apk_qknorm_rope_kv_store (all NULL/0: plain op)
+    const void* v = nullptr;
+    const uint32_t* cache_pos = nullptr;
+    void* k_cache = nullptr;
+    void* v_cache = nullptr;
+    size_t capacity = 0;
+};
+
+static int qknorm_rope_common(apk_ctx* c, void* q, void* k, const float* qw, const float* kw, const float* rope, size_t rows,
+                              size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim, float eps, int dtype,
+                              const KvStore* kv) {
     const int es = elem_size(dtype);
     if (!es) return fail(APK_DECLINE_UNSUPPORTED, "apk_qknorm_rope_neox: dtype %d", dtype);
     if (head_dim != 64 && head_dim != 128 && head_dim != 256)
@@ -402,6 +411,13 @@ int apk_qknorm_rope_neox(apk_ctx* c, void* q, void* k, const float* qw, const fl
     if ((n_q && !q) || (n_kv && !k) || !rope) return fail(APK_DECLINE_NULL, "apk_qknorm_rope_neox: NULL tensor");
     if ((q && !aligned16(q)) || (k && !aligned16(k)) || !aligned16(rope) || (qw && !aligned16(qw)) || (kw && !aligned16(kw)))
         return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_neox: tensors must be 16-byte aligned");
+    if (kv) {
+        if (n_kv == 0) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_kv_store: no k heads");
+        if (!kv->v || !kv->cache_pos || !kv->k_cache || !kv->v_cache) return fail(APK_DECLINE_NULL, "apk_qknorm_rope_kv_store: NULL tensor");
+        if (!aligned16(kv->v) || !aligned16(kv->k_cache) || !aligned16(kv->v_cache))
+            return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_kv_store: tensors must be 16-byte aligned");
+        if (kv->capacity == 0 || kv->capacity > 0xffffffffu) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_kv_store: capacity");
+    }
     if (rows > 0x7fffffffu || n_q > 65535 || n_kv > 65535) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_neox: too large");
     // A wave owns (row, q or k, group of HPW*ITER heads), HPW = heads per wave pass; k waves
     // take one pass.  The largest ITER for q that still leaves >= 1536 waves (6 per CU)
@@ -419,12 +435,35 @@ int apk_qknorm_rope_neox(apk_ctx* c, void* q, void* k, const float* qw, const fl
     const unsigned block = iter >= 4 ? 64 : 256;
     const uint64_t grid = (waves * 64 + block - 1) / block;
     if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_neox: too large");
-    const std::string which = std::string("apk_qknorm_rope_") + (dtype == APK_F32 ? "f32" : "f16") + "_hd" +
-                              std::to_string(head_dim) + "_i" + std::to_string(iter);
+    const std::string which = std::string(kv ? "apk_qknorm_rope_kv_" : "apk_qknorm_rope_") + (dtype == APK_F32 ? "f32" : "f16") +
+                              "_hd" + std::to_string(head_dim) + "_i" + std::to_string(iter);
     if (int rc = set_device(c)) return rc;
     int rows_i = (int)rows, nq_i = (int)n_q, nkv_i = (int)n_kv;
+    if (kv) {
+        uint32_t cap32 = (uint32_t)kv->capacity;
+        void* kargs[] = {&q, &k, (void*)&kv->v, &qw, &kw, &rope, (void*)&kv->cache_pos, (void*)&kv->k_cache, (void*)&kv->v_cache,
+                         &cap32, &rows_i, &nq_i, &nkv_i, &eps, &c->fault_dev};
+        return launch(c, which, (unsigned)grid, block, 0, kargs);
+    }
     void* args[] = {&q, &k, &qw, &kw, &rope, &rows_i, &nq_i, &nkv_i, &eps};
     return launch(c, which, (unsigned)grid, block, 0, args);
+}
+
+int apk_qknorm_rope_neox(apk_ctx* c, void* q, void* k, const float* qw, const float* kw, const float* rope,
+                         size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim, float eps, int dtype) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_qknorm_rope_neox: ctx is NULL");
+    CallScope s(c);
+    return qknorm_rope_common(c, q, k, qw, kw, rope, rows, n_q, n_kv, head_dim, rot_dim, eps, dtype, nullptr);
+}
+
+int apk_qknorm_rope_kv_store(apk_ctx* c, void* q, void* k, const void* v, const float* qw, const float* kw,
+                             const float* rope, const uint32_t* cache_pos, void* k_cache, void* v_cache, size_t capacity,
+                             size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim, float eps, int dtype) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_qknorm_rope_kv_store: ctx is NULL");
+    CallScope s(c);
+    KvStore kv;
+    kv.v = v; kv.cache_pos = cache_pos; kv.k_cache = k_cache; kv.v_cache = v_cache; kv.capacity = capacity;
+    return qknorm_rope_common(c, q, k, qw, kw, rope, rows, n_q, n_kv, head_dim, rot_dim, eps, dtype, &kv);
 }
 
 int apk_layer_prologue(apk_ctx* c, void* x, const void* delta, void* h, const float* gamma, size_t n, void* q, void* k,

@@ -29,6 +29,7 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 #define APK_FAULT_TOKEN_RANGE 1u   // embedding id >= vocab
 #define APK_FAULT_EXPERT_RANGE 2u  // routed expert id >= n_expert
 #define APK_FAULT_ROW_RANGE 4u     // gather index >= source rows
+#define APK_FAULT_CACHE_RANGE 8u   // KV-cache position >= capacity
 
 DEV float h2f(uint32_t bits16) { return (float)__builtin_bit_cast(f16_t, (uint16_t)bits16); }
 
@@ -84,6 +85,17 @@ template <> struct io<f16_t> {
     DEV void store(f16_t* p, const float* v) { *(u32x4*)p = pack(v); }
     DEV void store_nt(f16_t* p, const float* v) { __builtin_nontemporal_store(pack(v), (u32x4*)p); }
 };
+
+// One tile of activations narrowed to fp16 (RNE) for the KV cache: 16 bytes from an
+// fp16 tile, 8 bytes from an f32 tile.
+template <typename T> DEV void store_f16_tile(f16_t* p, const float* v);
+template <> __device__ __forceinline__ void store_f16_tile<f16_t>(f16_t* p, const float* v) { io<f16_t>::store_nt(p, v); }
+template <> __device__ __forceinline__ void store_f16_tile<float>(f16_t* p, const float* v) {
+    f32x2 lo = {v[0], v[1]}, hi = {v[2], v[3]};
+    u32x2 t = {__builtin_bit_cast(uint32_t, __builtin_convertvector(lo, f16x2)),
+               __builtin_bit_cast(uint32_t, __builtin_convertvector(hi, f16x2))};
+    __builtin_nontemporal_store(t, (u32x2*)p);
+}
 
 DEV double wave_sum_f64(double v, int width) {
 #pragma unroll
@@ -276,8 +288,12 @@ APK_ADDNORM_ALL(f16_t, f16)
 // hardware rsq, and the norm weight folded into the rotation coefficients
 // (out_a = scale*(a*(wa*cos) - b*(wb*sin))): 3 instead of 5 multiplies/element.
 // =========================================================================
-template <typename T, int HD, int ITER>
-DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, float eps, int l, int sub) {
+// KV = true (k items only): the rotated k tiles are also narrowed to fp16 into the cache row
+// kc, and the same tiles of the row's v are narrowed into vc (KvCache::store_at,
+// crates/allpaka-model/src/kv.rs:682-697: k and v rows as f16 at pos*kv_dim).
+template <typename T, int HD, int ITER, bool KV = false>
+DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, float eps, int l, int sub,
+                 f16_t* kc = nullptr, const T* vrow = nullptr, f16_t* vc = nullptr) {
     constexpr int EPL = io<T>::VEC;   // elements per lane per half
     constexpr int HALF = HD / 2;
     constexpr int LPH = HALF / EPL;   // lanes per head
@@ -296,17 +312,23 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
         io<float>::load(wp + EPL * l + i, wa + i);
         io<float>::load(wp + HALF + EPL * l + i, wb + i);
     }
-    typename io<T>::raw_t araw[ITER], braw[ITER];
+    typename io<T>::raw_t araw[ITER], braw[ITER], varaw[ITER], vbraw[ITER];
     T* hp[ITER];
+    int hoff[ITER];
     bool live[ITER];
 #pragma unroll
     for (int it = 0; it < ITER; it++) {
         const int hh0 = (g * ITER + it) * HPW + sub;
         live[it] = hh0 < nheads;
-        hp[it] = base + (uint64_t)min(hh0, nheads - 1) * HD;
+        hoff[it] = min(hh0, nheads - 1) * HD;
+        hp[it] = base + hoff[it];
         __builtin_amdgcn_sched_barrier(0);  // loads stay in program order (returns are in order)
         araw[it] = io<T>::ldraw_nt(hp[it] + EPL * l);
         braw[it] = io<T>::ldraw_nt(hp[it] + HALF + EPL * l);
+        if constexpr (KV) {
+            varaw[it] = io<T>::ldraw_nt(vrow + hoff[it] + EPL * l);
+            vbraw[it] = io<T>::ldraw_nt(vrow + hoff[it] + HALF + EPL * l);
+        }
     }
     __builtin_amdgcn_sched_barrier(0);  // every load above; all uses below
     const bool normed = w != nullptr;  // uniform for the wave
@@ -357,13 +379,26 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
             io<T>::store_nt(hp[it] + EPL * l, oa);
             io<T>::store_nt(hp[it] + HALF + EPL * l, ob);
         }
+        if constexpr (KV) {
+            if (live[it] && kc != nullptr) {  // kc == nullptr: cache position out of range, row skipped
+                float va[EPL], vb[EPL];
+                io<T>::widen(varaw[it], va);
+                io<T>::widen(vbraw[it], vb);
+                store_f16_tile<T>(kc + hoff[it] + EPL * l, oa);
+                store_f16_tile<T>(kc + hoff[it] + HALF + EPL * l, ob);
+                store_f16_tile<T>(vc + hoff[it] + EPL * l, va);
+                store_f16_tile<T>(vc + hoff[it] + HALF + EPL * l, vb);
+            }
+        }
         __builtin_amdgcn_sched_barrier(0);  // pass by pass: pass it+1 waits only for its own tiles
     }
 }
 
-template <typename T, int HD, int ITERQ>
+template <typename T, int HD, int ITERQ, bool KV = false>
 DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv,
-                          float eps, uint32_t vblock) {
+                          float eps, uint32_t vblock, const T* v = nullptr, const uint32_t* cache_pos = nullptr,
+                          f16_t* k_cache = nullptr, f16_t* v_cache = nullptr, uint32_t capacity = 0,
+                          uint32_t* fault = nullptr) {
     constexpr int LPH = HD / 2 / io<T>::VEC, HPW = 64 / LPH;
     const int lane = threadIdx.x & 63;
     const int l = lane % LPH, sub = lane / LPH;
@@ -378,7 +413,17 @@ DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const fl
         qk_item<T, HD, ITERQ>(q + row * (uint64_t)n_q * HD, n_q, (int)(wid % gq), qw, rope + row * HD, eps, l, sub);
     } else {
         const uint64_t w2 = wid - nq_items, row = w2 / gk;
-        qk_item<T, HD, 1>(k + row * (uint64_t)n_kv * HD, n_kv, (int)(w2 % gk), kw, rope + row * HD, eps, l, sub);
+        const uint64_t kv_dim = (uint64_t)n_kv * HD;
+        if constexpr (KV) {
+            const uint32_t pos = cache_pos[row];
+            const bool ok = pos < capacity;
+            if (!ok && lane == 0 && w2 % gk == 0) atomicOr(fault, APK_FAULT_CACHE_RANGE);
+            qk_item<T, HD, 1, true>(k + row * kv_dim, n_kv, (int)(w2 % gk), kw, rope + row * HD, eps, l, sub,
+                                    ok ? k_cache + pos * kv_dim : nullptr, v + row * kv_dim,
+                                    ok ? v_cache + pos * kv_dim : nullptr);
+        } else {
+            qk_item<T, HD, 1>(k + row * kv_dim, n_kv, (int)(w2 % gk), kw, rope + row * HD, eps, l, sub);
+        }
     }
 }
 #define APK_QKROPE(T, TN, HD, ITER)                                                                          \
@@ -392,6 +437,22 @@ DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const fl
     APK_QKROPE(T, TN, 256, 1) APK_QKROPE(T, TN, 256, 2) APK_QKROPE(T, TN, 256, 4) APK_QKROPE(T, TN, 256, 8)
 APK_QKROPE_ALL(float, f32)
 APK_QKROPE_ALL(f16_t, f16)
+
+// The same with the K/V cache store fused in: rotated k and the row's v narrowed to fp16
+// at cache row cache_pos[row] (one launch instead of QK-norm+RoPE, then two narrowing copies).
+#define APK_QKROPE_KV(T, TN, HD, ITER)                                                                            \
+    extern "C" __global__ __launch_bounds__(256) void apk_qknorm_rope_kv_##TN##_hd##HD##_i##ITER(                \
+        T* q, T* k, const T* v, const float* qw, const float* kw, const float* rope, const uint32_t* cache_pos,  \
+        f16_t* k_cache, f16_t* v_cache, uint32_t capacity, int rows, int n_q, int n_kv, float eps, uint32_t* fault) { \
+        qknorm_rope_body<T, HD, ITER, true>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, blockIdx.x, v, cache_pos,   \
+                                            k_cache, v_cache, capacity, fault);                                   \
+    }
+#define APK_QKROPE_KV_ALL(T, TN)                                                                                       \
+    APK_QKROPE_KV(T, TN, 64, 1) APK_QKROPE_KV(T, TN, 64, 2) APK_QKROPE_KV(T, TN, 64, 4) APK_QKROPE_KV(T, TN, 64, 8)    \
+    APK_QKROPE_KV(T, TN, 128, 1) APK_QKROPE_KV(T, TN, 128, 2) APK_QKROPE_KV(T, TN, 128, 4) APK_QKROPE_KV(T, TN, 128, 8) \
+    APK_QKROPE_KV(T, TN, 256, 1) APK_QKROPE_KV(T, TN, 256, 2) APK_QKROPE_KV(T, TN, 256, 4) APK_QKROPE_KV(T, TN, 256, 8)
+APK_QKROPE_KV_ALL(float, f32)
+APK_QKROPE_KV_ALL(f16_t, f16)
 
 // Layer prologue for small decode batches: the residual add + RMSNorm of the hidden
 // rows and the QK-norm + RoPE of the q/k rows as ONE launch.  They are two independent

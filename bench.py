@@ -178,7 +178,15 @@ def main():
                 p(qk[i % len(qk)]["q"]), p(qk[i % len(qk)]["k"]), p(qw), p(kw), p(rope), rows, NQ, NKV, HD, HD, EPS, F16)), 200)
             record("layer_prologue (add_rmsnorm || qknorm_rope, one launch)", sh, us,
                    4 * rows * H * b + 4 * H + 2 * rows * (NQ + NKV) * HD * b + rows * (HD // 2) * 8 + 2 * HD * 4, note="launch-bound")
-        del an, qk, sw
+        # QK-norm + RoPE with the K/V cache store fused in (one launch; the cache planes of one layer, capacity T)
+        kvp = [dict(v=randn((T, NKV * HD)), kc=torch.empty((T, NKV * HD), dtype=torch.float16, device=dev),
+                    vc=torch.empty((T, NKV * HD), dtype=torch.float16, device=dev)) for _ in range(len(qk))]
+        torch.cuda.synchronize()
+        us = timed(lambda i: apklib.check(L.apk_qknorm_rope_kv_store(
+            h, p(qk[i % len(qk)]["q"]), p(qk[i % len(qk)]["k"]), p(kvp[i % len(qk)]["v"]), p(qw), p(kw), p(rope), p(pos),
+            p(kvp[i % len(qk)]["kc"]), p(kvp[i % len(qk)]["vc"]), T, T, NQ, NKV, HD, HD, EPS, F16)), reps)
+        record("qknorm_rope_neox + K/V cache store (one launch)", tag, us, bytes_qkrope + T * NKV * HD * b + 2 * T * NKV * HD * 2 + T * 4)
+        del an, qk, sw, kvp
         other_shapes(args, L, h, apklib, synth, torch, gen, dev, randn, pool, p, timed, record, reps, m, qw, kw, rope)
     sync()
 

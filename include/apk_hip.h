@@ -63,7 +63,8 @@ enum apk_dq_fmt {
 enum apk_fault {
     APK_FAULT_TOKEN_RANGE = 1,  /* an embedding id >= vocab was met on the device  */
     APK_FAULT_EXPERT_RANGE = 2, /* a routed expert id >= n_expert                  */
-    APK_FAULT_ROW_RANGE = 4     /* a gather index >= source rows                   */
+    APK_FAULT_ROW_RANGE = 4,    /* a gather / scatter row index out of range       */
+    APK_FAULT_CACHE_RANGE = 8   /* a KV-cache position >= capacity                 */
 };
 
 /* ------------------------------------------------------------ life cycle ---- */
@@ -149,6 +150,22 @@ int apk_add_rmsnorm_rows(apk_ctx* ctx, void* x, const void* delta, void* h, cons
 int apk_qknorm_rope_neox(apk_ctx* ctx, void* q, void* k, const float* qw, const float* kw, const float* rope,
                          size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim, float eps,
                          int dtype);
+
+/* apk_qknorm_rope_neox with the K/V cache store fused in: after the rotation, row r's k
+ * (all n_kv heads) and the same row of v are narrowed to fp16 (RNE) into cache row
+ * cache_pos[r].  Replaces the QK-norm+RoPE loop followed by KvCache::store_at(layer,
+ * base_pos + i, k_row, v_row) (crates/allpaka-model/src/kv.rs:682-697; call site
+ * model/attention.rs:170-200); every accelerator path of the reference fuses the same
+ * store (rmsnorm_rope_qk_store_table_dpos, gpu/cuda/kernels.rs:687-765; qk_prep,
+ * gpu/shaders/kernels.metal:7705-7712).  q and k are still updated in place.
+ * v: [rows][n_kv*head_dim] of dtype (read only); cache_pos: u32[rows] on the device;
+ * k_cache, v_cache: fp16 [capacity][n_kv*head_dim] (one layer's K and V planes).
+ * A position >= capacity skips that row's cache store and raises APK_FAULT_CACHE_RANGE
+ * (the reference asserts "position past capacity"). */
+int apk_qknorm_rope_kv_store(apk_ctx* ctx, void* q, void* k, const void* v, const float* qw, const float* kw,
+                             const float* rope, const uint32_t* cache_pos, void* k_cache, void* v_cache,
+                             size_t capacity, size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim,
+                             float eps, int dtype);
 
 /* Layer prologue as ONE launch: apk_add_rmsnorm_rows(x, delta, h, gamma, n, rows) and
  * apk_qknorm_rope_neox(q, k, qw, kw, rope, rows, ...) with the same arguments and the

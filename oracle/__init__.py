@@ -83,6 +83,8 @@ def lib():
         L.ora_moe_group.argtypes = [vp, vp, sz, sz, sz, vp, vp, vp, vp, vp]
         L.ora_gather_rows.argtypes = [vp, vp, sz, sz, vp]
         L.ora_gather_rows_f16.argtypes = [vp, vp, sz, sz, vp]
+        L.ora_kv_store_rows.argtypes = [vp, vp, sz, sz, vp, sz, vp, vp]
+        L.ora_kv_store_rows_f16.argtypes = [vp, vp, sz, sz, vp, sz, vp, vp]
         L.ora_add_rmsnorm_rows.argtypes = [vp, vp, vp, vp, sz, sz, f32]
         L.ora_add_rmsnorm_rows_f16.argtypes = [vp, vp, vp, vp, sz, sz, f32]
         _lib = L
@@ -370,3 +372,13 @@ def gather_rows(src, tok):
         _chk(src, np.uint16)
         lib().ora_gather_rows_f16(_p(src), _p(tok), tok.size, src.shape[1], _p(dst))
     return dst
+
+
+def kv_store_rows(k, v, pos, k_cache, v_cache):
+    """KvCache::store_at per row: k, v [rows, kv_dim] (f32, or fp16 bits) into the u16 caches [capacity, kv_dim]."""
+    pos = np.ascontiguousarray(pos, dtype=np.uint32)
+    rows, kv_dim = k.shape
+    _chk(k_cache, np.uint16), _chk(v_cache, np.uint16)
+    fn = lib().ora_kv_store_rows if k.dtype == np.float32 else lib().ora_kv_store_rows_f16
+    if fn(_p(k), _p(v), rows, kv_dim, _p(pos), k_cache.shape[0], _p(k_cache), _p(v_cache)):
+        raise OracleError("position past capacity")

@@ -802,3 +802,30 @@ ORA_API int ora_embed_rows_f16(const uint8_t *data, size_t data_len, int fmt, si
 ORA_API void ora_gather_rows_f16(const uint16_t *src, const uint32_t *tok, size_t total_rows, size_t cols, uint16_t *dst) {
     for (size_t r = 0; r < total_rows; r++) memcpy(dst + r * cols, src + (size_t)tok[r] * cols, cols * sizeof(uint16_t));
 }
+
+/* ----------------------------------------------------------- KV cache store
+ * KvCache::store_at (crates/allpaka-model/src/kv.rs:682-697): row i's k and v (kv_dim
+ * floats each) narrowed to f16 with ops::f16::from_f32 (= f32_to_f16, RNE) at cache row
+ * pos[i] of the layer's K and V planes.  Returns 1 where the reference asserts
+ * "position past capacity" (nothing is written for that row). */
+ORA_API int ora_kv_store_rows(const float *k, const float *v, size_t rows, size_t kv_dim, const uint32_t *pos,
+                              size_t capacity, uint16_t *k_cache, uint16_t *v_cache) {
+    int bad = 0;
+    for (size_t i = 0; i < rows; i++) {
+        if (pos[i] >= capacity) { bad = 1; continue; }
+        ora_f32_to_f16_slice(k + i * kv_dim, k_cache + (size_t)pos[i] * kv_dim, kv_dim);
+        ora_f32_to_f16_slice(v + i * kv_dim, v_cache + (size_t)pos[i] * kv_dim, kv_dim);
+    }
+    return bad;
+}
+/* fp16 activations: the rows are already halves; the store is a copy. */
+ORA_API int ora_kv_store_rows_f16(const uint16_t *k, const uint16_t *v, size_t rows, size_t kv_dim, const uint32_t *pos,
+                                  size_t capacity, uint16_t *k_cache, uint16_t *v_cache) {
+    int bad = 0;
+    for (size_t i = 0; i < rows; i++) {
+        if (pos[i] >= capacity) { bad = 1; continue; }
+        memcpy(k_cache + (size_t)pos[i] * kv_dim, k + i * kv_dim, kv_dim * 2);
+        memcpy(v_cache + (size_t)pos[i] * kv_dim, v + i * kv_dim, kv_dim * 2);
+    }
+    return bad;
+}

@@ -268,6 +268,53 @@ def test_rope_table_on_device(be, ora):
     assert f16_ulp_diff(host(tq), wq) <= TOL_F16_ULP and f16_ulp_diff(host(tk), wk) <= TOL_F16_ULP
 
 
+# --------------------------------------------- fused K/V cache store
+@pytest.mark.parametrize("rows,n_q,n_kv,hd,f16", [(1, 16, 8, 128, False), (64, 64, 8, 128, True), (300, 64, 8, 128, True),
+                                                   (7, 4, 4, 64, False), (5, 2, 1, 256, True), (2048, 16, 8, 128, False)])
+def test_qknorm_rope_kv_store(be, ora, rows, n_q, n_kv, hd, f16):
+    """QK-norm + RoPE with KvCache::store_at fused: q, k as the plain op; the cache rows hold
+    the rotated k and the row's v narrowed to f16 (RNE) at each row's position."""
+    s = synth()
+    g = s.rng(3, rows * 3 + hd)
+    cap = max(rows + 9, 40)
+    positions = g.permutation(cap)[:rows].astype(np.uint32)  # distinct cache rows, any order
+    q, k, qw, kw, inv, ropes = _qk_case(ora, 3, rows, n_q, n_kv, hd, f16, [int(p) for p in positions])
+    v = s.normal_f32(g, (rows, n_kv * hd))
+    if f16:
+        v = s.to_f16_bits(v)
+    wq, wk = q.copy(), k.copy()
+    ora.qknorm_rope_rows(wq, wk, n_q, n_kv, hd, qw, kw, ropes, 1e-6)
+    wkc, wvc = np.zeros((cap, n_kv * hd), np.uint16), np.zeros((cap, n_kv * hd), np.uint16)
+    ora.kv_store_rows(wk, v, positions, wkc, wvc)
+    tq, tk = dev(q), dev(k)
+    kc = torch.zeros((cap, n_kv * hd), dtype=torch.float16, device="cuda")
+    vc = torch.zeros_like(kc)
+    be.qknorm_rope_kv_store(tq, tk, dev(v), dev(qw), dev(kw), dev(ropes), dev(positions), kc, vc, n_q, n_kv, hd, 1e-6)
+    gk = host(tk)
+    for got, want in ((host(tq), wq), (gk, wk)):
+        if f16:
+            assert f16_ulp_diff(got, want) <= TOL_F16_ULP
+        else:
+            assert rel_err_f32(got, want) <= TOL_F32 and close_idiom(got, want)
+    assert np.array_equal(host(vc), wvc)  # v: a pure narrowing, bit-exact
+    # k cache: exactly the narrowing of the k this launch produced, and within 1 fp16 ulp (2 on the fp16 path) of the oracle's
+    mine_k, mine_v = np.zeros_like(wkc), np.zeros_like(wvc)
+    ora.kv_store_rows(gk, v, positions, mine_k, mine_v)
+    assert np.array_equal(host(kc), mine_k)
+    assert f16_ulp_diff(host(kc), wkc) <= (TOL_F16_ULP if f16 else 1)
+
+
+def test_kv_store_position_past_capacity_is_flagged_not_faulted(be, ora):
+    rows, n_q, n_kv, hd = 3, 2, 1, 128
+    q, k, qw, kw, inv, ropes = _qk_case(ora, 3, rows, n_q, n_kv, hd, False, [1, 2, 3])
+    kc = torch.zeros((4, n_kv * hd), dtype=torch.float16, device="cuda")
+    vc = torch.zeros_like(kc)
+    with pytest.raises(AssertionError, match="position past capacity"):
+        be.qknorm_rope_kv_store(dev(q), dev(k), dev(k), dev(qw), dev(kw), dev(ropes), dev(np.array([1, 4, 3], np.uint32)), kc, vc,
+                                n_q, n_kv, hd, 1e-6)
+    assert host(kc)[1].any() and host(kc)[3].any() and not host(kc)[[0, 2]].any()
+
+
 # ------------------------------------------- single-launch layer prologue
 @pytest.mark.parametrize("rows,n,n_q,n_kv,hd,f16", [
     (64, 5120, 64, 8, 128, True), (1, 5120, 64, 8, 128, True), (6, 5120, 64, 8, 128, True),

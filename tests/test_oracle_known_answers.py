@@ -666,3 +666,21 @@ def test_f16_variants_are_widen_op_round_once(ora):
     gf, uf = ora.f16_bits_to_f32(x.reshape(-1)), ora.f16_bits_to_f32(d.reshape(-1))
     ora.swiglu(gf, uf)
     assert np.array_equal(a, ora.f32_to_f16_bits(gf))
+
+
+def test_kv_store_rows_narrows_with_rne_at_the_right_rows(ora):
+    # crates/allpaka-model/src/kv.rs:682-697 (store_at) and :855 (vectors come back from the right position)
+    rng = np.random.default_rng(29)
+    k = rng.standard_normal((3, 16)).astype(np.float32)
+    v = rng.standard_normal((3, 16)).astype(np.float32)
+    kc, vc = np.zeros((8, 16), np.uint16), np.zeros((8, 16), np.uint16)
+    ora.kv_store_rows(k, v, [5, 0, 7], kc, vc)
+    assert np.array_equal(kc[[5, 0, 7]], k.astype(np.float16).view(np.uint16))
+    assert np.array_equal(vc[[5, 0, 7]], v.astype(np.float16).view(np.uint16))
+    assert not kc[[1, 2, 3, 4, 6]].any()
+    with pytest.raises(ora.OracleError):
+        ora.kv_store_rows(k, v, [5, 0, 8], kc, vc)
+    kh, vh = ora.f32_to_f16_bits(k), ora.f32_to_f16_bits(v)
+    kc2, vc2 = np.zeros_like(kc), np.zeros_like(vc)
+    ora.kv_store_rows(kh, vh, [5, 0, 7], kc2, vc2)
+    assert np.array_equal(kc2, kc) and np.array_equal(vc2, vc)
