@@ -66,6 +66,7 @@ std::vector<std::string> all_kernel_names() {
                                   "apk_embed_q4k_f16", "apk_embed_q8_0_f32", "apk_embed_q8_0_f16", "apk_route_topk",
                                   "apk_moe_permute", "apk_gather_rows", "apk_scatter_rows", "apk_copy"};
     for (const char* t : {"f32", "f16"}) {
+        for (const char* f : {"q5k", "q6k", "q2k", "q3k", "q5_0", "f16", "f32", "bf16"}) v.push_back(std::string("apk_embed_") + f + "_" + t);
         for (int c : kAddnormTiles) v.push_back(std::string("apk_add_rmsnorm_") + t + "_c" + std::to_string(c));
         for (int hd : kQkHeadDims) v.push_back(std::string("apk_layer_prologue_") + t + "_hd" + std::to_string(hd));
         for (int hd : kQkHeadDims)
@@ -146,8 +147,11 @@ size_t apk_row_bytes(int fmt, size_t n_in) {
 }
 
 int apk_can_embed(int fmt, size_t n_in) {
-    if (fmt != APK_FMT_Q8_0 && fmt != APK_FMT_Q4K) return 0;
-    return n_in > 0 && apk_row_bytes(fmt, n_in) != 0;
+    // every format of the unified codes; rows must be whole 16-byte output tiles and
+    // (all but Q4_K, which reads global memory directly) fit the 64 KiB LDS staging
+    const size_t rb = apk_row_bytes(fmt, n_in);
+    if (rb == 0 || n_in == 0 || n_in % 8) return 0;
+    return fmt == APK_FMT_Q4K || rb + 32 <= 64 * 1024;
 }
 
 int apk_init(int device, apk_ctx** out) {
@@ -534,16 +538,17 @@ static int embed_common(apk_ctx* c, int fmt, const void* table, size_t vocab, si
         void* args[] = {&table, &vocab32, &n_i, &ids_dev, &out, &c->fault_dev};
         return launch(c, out_dtype == APK_F32 ? "apk_embed_q4k_f32" : "apk_embed_q4k_f16", (unsigned)t, (unsigned)threads, 0, args);
     }
-    // Q8_0: one workgroup per row, the row staged in LDS
-    const size_t row_bytes = n_in / 32 * 34;
+    // every other format: one workgroup per row, the row staged in LDS
+    static const char* const kFmtName[10] = {"q4k", "q5k", "q6k", "q8_0", "q2k", "q3k", "q5_0", "f16", "f32", "bf16"};
+    const size_t row_bytes = apk_row_bytes(fmt, n_in);
     const size_t shmem = row_bytes + 32;
-    if (shmem > 64 * 1024) return fail(APK_DECLINE_SHAPE, "apk_embed_rows: Q8_0 row of %zu elements is too long", n_in);
     size_t threads = (n_in / (16 / elem_size(out_dtype)) + 63) / 64 * 64;  // one output tile per lane
-    if (threads > 1024) threads = 1024;
+    const size_t max_threads = fmt == APK_FMT_Q8_0 ? 1024 : 256;
+    if (threads > max_threads) threads = max_threads;
     uint64_t table_bytes = (uint64_t)vocab * row_bytes;
     void* args[] = {&table, &table_bytes, &vocab32, &n_i, &ids_dev, &out, &c->fault_dev};
-    return launch(c, out_dtype == APK_F32 ? "apk_embed_q8_0_f32" : "apk_embed_q8_0_f16", (unsigned)t, (unsigned)threads,
-                  (unsigned)shmem, args);
+    const std::string which = std::string("apk_embed_") + kFmtName[fmt] + (out_dtype == APK_F32 ? "_f32" : "_f16");
+    return launch(c, which, (unsigned)t, (unsigned)threads, (unsigned)shmem, args);
 }
 
 int apk_embed_rows(apk_ctx* c, int fmt, const void* table, size_t vocab, size_t n_in, const uint32_t* ids, size_t t,

@@ -648,6 +648,157 @@ extern "C" __global__ __launch_bounds__(1024) void apk_embed_q8_0_f16(const uint
     embed_q8_0_body<f16_t>(table, table_bytes, vocab, n_in, ids, out, fault);
 }
 
+// ---- the other GGUF formats of the unified dequant codes (gpu/common.rs:47-61) -------
+// One element decoder per format, a restatement of its block function in
+// crates/allpaka-gguf/src/dequant.rs with the same operation order (bit-exact), reading
+// the block's bytes from LDS.  `e` is the element index inside the block.
+DEV float lds_f16(const uint8_t* p) { return h2f(*(const uint16_t*)p); }  // blocks are 2-byte aligned
+
+template <int FMT> struct dq;
+template <> struct dq<6> {  // Q5_0, dequant.rs:131-141
+    static constexpr int BE = 32, BB = 22;
+    DEV float elem(const uint8_t* b, int e) {
+        const float d = lds_f16(b);
+        const uint32_t qh = (uint32_t)b[2] | ((uint32_t)b[3] << 8) | ((uint32_t)b[4] << 16) | ((uint32_t)b[5] << 24);
+        const int j = e & 15;
+        const uint32_t nib = e < 16 ? (b[6 + j] & 0x0fu) : (uint32_t)(b[6 + j] >> 4);
+        const uint32_t hb = (qh >> (e < 16 ? j : j + 16)) & 1u;
+        return d * (float)((int)(nib | (hb << 4)) - 16);
+    }
+};
+template <> struct dq<4> {  // Q2_K, dequant.rs:150-174
+    static constexpr int BE = 256, BB = 84;
+    DEV float elem(const uint8_t* b, int e) {
+        const int half = e >> 7, r = e & 127, si = r >> 5, within = r & 31, group = within >> 4, l = within & 15;
+        const uint32_t sc = b[half * 8 + si * 2 + group];
+        const float d = lds_f16(b + 80), dmin = lds_f16(b + 82);
+        const float dl = d * (float)(sc & 0xfu), ml = dmin * (float)(sc >> 4);
+        const uint32_t quant = (b[16 + half * 32 + group * 16 + l] >> (2 * si)) & 3u;
+        return dl * (float)quant - ml;
+    }
+};
+template <> struct dq<5> {  // Q3_K, dequant.rs:176-204 (scales: allpaka-dtype lib.rs:395-422)
+    static constexpr int BE = 256, BB = 110;
+    DEV float elem(const uint8_t* b, int e) {
+        const int half = e >> 7, r = e & 127, si = r >> 5, within = r & 31, group = within >> 4, l = within & 15;
+        const int is = half * 8 + si * 2 + group;
+        const uint8_t* pk = b + 96;
+        const uint32_t lo = is < 8 ? (pk[is] & 0xfu) : (uint32_t)(pk[is - 8] >> 4);
+        const uint32_t hi = (pk[8 + (is & 3)] >> (2 * (is >> 2))) & 3u;
+        const int sraw = (int)(int8_t)(lo | (hi << 4));
+        const float dl = lds_f16(b + 108) * (float)(sraw - 32);
+        const int idx = group * 16 + l;
+        const uint32_t m = 1u << (half * 4 + si);
+        const int quant = (int)((b[32 + half * 32 + idx] >> (2 * si)) & 3u) - ((b[idx] & m) ? 0 : 4);
+        return dl * (float)quant;
+    }
+};
+template <> struct dq<1> {  // Q5_K, dequant.rs:238-263
+    static constexpr int BE = 256, BB = 176;
+    DEV float elem(const uint8_t* b, int e) {
+        const int pair = e >> 6, r = e & 63, hn = r >> 5, l = r & 31, sub = 2 * pair + hn;
+        const uint8_t* pk = b + 4;
+        uint32_t sc, mn;
+        if (sub < 4) {
+            sc = pk[sub] & 63u;
+            mn = pk[sub + 4] & 63u;
+        } else {
+            sc = (pk[sub + 4] & 0xfu) | ((uint32_t)(pk[sub - 4] >> 6) << 4);
+            mn = (uint32_t)(pk[sub + 4] >> 4) | ((uint32_t)(pk[sub] >> 6) << 4);
+        }
+        const float dsc = lds_f16(b) * (float)sc, dm = lds_f16(b + 2) * (float)mn;
+        const uint32_t byte = b[48 + pair * 32 + l];
+        const uint32_t q4 = hn ? (byte >> 4) : (byte & 0xfu);
+        const uint32_t hb = (b[16 + l] >> sub) & 1u;
+        return dsc * (float)(q4 + 16u * hb) - dm;
+    }
+};
+template <> struct dq<2> {  // Q6_K, dequant.rs:271-295: (d * scale) * q
+    static constexpr int BE = 256, BB = 210;
+    DEV float elem(const uint8_t* b, int e) {
+        const int half = e >> 7, r = e & 127, quarter = r >> 5, l = r & 31, is = l >> 4;
+        const uint8_t* ql = b + half * 64;
+        const uint32_t qh = b[128 + half * 32 + l];
+        const uint32_t lo = (quarter & 1) ? ql[l + 32] : ql[l];
+        const uint32_t nib = quarter < 2 ? (lo & 0xfu) : (lo >> 4);
+        const int qv = (int)(int8_t)(nib | (((qh >> (2 * quarter)) & 3u) << 4)) - 32;
+        const float sc = (float)(int8_t)b[192 + half * 8 + is + 2 * quarter];
+        return lds_f16(b + 208) * sc * (float)qv;
+    }
+};
+template <> struct dq<7> {  // F16
+    static constexpr int BE = 1, BB = 2;
+    DEV float elem(const uint8_t* b, int) { return lds_f16(b); }
+};
+template <> struct dq<9> {  // BF16, allpaka-dtype lib.rs:188-190
+    static constexpr int BE = 1, BB = 2;
+    DEV float elem(const uint8_t* b, int) { return __builtin_bit_cast(float, (uint32_t)(*(const uint16_t*)b) << 16); }
+};
+template <> struct dq<8> {  // F32 (rows are 4-byte aligned)
+    static constexpr int BE = 1, BB = 4;
+    DEV float elem(const uint8_t* b, int) { return *(const float*)b; }
+};
+
+// One workgroup per row: the row's bytes are staged in LDS with 16-byte loads (from the
+// aligned address at or below the row start; rows of these formats are not 16-byte
+// multiples), then each lane decodes one 16-byte output tile per pass, consecutive lanes
+// writing consecutive tiles.
+template <int FMT, typename TO>
+DEV void embed_staged_body(const uint8_t* table, uint64_t table_bytes, uint32_t vocab, int n_in, const uint32_t* ids,
+                           TO* out, uint32_t* fault) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t stage[];
+    constexpr int OPT = io<TO>::VEC, BE = dq<FMT>::BE, BB = dq<FMT>::BB;
+    const uint64_t t = blockIdx.x;
+    const uint32_t id = ids[t];
+    if (id >= vocab) {
+        if (threadIdx.x == 0) atomicOr(fault, APK_FAULT_TOKEN_RANGE);
+        return;
+    }
+    const uint64_t row_bytes = (uint64_t)(n_in / BE) * BB;
+    const uint64_t start = (uint64_t)id * row_bytes;
+    const uint64_t astart = start & ~(uint64_t)15;  // table base is 16-byte aligned
+    const int mis = (int)(start - astart);
+    const int nvec = (int)((mis + row_bytes + 15) / 16);
+    for (int i = threadIdx.x; i < nvec; i += blockDim.x) {
+        const uint64_t off = astart + (uint64_t)i * 16;
+        u32x4 v;
+        if (off + 16 <= table_bytes) {
+            v = __builtin_nontemporal_load((const u32x4*)(table + off));
+        } else {  // last tile of the last row: stay inside the table
+            uint32_t w[4] = {0, 0, 0, 0};
+            for (int b = 0; b < 16; b++)
+                if (off + b < table_bytes) w[b >> 2] |= (uint32_t)table[off + b] << (8 * (b & 3));
+            v = u32x4{w[0], w[1], w[2], w[3]};
+        }
+        *(u32x4*)(stage + i * 16) = v;
+    }
+    __syncthreads();
+    const int ntiles = n_in / OPT;  // the host admits only n_in that are whole tiles
+    for (int g = threadIdx.x; g < ntiles; g += blockDim.x) {
+        const int e0 = g * OPT;
+        float o[OPT];
+#pragma unroll
+        for (int i = 0; i < OPT; i++) {
+            const int e = e0 + i;
+            o[i] = dq<FMT>::elem(stage + mis + (e / BE) * BB, e % BE);
+        }
+        io<TO>::store_nt(out + t * (uint64_t)n_in + e0, o);
+    }
+}
+#define APK_EMBED_GEN(NAME, FMT)                                                                                          \
+    extern "C" __global__ __launch_bounds__(256) void apk_embed_##NAME##_f32(                                             \
+        const uint8_t* table, uint64_t table_bytes, uint32_t vocab, int n_in, const uint32_t* ids, float* out,            \
+        uint32_t* fault) {                                                                                                \
+        embed_staged_body<FMT, float>(table, table_bytes, vocab, n_in, ids, out, fault);                                  \
+    }                                                                                                                     \
+    extern "C" __global__ __launch_bounds__(256) void apk_embed_##NAME##_f16(                                             \
+        const uint8_t* table, uint64_t table_bytes, uint32_t vocab, int n_in, const uint32_t* ids, f16_t* out,            \
+        uint32_t* fault) {                                                                                                \
+        embed_staged_body<FMT, f16_t>(table, table_bytes, vocab, n_in, ids, out, fault);                                  \
+    }
+APK_EMBED_GEN(q5k, 1) APK_EMBED_GEN(q6k, 2) APK_EMBED_GEN(q2k, 4) APK_EMBED_GEN(q3k, 5) APK_EMBED_GEN(q5_0, 6)
+APK_EMBED_GEN(f16, 7) APK_EMBED_GEN(f32, 8) APK_EMBED_GEN(bf16, 9)
+
 // =========================================================================
 // MoE router: per token softmax (or sigmoid) over n_expert <= 256 logits, top-k
 // by descending selection score with the LOWER INDEX winning ties, winners

@@ -122,7 +122,9 @@ int apk_timer_end(apk_ctx* ctx, float* ms_out);
  * embed_row_f32_dtoken kernels (token id read on the device).
  * table: [vocab][apk_row_bytes(fmt,n_in)] bytes, 16-byte aligned; ids: u32[t];
  * out: [t][n_in] of out_dtype.  An id >= vocab leaves its row untouched and
- * raises APK_FAULT_TOKEN_RANGE.  Formats taken: APK_FMT_Q8_0, APK_FMT_Q4K. */
+ * raises APK_FAULT_TOKEN_RANGE.  All ten formats of apk_dq_fmt are taken (Q8_0 and Q4_K,
+ * the formats of the benchmark configurations, by dedicated kernels); n_in must be a
+ * multiple of 8 and a row must fit 64 KiB (apk_can_embed tells). */
 int apk_embed_rows(apk_ctx* ctx, int fmt, const void* table, size_t vocab, size_t n_in, const uint32_t* ids,
                    size_t t, void* out, int out_dtype);
 /* Same with the ids on the host: range-checked BEFORE anything is enqueued

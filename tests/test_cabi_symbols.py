@@ -60,7 +60,8 @@ def test_row_bytes_and_format_codes_follow_the_reference():
     assert [lib.FMT_Q4K, lib.FMT_Q5K, lib.FMT_Q6K, lib.FMT_Q8_0, lib.FMT_Q2K, lib.FMT_Q3K, lib.FMT_Q5_0, lib.FMT_F16,
             lib.FMT_F32, lib.FMT_BF16] == list(range(10))
     assert L.apk_can_embed(lib.FMT_Q8_0, 1024) == 1 and L.apk_can_embed(lib.FMT_Q4K, 5120) == 1
-    assert L.apk_can_embed(lib.FMT_Q4K, 100) == 0 and L.apk_can_embed(lib.FMT_Q6K, 256) == 0
+    assert L.apk_can_embed(lib.FMT_Q4K, 100) == 0 and L.apk_can_embed(77, 256) == 0 and L.apk_can_embed(lib.FMT_F32, 3) == 0
+    assert all(L.apk_can_embed(f, 512) == 1 for f in range(10))  # gpu_parity.rs:1147: all ten formats embed
 
 
 def test_no_device_declines_instead_of_failing():

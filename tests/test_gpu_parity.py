@@ -83,6 +83,51 @@ def test_embed_rows_bit_exact(be, ora, fmt_name, n_in, vocab, t, out_f16):
     assert np.array_equal(host(r), want[0])
 
 
+def _lcg_bytes(n, state=0x243F6A8885A308D3):
+    """The byte stream of the reference's GPU parity region (crates/allpaka-backend/tests/gpu_parity.rs:73-80)."""
+    out = np.empty(n, np.uint8)
+    mul, inc, mask = 6364136223846793005, 1442695040888963407, (1 << 64) - 1
+    for i in range(n):
+        state = (state * mul + inc) & mask
+        out[i] = state >> 56
+    return out
+
+
+_SCALE_OFFS = {"Q8_0": (34, [0]), "Q2K": (84, [80, 82]), "Q3K": (110, [108]), "Q4K": (144, [0, 2]), "Q5K": (176, [0, 2]),
+               "Q6K": (210, [208]), "Q5_0": (22, [0])}
+
+
+@pytest.mark.parametrize("fmt_name", ["Q4K", "Q5K", "Q6K", "Q8_0", "Q2K", "Q3K", "Q5_0", "F16", "F32", "BF16"])
+@pytest.mark.parametrize("out_f16", [False, True])
+def test_embed_all_ten_formats_bit_exact(be, ora, fmt_name, out_f16):
+    """All ten formats, hidden 512, 6 rows, the reference's fixture style: LCG bytes with the f16
+    scale fields tamed to 0x211F (gpu_parity.rs:100-137, :1147-1214) -- here bit-exact, not 1e-4."""
+    import allpaka_amd as apk
+
+    fmt, hidden, vocab = ora.FMT[fmt_name], 512, 6
+    rb = ora.expected_bytes(fmt, hidden)
+    raw = _lcg_bytes(vocab * rb, 0x243F6A8885A308D3 + fmt)
+    if fmt_name in _SCALE_OFFS:
+        bb, offs = _SCALE_OFFS[fmt_name]
+        blocks = raw.reshape(-1, bb)
+        for o in offs:
+            blocks[:, o], blocks[:, o + 1] = 0x1F, 0x21
+        blocks[0, offs[0]:offs[0] + 2] = [0x01, 0x00]  # one f16-subnormal scale
+    elif fmt_name == "F32":
+        raw = ((np.arange(vocab * hidden) % 61 - 30) * np.float32(0.03)).astype(np.float32).view(np.uint8)
+    else:  # F16 / BF16: keep the exponent away from inf/NaN so equality is meaningful
+        w = raw.view(np.uint16)
+        w &= np.uint16(0xBFFF)
+    ids = np.array([3, 0, 5, 5, 1, 2, 4], np.uint32)
+    want = ora.embed_rows(raw, fmt, vocab, hidden, ids, out_f16=out_f16)
+    qm = apk.QuantMat(be, dev(raw), fmt, vocab, hidden)
+    out = torch.zeros((ids.size, hidden), dtype=torch.float16 if out_f16 else torch.float32, device="cuda")
+    qm.rows_into(dev(ids), out)
+    got = host(out)
+    assert np.array_equal(got.view(np.uint16 if out_f16 else np.uint32), want.view(np.uint16 if out_f16 else np.uint32))
+    assert np.array_equal(host(qm.row(3, dtype=out.dtype)), want[0])  # token 3 of 6, as the reference's test
+
+
 def test_embed_subnormal_scales_and_reference_vectors(be, ora):
     import allpaka_amd as apk
 
@@ -130,10 +175,12 @@ def test_embed_errors_and_declines(be, ora):
         qm.rows_into(dev(np.array([0, 5], np.uint32)), out)
     assert np.all(host(out)[1] == 3.0) and np.all(host(out)[0] == 0.0)
     assert be.take_faults() == 0  # cleared by the read above
-    # a format outside the device path declines, it does not fail
-    q6 = apk.QuantMat(be, dev(np.zeros(210, np.uint8)), ora.FMT["Q6K"], 1, 256)
+    # a row the device path does not take (not whole 16-byte output tiles) declines, it does not fail
+    f32m = apk.QuantMat(be, dev(np.zeros(12, np.uint8)), ora.FMT["F32"], 1, 3)
     with pytest.raises(apk.Declined):
-        q6.row(0)
+        f32m.row(0)
+    with pytest.raises(ValueError):
+        apk.QuantMat(be, data, 42, 1, 64)
 
 
 # ------------------------------------------------------------- add + RMSNorm
