@@ -261,6 +261,28 @@ class Backend:
         self.sync()
         return dst
 
+    def moe_combine_add_rmsnorm(self, x, flat, tok_off, hit_row, hit_w, h, gamma, eps):
+        """x[t] += sum over the token's hits of hit_w * flat[hit_row] (add_scaled_slice order), then
+        h = rmsnorm(x) * gamma (moe.rs:298-333 + the residual add + the next norm); h=None: no norm."""
+        n = flat.shape[1]
+        rows = x.numel() // n
+        assert x.numel() == rows * n and tok_off.numel() == rows + 1 and flat.dtype == x.dtype
+        assert h is None or (h.numel() >= rows * n and gamma is not None and gamma.numel() == n)
+        self._enter()
+        check(self.L.apk_moe_combine_add_rmsnorm(self.h, _ptr(x), _ptr(flat), _ptr(tok_off), _ptr(hit_row), _ptr(hit_w),
+                                                 flat.shape[0], _ptr(h), _ptr(gamma), n, rows, eps, _dt(x)))
+        self.sync()
+
+    def argmax_rows(self, logits):
+        """Greedy pick per row: (0..n).max_by(total_cmp) of forward_greedy (decode.rs:628-630)."""
+        rows, n = logits.shape
+        assert logits.dtype == torch.float32
+        out = torch.empty(rows, dtype=torch.int32, device=self.device)
+        self._enter()
+        check(self.L.apk_argmax_rows(self.h, _ptr(logits), rows, n, _ptr(out)))
+        self.sync()
+        return out
+
 
 class QuantMat:
     """QuantMat::{new,row,row_into} (quantmat/mod.rs:39-89) over a device-resident table."""

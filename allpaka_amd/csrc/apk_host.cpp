@@ -64,10 +64,11 @@ const int kQkHeadDims[] = {64, 128, 256};
 std::vector<std::string> all_kernel_names() {
     std::vector<std::string> v = {"apk_swiglu_f32", "apk_swiglu_f16", "apk_rope_table", "apk_embed_q4k_f32",
                                   "apk_embed_q4k_f16", "apk_embed_q8_0_f32", "apk_embed_q8_0_f16", "apk_route_topk",
-                                  "apk_moe_permute", "apk_gather_rows", "apk_scatter_rows", "apk_copy"};
+                                  "apk_moe_permute", "apk_gather_rows", "apk_scatter_rows", "apk_argmax_rows", "apk_copy"};
     for (const char* t : {"f32", "f16"}) {
         for (const char* f : {"q5k", "q6k", "q2k", "q3k", "q5_0", "f16", "f32", "bf16"}) v.push_back(std::string("apk_embed_") + f + "_" + t);
         for (int c : kAddnormTiles) v.push_back(std::string("apk_add_rmsnorm_") + t + "_c" + std::to_string(c));
+        for (int c : {1, 2, 4}) v.push_back(std::string("apk_combine_add_rmsnorm_") + t + "_c" + std::to_string(c));
         for (int hd : kQkHeadDims) v.push_back(std::string("apk_layer_prologue_") + t + "_hd" + std::to_string(hd));
         for (int hd : kQkHeadDims)
             for (int it : kQkIters) {
@@ -90,6 +91,8 @@ struct apk_ctx {
     uint32_t* ids_stage_dev = nullptr;
     size_t ids_stage_cap = 0;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    void* argmax_scratch = nullptr;  // one 128-byte line per row: u64 running best + u32 arrivals; zero between calls
+    size_t argmax_rows_cap = 0;
     std::mutex mu;
     std::map<uintptr_t, Mapping> attached;
     std::atomic<uint64_t> calls{0}, dispatches{0}, encode_ns{0}, wait_ns{0};
@@ -199,6 +202,7 @@ int apk_shutdown(apk_ctx* c) {
     if (c->ids_stage_dev) (void)hipFree(c->ids_stage_dev);
     if (c->ids_stage_host) (void)hipHostFree(c->ids_stage_host);
     if (c->fault_dev) (void)hipFree(c->fault_dev);
+    if (c->argmax_scratch) (void)hipFree(c->argmax_scratch);
     if (c->ev0) (void)hipEventDestroy(c->ev0);
     if (c->ev1) (void)hipEventDestroy(c->ev1);
     if (c->stream) (void)hipStreamDestroy(c->stream);
@@ -657,6 +661,70 @@ int apk_scatter_rows(apk_ctx* c, const void* src, const uint32_t* hit_row, size_
     uint32_t total32 = (uint32_t)total_rows;
     void* args[] = {&src, &hit_row, &k_i, &total32, &row_vecs, &dst, &c->fault_dev};
     return launch(c, "apk_scatter_rows", (unsigned)rows, 256, 0, args);
+}
+
+int apk_moe_combine_add_rmsnorm(apk_ctx* c, void* x, const void* flat, const uint32_t* tok_off, const uint32_t* hit_row,
+                                const float* hit_w, size_t total_rows, void* h, const float* gamma, size_t n, size_t rows,
+                                float eps, int dtype) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_moe_combine_add_rmsnorm: ctx is NULL");
+    CallScope s(c);
+    const int es = elem_size(dtype);
+    if (!es) return fail(APK_DECLINE_UNSUPPORTED, "apk_moe_combine_add_rmsnorm: dtype %d", dtype);
+    if (rows == 0) return APK_OK;
+    if (!x || !flat || !tok_off || !hit_row || !hit_w || (h && !gamma))
+        return fail(APK_DECLINE_NULL, "apk_moe_combine_add_rmsnorm: NULL tensor");
+    const size_t vec = 16 / es;
+    if (n == 0 || n % vec) return fail(APK_DECLINE_SHAPE, "apk_moe_combine_add_rmsnorm: n=%zu is not a multiple of %zu", n, vec);
+    if (!aligned16(x) || !aligned16(flat) || (h && !aligned16(h)) || (gamma && !aligned16(gamma)))
+        return fail(APK_DECLINE_SHAPE, "apk_moe_combine_add_rmsnorm: tensors must be 16-byte aligned");
+    if (rows > 0x7fffffffu || n > 0x7fffffffu || total_rows > 0xffffffffu)
+        return fail(APK_DECLINE_SHAPE, "apk_moe_combine_add_rmsnorm: too large");
+    const size_t nchunks = n / vec;
+    int nch = 0;
+    size_t waves = 0;
+    for (int cand : {1, 2, 4}) {
+        const size_t w = (nchunks + 64 * (size_t)cand - 1) / (64 * (size_t)cand);
+        if (w * 64 > 1024) continue;
+        nch = cand;
+        waves = w;
+        if (rows * w <= 2048) break;
+    }
+    if (!nch) return fail(APK_DECLINE_SHAPE, "apk_moe_combine_add_rmsnorm: row of %zu elements is too long", n);
+    if (int rc = set_device(c)) return rc;
+    int n_i = (int)n;
+    uint32_t total32 = (uint32_t)total_rows;
+    void* args[] = {&x, &flat, &tok_off, &hit_row, &hit_w, &total32, &h, &gamma, &n_i, &eps, &c->fault_dev};
+    const std::string which = std::string("apk_combine_add_rmsnorm_") + (dtype == APK_F32 ? "f32" : "f16") + "_c" + std::to_string(nch);
+    return launch(c, which, (unsigned)rows, (unsigned)(waves * 64), 0, args);
+}
+
+int apk_argmax_rows(apk_ctx* c, const float* logits, size_t rows, size_t n, uint32_t* out) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_argmax_rows: ctx is NULL");
+    CallScope s(c);
+    if (rows == 0) return APK_OK;
+    if (!logits || !out) return fail(APK_DECLINE_NULL, "apk_argmax_rows: NULL tensor");
+    if (n == 0 || n > 0xffffffffu || rows > (1u << 20)) return fail(APK_DECLINE_SHAPE, "apk_argmax_rows: sizes out of range");
+    if (int rc = set_device(c)) return rc;
+    if (rows > c->argmax_rows_cap) {
+        HIP_TRY(hipStreamSynchronize(c->stream));  // a previous launch may still use the old scratch
+        if (c->argmax_scratch) (void)hipFree(c->argmax_scratch);
+        c->argmax_scratch = nullptr;
+        c->argmax_rows_cap = 0;
+        const size_t cap = rows < 256 ? 256 : rows;
+        HIP_TRY(hipMalloc(&c->argmax_scratch, cap * 128));
+        HIP_TRY(hipMemsetAsync(c->argmax_scratch, 0, cap * 128, c->stream));
+        c->argmax_rows_cap = cap;
+    }
+    // enough workgroups per row to spread a vocabulary-sized row over the chip: ~4 K logits each
+    // (one pass of 4 16-byte loads per lane)
+    size_t parts = (n + 4095) / 4096;
+    if (parts > 64) parts = 64;
+    if (parts < 1) parts = 1;
+    while (parts > 1 && rows * parts > 8192) parts /= 2;
+    uint64_t n64 = n;
+    int parts_i = (int)parts;
+    void* args[] = {&logits, &n64, &parts_i, &c->argmax_scratch, &out};
+    return launch(c, "apk_argmax_rows", (unsigned)(rows * parts), 256, 0, args);
 }
 
 int apk_copy(apk_ctx* c, const void* src, void* dst, size_t bytes) {

@@ -104,6 +104,20 @@ DEV double wave_sum_f64(double v, int width) {
     return v;
 }
 
+DEV uint32_t total_order_key(float f) {  // f32::total_cmp as an unsigned key
+    int32_t b = __builtin_bit_cast(int32_t, f);
+    b ^= (int32_t)(((uint32_t)(b >> 31)) >> 1);
+    return (uint32_t)b ^ 0x80000000u;
+}
+DEV uint64_t wave_max_u64(uint64_t v) {
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        uint64_t other = __shfl_xor(v, o, 64);
+        v = other > v ? other : v;
+    }
+    return v;
+}
+
 // =========================================================================
 // SwiGLU: gate[i] = silu(gate[i]) * up[i], silu(x) = x / (1 + exp(-x))
 // (activation.rs:19-22, :116-119).  Pure stream: 2 reads + 1 write / element.
@@ -268,6 +282,179 @@ DEV void add_rmsnorm_body(T* x, const T* delta, T* h, const float* gamma, int n,
     APK_ADDNORM(T, TN, 12, 256) APK_ADDNORM(T, TN, 16, 256) APK_ADDNORM(T, TN, 20, 256)
 APK_ADDNORM_ALL(float, f32)
 APK_ADDNORM_ALL(f16_t, f16)
+
+// =========================================================================
+// MoE combine + residual add + the next RMSNorm, one pass per token row
+// (moe.rs:298-333 then decode.rs:775 / prefill.rs:308-314):
+//   out = 0; for each hit of the token, in CSR order: out = fma(down[hit_row], hit_w, out)
+//   (ops::add_scaled_slice, blas.rs:25-102, x86 arm: one rounding per hit);
+//   x += out;  h = rmsnorm(x) * gamma  (skipped when h is null).
+// Same row layout as add+RMSNorm: W waves per row, NCH tiles per lane; the k
+// expert rows of a token are streamed two hits at a time.
+// =========================================================================
+template <typename T, int NCH>
+DEV void combine_add_rmsnorm_body(T* x, const T* flat, const uint32_t* tok_off, const uint32_t* hit_row,
+                                  const float* hit_w, uint32_t total_rows, T* h, const float* gamma, int n, float eps,
+                                  uint32_t* fault) {
+    constexpr int VEC = io<T>::VEC;
+    typedef typename stat<T>::acc_t acc_t;
+    __shared__ acc_t part[16];
+    const int nchunks = n / VEC;
+    const uint64_t row = blockIdx.x;
+    T* xr = x + row * (uint64_t)n;
+    const uint32_t h0 = tok_off[row], h1 = tok_off[row + 1];
+    int cidx[NCH];
+    typename io<T>::raw_t xraw[NCH];
+#pragma unroll
+    for (int j = 0; j < NCH; j++) {
+        cidx[j] = min((int)(threadIdx.x + j * blockDim.x), nchunks - 1);
+        xraw[j] = io<T>::ldraw_nt(xr + cidx[j] * VEC);
+    }
+    float acc[NCH][VEC];
+#pragma unroll
+    for (int j = 0; j < NCH; j++)
+#pragma unroll
+        for (int i = 0; i < VEC; i++) acc[j][i] = 0.0f;
+    for (uint32_t k = h0; k < h1; k += 2) {  // uniform for the workgroup
+        const bool two = k + 1 < h1;
+        uint32_t r0 = hit_row[k], r1 = two ? hit_row[k + 1] : 0u;
+        const float w0 = hit_w[k], w1 = two ? hit_w[k + 1] : 0.0f;
+        const bool ok0 = r0 < total_rows, ok1 = two && r1 < total_rows;
+        if ((!ok0 || (two && !ok1)) && threadIdx.x == 0) atomicOr(fault, APK_FAULT_ROW_RANGE);
+        r0 = ok0 ? r0 : 0u;
+        r1 = ok1 ? r1 : 0u;
+        typename io<T>::raw_t d0[NCH], d1[NCH];
+#pragma unroll
+        for (int j = 0; j < NCH; j++) {
+            d0[j] = io<T>::ldraw_nt(flat + (uint64_t)r0 * n + cidx[j] * VEC);
+            d1[j] = io<T>::ldraw_nt(flat + (uint64_t)r1 * n + cidx[j] * VEC);
+        }
+#pragma unroll
+        for (int j = 0; j < NCH; j++) {
+            float a[VEC], b[VEC];
+            io<T>::widen(d0[j], a);
+            io<T>::widen(d1[j], b);
+#pragma unroll
+            for (int i = 0; i < VEC; i++) {
+                if (ok0) acc[j][i] = __builtin_fmaf(a[i], w0, acc[j][i]);
+                if (ok1) acc[j][i] = __builtin_fmaf(b[i], w1, acc[j][i]);
+            }
+        }
+    }
+    float v[NCH][VEC];
+    acc_t ss = 0;
+#pragma unroll
+    for (int j = 0; j < NCH; j++) {
+        const int c = threadIdx.x + j * blockDim.x;
+        io<T>::widen(xraw[j], v[j]);
+#pragma unroll
+        for (int i = 0; i < VEC; i++) v[j][i] = v[j][i] + acc[j][i];
+        if (c < nchunks) io<T>::store(xr + c * VEC, v[j]);
+        acc_t s8 = 0;
+#pragma unroll
+        for (int i = 0; i < VEC; i++) s8 = stat<T>::sq(s8, v[j][i]);
+        ss += c < nchunks ? s8 : (acc_t)0;
+    }
+    if (h == nullptr) return;  // uniform: combine + residual only
+    ss = stat<T>::wave_sum(ss);
+    const int nwaves = (blockDim.x + 63) >> 6;
+    if (nwaves > 1) {
+        if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+        __syncthreads();
+        ss = 0;
+        for (int w = 0; w < nwaves; w++) ss += part[w];
+    }
+    const acc_t scale = stat<T>::rscale(ss, n, eps);
+    T* hr = h + row * (uint64_t)n;
+#pragma unroll
+    for (int j = 0; j < NCH; j++) {
+        const int c = threadIdx.x + j * blockDim.x;
+        if (c < nchunks) {
+            float g[VEC], o[VEC];
+#pragma unroll
+            for (int q = 0; q < VEC; q += 4) io<float>::load(gamma + c * VEC + q, g + q);
+#pragma unroll
+            for (int i = 0; i < VEC; i++) o[i] = stat<T>::apply(v[j][i], scale, g[i]);
+            io<T>::store_nt(hr + c * VEC, o);
+        }
+    }
+}
+#define APK_COMBINE(T, TN, NCH)                                                                                        \
+    extern "C" __global__ __launch_bounds__(1024) void apk_combine_add_rmsnorm_##TN##_c##NCH(                         \
+        T* x, const T* flat, const uint32_t* tok_off, const uint32_t* hit_row, const float* hit_w, uint32_t total_rows, \
+        T* h, const float* gamma, int n, float eps, uint32_t* fault) {                                                 \
+        combine_add_rmsnorm_body<T, NCH>(x, flat, tok_off, hit_row, hit_w, total_rows, h, gamma, n, eps, fault);       \
+    }
+APK_COMBINE(float, f32, 1) APK_COMBINE(float, f32, 2) APK_COMBINE(float, f32, 4)
+APK_COMBINE(f16_t, f16, 1) APK_COMBINE(f16_t, f16, 2) APK_COMBINE(f16_t, f16, 4)
+
+// Greedy pick over rows of logits: the LAST maximum under f32::total_cmp, i.e. Rust's
+// (0..n).max_by(total_cmp) of Model::forward_greedy (model/decode.rs:628-630): ties go to
+// the higher index.  A row is split over `parts` workgroups; each folds its slice into a
+// (key << 32 | index) word and merges it with an atomic max into best[row]; the last
+// workgroup of a row (counted next to it) writes out[row] and re-arms both words.
+// scratch: one 128-byte line per row (word 0: running best, word 1: arrivals), so the
+// atomics of different rows never share a cache line.
+extern "C" __global__ __launch_bounds__(256) void apk_argmax_rows(const float* logits, uint64_t n, int parts,
+                                                                 unsigned long long* scratch, uint32_t* out) {
+    __shared__ unsigned long long wbest[4];
+    const uint32_t row = blockIdx.x / parts, part = blockIdx.x % parts;
+    unsigned long long* best = scratch + (uint64_t)row * 16;
+    uint32_t* done = (uint32_t*)(best + 1);
+    const float* lr = logits + (uint64_t)row * n;
+    unsigned long long b = 0;
+    auto fold = [&](float v, uint64_t i) {
+        const unsigned long long cand = ((unsigned long long)total_order_key(v) << 32) | (unsigned long long)i;
+        b = cand > b ? cand : b;  // equal keys: the higher index is the larger word
+    };
+    uint64_t lo, hi;
+    if ((n & 3) == 0) {  // rows are 16-byte aligned: 16-byte tiles, 4 loads in flight per lane
+        const uint64_t ntile = n >> 2, per = (ntile + parts - 1) / parts;
+        lo = (uint64_t)part * per;
+        hi = min(lo + per, ntile);
+        const f32x4* lt = (const f32x4*)lr;
+        for (uint64_t i0 = lo + threadIdx.x; i0 < hi; i0 += 4 * blockDim.x) {
+            f32x4 t[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const uint64_t i = i0 + (uint64_t)j * blockDim.x;
+                t[j] = __builtin_nontemporal_load(lt + (i < hi ? i : i0));
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const uint64_t i = i0 + (uint64_t)j * blockDim.x;
+                if (i < hi) {
+                    fold(t[j].x, 4 * i);
+                    fold(t[j].y, 4 * i + 1);
+                    fold(t[j].z, 4 * i + 2);
+                    fold(t[j].w, 4 * i + 3);
+                }
+            }
+        }
+    } else {
+        const uint64_t per = (n + parts - 1) / parts;
+        lo = (uint64_t)part * per;
+        hi = min(lo + per, n);
+        for (uint64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) fold(lr[i], i);
+    }
+    b = wave_max_u64(b);
+    if ((threadIdx.x & 63) == 0) wbest[threadIdx.x >> 6] = b;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < (int)(blockDim.x >> 6); w++) b = wbest[w] > b ? wbest[w] : b;
+        // No device-scope fence (it would write back the whole L2): the arrival count is made
+        // data-dependent on the returned value of the max, so the max is performed first; the
+        // last arrival therefore sees every max of the row.
+        const unsigned long long prev = atomicMax(best, b);
+        uint32_t inc = 1u;
+        asm volatile("" : "+v"(inc) : "v"((uint32_t)prev));
+        if (atomicAdd(done, inc) == (uint32_t)parts - 1u) {  // last workgroup of the row
+            const unsigned long long win = atomicExch(best, 0ull);
+            out[row] = (uint32_t)(win & 0xffffffffull);
+            atomicExch(done, 0u);
+        }
+    }
+}
 
 // =========================================================================
 // Per-head QK-norm + NeoX RoPE, in place on q [rows, n_q*HD] and k [rows, n_kv*HD]
@@ -806,11 +993,6 @@ APK_EMBED_GEN(f16, 7) APK_EMBED_GEN(f32, 8) APK_EMBED_GEN(bf16, 9)
 // l, l+64, l+128, l+192.  For softmax without bias the selection runs on the
 // raw logits (same order as the probabilities, no dependence on exp rounding).
 // =========================================================================
-DEV uint32_t total_order_key(float f) {  // f32::total_cmp as an unsigned key
-    int32_t b = __builtin_bit_cast(int32_t, f);
-    b ^= (int32_t)(((uint32_t)(b >> 31)) >> 1);
-    return (uint32_t)b ^ 0x80000000u;
-}
 DEV float wave_max_f32(float v) {
 #pragma unroll
     for (int o = 1; o < 64; o <<= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
@@ -821,15 +1003,6 @@ DEV float wave_sum_f32(float v) {
     for (int o = 1; o < 64; o <<= 1) v += __shfl_xor(v, o, 64);
     return v;
 }
-DEV uint64_t wave_max_u64(uint64_t v) {
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-        uint64_t other = __shfl_xor(v, o, 64);
-        v = other > v ? other : v;
-    }
-    return v;
-}
-
 extern "C" __global__ __launch_bounds__(256) void apk_route_topk(const float* logits, const float* bias, int rows,
                                                                 int n_expert, int k, int norm, float scale,
                                                                 int sigmoid, uint32_t* ids, float* wout) {

@@ -44,6 +44,8 @@ SYMBOLS = {
     "apk_moe_permute": (_i, [_vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp]),
     "apk_gather_rows": (_i, [_vp, _vp, _vp, _sz, _sz, _sz, _vp, _i]),
     "apk_scatter_rows": (_i, [_vp, _vp, _vp, _sz, _sz, _sz, _sz, _vp, _i]),
+    "apk_moe_combine_add_rmsnorm": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _sz, _sz, _f, _i]),
+    "apk_argmax_rows": (_i, [_vp, _vp, _sz, _sz, _vp]),
     "apk_copy": (_i, [_vp, _vp, _vp, _sz]),
 }
 

@@ -311,6 +311,24 @@ def other_shapes(args, L, h, apklib, synth, torch, gen, dev, randn, pool, p, tim
     record("scatter_rows (permute, token-side)", tagm, us, TM * HM * 4 + TM * K * HM * 4 + TM * K * 4)
     us = timed(lambda i: check(L.apk_swiglu(h, p(se[i % len(se)]["gate"]), p(se[i % len(se)]["up"]), TM * K * FM, F32)), reps)
     record("swiglu", f"qwen3-30b-a3b [{TM * K}x{FM}] f32", us, 3 * TM * K * FM * 4)
+    # MoE combine + residual + next norm: the expert down rows [8192 x 2048] folded back into [1024 x 2048]
+    del se
+    cb = pool(TM * K * HM * 4 + 3 * TM * HM * 4, lambda: dict(flat=randn((TM * K, HM), f32), x=randn((TM, HM), f32),
+                                                          h=torch.empty((TM, HM), dtype=f32, device=dev)))
+    gm = 1 + 0.05 * randn(HM, f32)
+    torch.cuda.synchronize()
+    us = timed(lambda i: check(L.apk_moe_combine_add_rmsnorm(h, p(cb[i % len(cb)]["x"]), p(cb[i % len(cb)]["flat"]), p(tok_off), p(hit_row),
+                                                             p(hit_w), TM * K, p(cb[i % len(cb)]["h"]), p(gm), HM, TM, EPS, F32)), reps)
+    record("moe_combine + add + rmsnorm (one launch)", tagm, us, TM * K * HM * 4 + 3 * TM * HM * 4 + HM * 4 + TM * K * 8)
+    del cb
+    # greedy pick over the vocabulary (after the output head): 1 and 64 rows of 151936 logits
+    V = synth.MODELS["qwen3-32b"]["vocab"]
+    lg = [randn((64, V), f32) for _ in range(17)]  # 17 x 38.9 MB
+    pick = torch.empty(64, dtype=i32, device=dev)
+    torch.cuda.synchronize()
+    for rows in (1, 64):
+        us = timed(lambda i: check(L.apk_argmax_rows(h, p(lg[i % 17]), rows, V, p(pick))), 200)
+        record("argmax_rows", f"{rows} x {V} logits f32", us, rows * V * 4 + rows * 4, note="launch-bound" if rows == 1 else None)
 
 
 def cpu_baseline(np, T, H, NQ, NKV, HD, FF, EPS):

@@ -228,6 +228,28 @@ int apk_gather_rows(apk_ctx* ctx, const void* src, const uint32_t* tok, size_t s
 int apk_scatter_rows(apk_ctx* ctx, const void* src, const uint32_t* hit_row, size_t rows, size_t k, size_t total_rows,
                      size_t cols, void* dst, int dtype);
 
+/* MoE combine + residual add + the next RMSNorm in one pass per token row:
+ *   out = 0; for each hit j in [tok_off[t], tok_off[t+1]): out = fma(flat[hit_row[j]], hit_w[j], out);
+ *   x[t] += out;  h[t] = rmsnorm(x[t]) * gamma.
+ * Replaces the per-token ops::add_scaled_slice loop of Ffn::moe_batch (model/moe.rs:298-333;
+ * ops/blas.rs:25-102, one fused multiply-add per hit), the residual ops::add_assign_slice
+ * (model/decode.rs:775, model/prefill.rs:308) and the next ops::rmsnorm_rows_into
+ * (model/prefill.rs:155/314); the reference's accelerators fuse the same three
+ * (combine_rows_resnorm, gpu/shaders/kernels.metal:1905-1974; GroupedCombine.next_norm,
+ * gpu/types.rs:429-443).  flat: [total_rows][n] expert down-projection rows of dtype;
+ * tok_off/hit_row/hit_w: the CSR lists of apk_moe_permute.  h (and gamma) may be NULL:
+ * combine and residual only.  A hit >= total_rows is skipped and raises APK_FAULT_ROW_RANGE. */
+int apk_moe_combine_add_rmsnorm(apk_ctx* ctx, void* x, const void* flat, const uint32_t* tok_off,
+                                const uint32_t* hit_row, const float* hit_w, size_t total_rows, void* h,
+                                const float* gamma, size_t n, size_t rows, float eps, int dtype);
+
+/* Greedy next token per row of logits: the LAST maximum under f32::total_cmp, exactly
+ * (0..n).max_by(|a, b| logits[a].total_cmp(&logits[b])) of Model::forward_greedy
+ * (model/decode.rs:628-630; ties -> higher index, as the reference's Metal argmax,
+ * gpu/shaders/kernels.metal:3726-3728).  logits: f32[rows][n]; out: u32[rows].
+ * Uses a small per-context scratch (128 bytes per row, allocated on first use). */
+int apk_argmax_rows(apk_ctx* ctx, const float* logits, size_t rows, size_t n, uint32_t* out);
+
 /* dst = src, `bytes` a multiple of 16: the plain stream kernel the bandwidth
  * figures of the other kernels are calibrated against. */
 int apk_copy(apk_ctx* ctx, const void* src, void* dst, size_t bytes);

@@ -83,6 +83,10 @@ def lib():
         L.ora_moe_group.argtypes = [vp, vp, sz, sz, sz, vp, vp, vp, vp, vp]
         L.ora_gather_rows.argtypes = [vp, vp, sz, sz, vp]
         L.ora_gather_rows_f16.argtypes = [vp, vp, sz, sz, vp]
+        L.ora_moe_combine_add_rmsnorm.argtypes = [vp, vp, vp, vp, vp, vp, vp, sz, sz, f32]
+        L.ora_moe_combine_add_rmsnorm_f16.argtypes = [vp, vp, vp, vp, vp, vp, vp, sz, sz, f32]
+        L.ora_argmax_last.restype = u32
+        L.ora_argmax_last.argtypes = [vp, sz]
         L.ora_kv_store_rows.argtypes = [vp, vp, sz, sz, vp, sz, vp, vp]
         L.ora_kv_store_rows_f16.argtypes = [vp, vp, sz, sz, vp, sz, vp, vp]
         L.ora_add_rmsnorm_rows.argtypes = [vp, vp, vp, vp, sz, sz, f32]
@@ -382,3 +386,16 @@ def kv_store_rows(k, v, pos, k_cache, v_cache):
     fn = lib().ora_kv_store_rows if k.dtype == np.float32 else lib().ora_kv_store_rows_f16
     if fn(_p(k), _p(v), rows, kv_dim, _p(pos), k_cache.shape[0], _p(k_cache), _p(v_cache)):
         raise OracleError("position past capacity")
+
+
+def moe_combine_add_rmsnorm(x, flat, tok_off, hit_row, hit_w, h, gamma, eps):
+    """x [rows, n] += weighted hits of flat [total_rows, n]; h = rmsnorm(x) * gamma (h may be None)."""
+    rows, n = x.shape
+    _chk(tok_off, np.uint32), _chk(hit_row, np.uint32), _chk(hit_w, np.float32)
+    fn = lib().ora_moe_combine_add_rmsnorm if x.dtype == np.float32 else lib().ora_moe_combine_add_rmsnorm_f16
+    fn(_p(x), _p(flat), _p(tok_off), _p(hit_row), _p(hit_w), _p(h), _p(gamma), n, rows, eps)
+
+
+def argmax_last(logits):
+    _chk(logits, np.float32)
+    return int(lib().ora_argmax_last(_p(logits), logits.size))

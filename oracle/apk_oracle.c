@@ -829,3 +829,52 @@ ORA_API int ora_kv_store_rows_f16(const uint16_t *k, const uint16_t *v, size_t r
     }
     return bad;
 }
+
+/* ------------------------------------------------- MoE combine + residual + norm
+ * Ffn::moe_batch combine (crates/allpaka-model/src/model/moe.rs:298-333): per token, out row
+ * starts at zero and gains every hit with ops::add_scaled_slice (fma(src, w, dst), blas.rs:25-102)
+ * in CSR order; the caller then does ops::add_assign_slice(x, out) (decode.rs:775) and the next
+ * ops::rmsnorm_into (prefill.rs:155/314).  h may be NULL (no norm). */
+ORA_API void ora_moe_combine_add_rmsnorm(float *x, const float *flat, const uint32_t *tok_off, const uint32_t *hit_row,
+                                         const float *hit_w, float *h, const float *gamma, size_t n, size_t rows, float eps) {
+    float *out = (float *)malloc(sizeof(float) * n);
+    for (size_t t = 0; t < rows; t++) {
+        for (size_t i = 0; i < n; i++) out[i] = 0.0f;
+        for (uint32_t k = tok_off[t]; k < tok_off[t + 1]; k++)
+            ora_add_scaled_slice(out, n, flat + (size_t)hit_row[k] * n, n, hit_w[k]);
+        ora_add_assign_slice(x + t * n, n, out, n);
+        if (h) ora_rmsnorm_into(h + t * n, x + t * n, gamma, n, eps);
+    }
+    free(out);
+}
+/* fp16 activations (build-defined): widen, the f32 arithmetic above, one RNE rounding of x and of h;
+ * the norm uses the unrounded sum, as ora_add_rmsnorm_rows_f16. */
+ORA_API void ora_moe_combine_add_rmsnorm_f16(uint16_t *x, const uint16_t *flat, const uint32_t *tok_off, const uint32_t *hit_row,
+                                             const float *hit_w, uint16_t *h, const float *gamma, size_t n, size_t rows, float eps) {
+    float *out = (float *)malloc(sizeof(float) * n), *v = (float *)malloc(sizeof(float) * n), *o = (float *)malloc(sizeof(float) * n);
+    for (size_t t = 0; t < rows; t++) {
+        for (size_t i = 0; i < n; i++) out[i] = 0.0f;
+        for (uint32_t k = tok_off[t]; k < tok_off[t + 1]; k++)
+            for (size_t i = 0; i < n; i++) out[i] = fmaf(ora_f16_to_f32(flat[(size_t)hit_row[k] * n + i]), hit_w[k], out[i]);
+        for (size_t i = 0; i < n; i++) {
+            v[i] = ora_f16_to_f32(x[t * n + i]) + out[i];
+            x[t * n + i] = ora_f32_to_f16(v[i]);
+        }
+        if (h) {
+            ora_rmsnorm_into(o, v, gamma, n, eps);
+            for (size_t i = 0; i < n; i++) h[t * n + i] = ora_f32_to_f16(o[i]);
+        }
+    }
+    free(out); free(v); free(o);
+}
+
+/* Model::forward_greedy's pick (crates/allpaka-model/src/model/decode.rs:628-630):
+ * (0..n).max_by(|a, b| logits[a].total_cmp(&logits[b])) -- Iterator::max_by keeps the LAST
+ * maximum, so ties go to the higher index; empty -> 0. */
+ORA_API uint32_t ora_argmax_last(const float *logits, size_t n) {
+    if (n == 0) return 0;
+    size_t best = 0;
+    for (size_t i = 1; i < n; i++)
+        if (total_key(logits[i]) >= total_key(logits[best])) best = i;
+    return (uint32_t)best;
+}

@@ -684,3 +684,43 @@ def test_kv_store_rows_narrows_with_rne_at_the_right_rows(ora):
     kc2, vc2 = np.zeros_like(kc), np.zeros_like(vc)
     ora.kv_store_rows(kh, vh, [5, 0, 7], kc2, vc2)
     assert np.array_equal(kc2, kc) and np.array_equal(vc2, vc)
+
+
+def test_argmax_is_rusts_max_by_last_wins(ora):
+    # Iterator::max_by returns the last element among equal maxima (decode.rs:628-630)
+    assert ora.argmax_last(np.float32([1, 5, 3, 5, 2])) == 3
+    assert ora.argmax_last(np.float32([7])) == 0
+    assert ora.argmax_last(np.float32([-np.inf, -np.inf])) == 1
+    assert ora.argmax_last(np.float32([0.0, -0.0])) == 0  # total_cmp: -0 < +0
+    assert ora.argmax_last(np.float32([1.0, np.nan, 2.0])) == 1  # total_cmp puts +NaN above everything
+    rng = np.random.default_rng(31)
+    for _ in range(20):
+        x = rng.standard_normal(1000).astype(np.float32)
+        assert ora.argmax_last(x) == len(x) - 1 - int(np.argmax(x[::-1]))
+
+
+def test_moe_combine_is_fma_in_hit_order_then_residual_then_norm(ora):
+    rng = np.random.default_rng(37)
+    rows, k, ne, n = 9, 3, 6, 64
+    logits = rng.standard_normal((rows, ne)).astype(np.float32)
+    ids, w = ora.route_rows(logits, k)
+    table, tok, tok_off, hit_row, hit_w = ora.moe_group(ids, w, ne)
+    flat = rng.standard_normal((rows * k, n)).astype(np.float32)
+    x = rng.standard_normal((rows, n)).astype(np.float32)
+    gamma = rng.standard_normal(n).astype(np.float32)
+    x2, h2 = x.copy(), np.zeros_like(x)
+    ora.moe_combine_add_rmsnorm(x2, flat, tok_off, hit_row, hit_w, h2, gamma, 1e-6)
+    for t in range(rows):
+        out = np.zeros(n, np.float64)
+        acc = np.zeros(n, np.float32)
+        for j in range(tok_off[t], tok_off[t + 1]):
+            # one rounding per hit: fma(src, w, acc)
+            acc = (flat[hit_row[j]].astype(np.float64) * np.float64(hit_w[j]) + acc.astype(np.float64)).astype(np.float32)
+        want_x = x[t] + acc
+        assert np.array_equal(x2[t], want_x)
+        hh = np.zeros(n, np.float32)
+        ora.rmsnorm_into(hh, want_x.copy(), gamma, 1e-6)
+        assert np.array_equal(h2[t], hh)
+    x3 = x.copy()
+    ora.moe_combine_add_rmsnorm(x3, flat, tok_off, hit_row, hit_w, None, None, 1e-6)
+    assert np.array_equal(x3, x2)
