@@ -86,6 +86,45 @@ template <> struct io<f16_t> {
     DEV void store_nt(f16_t* p, const float* v) { __builtin_nontemporal_store(pack(v), (u32x4*)p); }
 };
 
+// ------------------------------------------------------- wave reductions (DPP)
+// Butterfly exchanges inside a 16-lane row as DPP modifiers (no LDS round trip):
+// lane^1 and lane^2 by quad permutes, then row_half_mirror (i <-> 7-i) and row_mirror
+// (i <-> 15-i): after step s every lane of a 2^s group holds the group's reduction, so
+// mirroring pairs each lane with one of the other half-group.  Across rows: readlane.
+#define DPP_XOR1 0xB1         // quad_perm:[1,0,3,2]
+#define DPP_XOR2 0x4E         // quad_perm:[2,3,0,1]
+#define DPP_HALF_MIRROR 0x141 // row_half_mirror
+#define DPP_MIRROR 0x140      // row_mirror
+template <int CTRL> DEV float dpp_f32(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+template <int CTRL> DEV double dpp_f64(double v) {
+    const uint64_t b = __builtin_bit_cast(uint64_t, v);
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_mov_dpp((int)(uint32_t)b, CTRL, 0xf, 0xf, true);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_mov_dpp((int)(uint32_t)(b >> 32), CTRL, 0xf, 0xf, true);
+    return __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);
+}
+template <int CTRL> DEV uint64_t dpp_u64(uint64_t b) {
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_mov_dpp((int)(uint32_t)b, CTRL, 0xf, 0xf, true);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_mov_dpp((int)(uint32_t)(b >> 32), CTRL, 0xf, 0xf, true);
+    return ((uint64_t)hi << 32) | lo;
+}
+DEV float dpp_step(float v, int s) {
+    return s == 0 ? dpp_f32<DPP_XOR1>(v) : s == 1 ? dpp_f32<DPP_XOR2>(v) : s == 2 ? dpp_f32<DPP_HALF_MIRROR>(v) : dpp_f32<DPP_MIRROR>(v);
+}
+DEV double dpp_step(double v, int s) {
+    return s == 0 ? dpp_f64<DPP_XOR1>(v) : s == 1 ? dpp_f64<DPP_XOR2>(v) : s == 2 ? dpp_f64<DPP_HALF_MIRROR>(v) : dpp_f64<DPP_MIRROR>(v);
+}
+// Sum over aligned groups of WIDTH lanes (4, 8, 16, 32 or 64); every lane gets the sum.
+template <int WIDTH, typename A> DEV A group_sum(A v) {
+#pragma unroll
+    for (int s = 0; s < 4; s++)
+        if ((1 << (s + 1)) <= WIDTH) v += dpp_step(v, s);
+    if (WIDTH >= 32) v += __shfl_xor(v, 16, 64);
+    if (WIDTH >= 64) v += __shfl_xor(v, 32, 64);
+    return v;
+}
+
 // One tile of activations narrowed to fp16 (RNE) for the KV cache: 16 bytes from an
 // fp16 tile, 8 bytes from an f32 tile.
 template <typename T> DEV void store_f16_tile(f16_t* p, const float* v);
@@ -97,25 +136,26 @@ template <> __device__ __forceinline__ void store_f16_tile<float>(f16_t* p, cons
     __builtin_nontemporal_store(t, (u32x2*)p);
 }
 
-DEV double wave_sum_f64(double v, int width) {
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1)
-        if (o < width) v += __shfl_xor(v, o, 64);
-    return v;
-}
 
 DEV uint32_t total_order_key(float f) {  // f32::total_cmp as an unsigned key
     int32_t b = __builtin_bit_cast(int32_t, f);
     b ^= (int32_t)(((uint32_t)(b >> 31)) >> 1);
     return (uint32_t)b ^ 0x80000000u;
 }
-DEV uint64_t wave_max_u64(uint64_t v) {
+DEV uint64_t max_u64(uint64_t a, uint64_t b) { return a > b ? a : b; }
+DEV uint64_t wave_max_u64(uint64_t v) {  // every lane gets the maximum
+    v = max_u64(v, dpp_u64<DPP_XOR1>(v));
+    v = max_u64(v, dpp_u64<DPP_XOR2>(v));
+    v = max_u64(v, dpp_u64<DPP_HALF_MIRROR>(v));
+    v = max_u64(v, dpp_u64<DPP_MIRROR>(v));  // uniform inside each 16-lane row
+    uint64_t r = 0;
 #pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-        uint64_t other = __shfl_xor(v, o, 64);
-        v = other > v ? other : v;
+    for (int row = 0; row < 4; row++) {
+        const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, row * 16);
+        const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), row * 16);
+        r = max_u64(r, ((uint64_t)hi << 32) | lo);
     }
-    return v;
+    return r;
 }
 
 // =========================================================================
@@ -187,18 +227,14 @@ template <typename T> struct stat;
 template <> struct stat<float> {
     typedef double acc_t;
     DEV double sq(double a, float v) { return __builtin_fma((double)v, (double)v, a); }
-    DEV double wave_sum(double v) { return wave_sum_f64(v, 64); }
+    DEV double wave_sum(double v) { return group_sum<64>(v); }
     DEV double rscale(double ss, int n, float eps) { return 1.0 / sqrt(ss / (double)n + (double)eps); }
     DEV float apply(float v, double scale, float g) { return (float)((double)v * scale) * g; }
 };
 template <> struct stat<f16_t> {
     typedef float acc_t;
     DEV float sq(float a, float v) { return __builtin_fmaf(v, v, a); }
-    DEV float wave_sum(float v) {
-#pragma unroll
-        for (int o = 1; o < 64; o <<= 1) v += __shfl_xor(v, o, 64);
-        return v;
-    }
+    DEV float wave_sum(float v) { return group_sum<64>(v); }
     DEV float rscale(float ss, int n, float eps) { return __builtin_amdgcn_rsqf(ss * (1.0f / (float)n) + eps); }
     DEV float apply(float v, float scale, float g) { return v * scale * g; }
 };
@@ -539,8 +575,7 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
             ss = stat<T>::sq(ss, a[i]);
             ss = stat<T>::sq(ss, b[i]);
         }
-#pragma unroll
-        for (int o = 1; o < LPH; o <<= 1) ss += __shfl_xor(ss, o, 64);
+        ss = group_sum<LPH>(ss);
         const acc_t scale = stat<T>::rscale(ss, HD, eps);
         if constexpr (sizeof(T) == 2) {
             const float sf = normed ? (float)scale : 1.0f;
@@ -995,14 +1030,11 @@ APK_EMBED_GEN(f16, 7) APK_EMBED_GEN(f32, 8) APK_EMBED_GEN(bf16, 9)
 // =========================================================================
 DEV float wave_max_f32(float v) {
 #pragma unroll
-    for (int o = 1; o < 64; o <<= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-    return v;
+    for (int s = 0; s < 4; s++) v = fmaxf(v, dpp_step(v, s));
+    v = fmaxf(v, __shfl_xor(v, 16, 64));
+    return fmaxf(v, __shfl_xor(v, 32, 64));
 }
-DEV float wave_sum_f32(float v) {
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) v += __shfl_xor(v, o, 64);
-    return v;
-}
+DEV float wave_sum_f32(float v) { return group_sum<64>(v); }
 extern "C" __global__ __launch_bounds__(256) void apk_route_topk(const float* logits, const float* bias, int rows,
                                                                 int n_expert, int k, int norm, float scale,
                                                                 int sigmoid, uint32_t* ids, float* wout) {
@@ -1013,10 +1045,13 @@ extern "C" __global__ __launch_bounds__(256) void apk_route_topk(const float* lo
     float lg[4], score[4];
     uint32_t key[4];
     float mx = -INFINITY;
+    float raw[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) raw[j] = lr[min(lane + 64 * j, n_expert - 1)];  // all four loads in flight, no branch
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         const int e = lane + 64 * j;
-        lg[j] = e < n_expert ? lr[e] : -INFINITY;
+        lg[j] = e < n_expert ? raw[j] : -INFINITY;
         if (e < n_expert) mx = fmaxf(mx, lg[j]);
     }
     if (!sigmoid) {
@@ -1098,27 +1133,62 @@ extern "C" __global__ __launch_bounds__(APK_PERMUTE_THREADS) void apk_moe_permut
     const uint32_t* ids, const float* w, int rows, int k, int n_expert, uint32_t* table, uint32_t* n_used_out,
     uint32_t* tok, uint32_t* tok_off, uint32_t* hit_row, float* hit_w, uint32_t* fault) {
     __shared__ uint32_t hist[1024];
-    __shared__ uint32_t wave_tot[APK_PERMUTE_THREADS / 64];
+    __shared__ uint32_t wave_tot[APK_PERMUTE_THREADS / 64], wave_used[APK_PERMUTE_THREADS / 64];
     __shared__ uint32_t s_row0, s_used;
     const int e = blockIdx.x;
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     for (int i = tid; i < n_expert; i += blockDim.x) hist[i] = 0;
     __syncthreads();
     const int total = rows * k;
-    for (int i = tid; i < total; i += blockDim.x) {
-        const uint32_t id = ids[i];
+    auto count = [&](uint32_t id) {
         if (id < (uint32_t)n_expert) atomicAdd(&hist[id], 1u);
         else if (e == 0) atomicOr(fault, APK_FAULT_EXPERT_RANGE);
+    };
+    {   // 16-byte loads, four in flight per lane (the ids sit in L2; one dependent load per
+        // pick would serialise a hit latency per iteration)
+        const int nvec = total >> 2;
+        const u32x4* ids4 = (const u32x4*)ids;
+        for (int base = 0; base < nvec; base += 4 * blockDim.x) {
+            u32x4 v[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) v[j] = ids4[min(base + tid + j * (int)blockDim.x, nvec - 1)];
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                if (base + tid + j * (int)blockDim.x < nvec) {
+                    count(v[j].x);
+                    count(v[j].y);
+                    count(v[j].z);
+                    count(v[j].w);
+                }
+        }
+        for (int i = (nvec << 2) + tid; i < total; i += blockDim.x) count(ids[i]);
     }
     __syncthreads();
-    if (tid == 0) {
+    {  // row0 = picks of lower experts, s_used = non-empty lower experts: a workgroup sum, not a serial walk
         uint32_t r0 = 0, used = 0;
-        for (int i = 0; i < e; i++) {
+        for (int i = tid; i < e; i += blockDim.x) {
             r0 += hist[i];
             used += hist[i] != 0;
         }
-        s_row0 = r0;
-        s_used = used;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            r0 += __shfl_xor(r0, o, 64);
+            used += __shfl_xor(used, o, 64);
+        }
+        if (lane == 0) {
+            wave_tot[wv] = r0;
+            wave_used[wv] = used;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            uint32_t a = 0, b = 0;
+            for (int i = 0; i < (int)(blockDim.x >> 6); i++) {
+                a += wave_tot[i];
+                b += wave_used[i];
+            }
+            s_row0 = a;
+            s_used = b;
+        }
     }
     __syncthreads();
     const uint32_t row0 = s_row0, mine = hist[e];
@@ -1138,8 +1208,21 @@ extern "C" __global__ __launch_bounds__(APK_PERMUTE_THREADS) void apk_moe_permut
         const int t = base + tid;
         int j_hit = -1, slot = 0;
         if (t < rows) {
-            for (int j = 0; j < k; j++) {
-                const uint32_t id = ids[(uint64_t)t * k + j];
+            const uint32_t* mine_ids = ids + (uint64_t)t * k;
+            int j = 0;
+            if ((k & 3) == 0) {  // rows of picks are 16-byte aligned: two tiles in flight
+                for (; j + 8 <= k; j += 8) {
+                    const u32x4 a = *(const u32x4*)(mine_ids + j), b = *(const u32x4*)(mine_ids + j + 4);
+                    const uint32_t v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        if (v[i] == (uint32_t)e && j_hit < 0) j_hit = j + i;
+                        slot += v[i] < (uint32_t)e;
+                    }
+                }
+            }
+            for (; j < k; j++) {
+                const uint32_t id = mine_ids[j];
                 if (id == (uint32_t)e && j_hit < 0) j_hit = j;
                 slot += id < (uint32_t)e;
             }

@@ -75,16 +75,20 @@ def main():
     def sync():
         apklib.check(L.apk_sync(h))
 
-    def timed(fn, reps):
-        """avg microseconds per call of fn(i): HIP events on the library's stream, after 3 untimed calls"""
+    def timed(fn, reps, batches=3):
+        """microseconds per call of fn(i): HIP events on the library's stream around `reps` back-to-back
+        launches, after 3 untimed calls; the median of `batches` such averages"""
         for i in range(3):
             fn(i)
         ms = C.c_float()
-        apklib.check(L.apk_timer_begin(h))
-        for i in range(reps):
-            fn(i + 3)
-        apklib.check(L.apk_timer_end(h, C.byref(ms)))
-        return ms.value * 1000.0 / reps
+        avgs = []
+        for bi in range(batches):
+            apklib.check(L.apk_timer_begin(h))
+            for i in range(reps):
+                fn(3 + bi * reps + i)
+            apklib.check(L.apk_timer_end(h, C.byref(ms)))
+            avgs.append(ms.value * 1000.0 / reps)
+        return sorted(avgs)[len(avgs) // 2]
 
     per_op = []
 
