@@ -64,7 +64,7 @@ const int kQkHeadDims[] = {64, 128, 256};
 std::vector<std::string> all_kernel_names() {
     std::vector<std::string> v = {"apk_swiglu_f32", "apk_swiglu_f16", "apk_rope_table", "apk_embed_q4k_f32",
                                   "apk_embed_q4k_f16", "apk_embed_q8_0_f32", "apk_embed_q8_0_f16", "apk_route_topk",
-                                  "apk_moe_permute", "apk_gather_rows", "apk_scatter_rows", "apk_argmax_rows", "apk_copy"};
+                                  "apk_moe_permute", "apk_gather_rows", "apk_scatter_rows", "apk_argmax_rows", "apk_add_rmsnorm_ragged_f32", "apk_copy"};
     for (const char* t : {"f32", "f16"}) {
         for (const char* f : {"q5k", "q6k", "q2k", "q3k", "q5_0", "f16", "f32", "bf16"}) v.push_back(std::string("apk_embed_") + f + "_" + t);
         for (int c : kAddnormTiles) v.push_back(std::string("apk_add_rmsnorm_") + t + "_c" + std::to_string(c));
@@ -368,10 +368,19 @@ int apk_add_rmsnorm_rows(apk_ctx* c, void* x, const void* delta, void* h, const 
     if (rows == 0) return APK_OK;
     if (!x || !h || !gamma) return fail(APK_DECLINE_NULL, "apk_add_rmsnorm_rows: NULL tensor");
     const size_t vec = 16 / es;
-    if (n == 0 || n % vec) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: n=%zu is not a multiple of %zu", n, vec);
+    if (rows > 0x7fffffffu || n > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: too large");
+    if (n == 0) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: n is 0");
+    if (n % vec) {
+        // rows that are not whole 16-byte tiles: f32 has an element-wise path, fp16 declines
+        if (dtype != APK_F32) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: n=%zu is not a multiple of %zu", n, vec);
+        if (h == x && delta) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: h aliases x while delta is given");
+        if (int rc = set_device(c)) return rc;
+        int n_r = (int)n;
+        void* rargs[] = {&x, &delta, &h, &gamma, &n_r, &eps};
+        return launch(c, "apk_add_rmsnorm_ragged_f32", (unsigned)rows, 256, 0, rargs);
+    }
     if (!aligned16(x) || !aligned16(h) || !aligned16(gamma) || (delta && !aligned16(delta)))
         return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: tensors must be 16-byte aligned");
-    if (rows > 0x7fffffffu || n > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: too large");
     const size_t nchunks = n / vec;
     // Tiles per lane (NCH) and waves per row (W = ceil(nchunks / (64*NCH))): the first
     // choice that keeps the whole batch resident in one round (rows * W <= 2048 waves,

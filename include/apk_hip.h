@@ -137,7 +137,8 @@ int apk_embed_rows_host_ids(apk_ctx* ctx, int fmt, const void* table, size_t voc
  * ops::rmsnorm_into / rmsnorm_rows_into (ops/blas.rs:105-178, ops/norm.rs:193-304;
  * call sites model/decode.rs:584,764, model/prefill.rs:155,308-314).
  * x, delta, h: [rows][n] of dtype (h may alias x when delta is NULL);
- * gamma: f32[n].  n must be a multiple of 4 (f32) / 8 (f16). */
+ * gamma: f32[n].  fp16 rows must be a multiple of 8 elements; f32 rows of any length are
+ * taken (a multiple of 4 takes the fast 16-byte-tile path). */
 int apk_add_rmsnorm_rows(apk_ctx* ctx, void* x, const void* delta, void* h, const float* gamma, size_t n,
                          size_t rows, float eps, int dtype);
 
