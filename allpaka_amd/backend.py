@@ -10,6 +10,7 @@ Tensors are torch CUDA tensors (float32, or float16 for the fp16 activation
 form); every op runs in place where the reference's does.
 """
 import ctypes as C
+import contextlib
 import enum
 
 import torch
@@ -62,6 +63,7 @@ class Backend:
         check(self.L.apk_init(device, C.byref(h)))
         self.h = h
         self.device = torch.device("cuda", device)
+        self._recording = False
 
     def close(self):
         if self.h:
@@ -92,6 +94,40 @@ class Backend:
         # torch owns the buffers and fills them on its own stream
         torch.cuda.current_stream(self.device).synchronize()
 
+    def _leave(self):
+        # the mirrored ops return with their result in place, like the CPU ops they stand
+        # for; inside a recording nothing runs, so there is nothing to wait for
+        if not self._recording:
+            self.sync()
+
+    # ---- record / replay (stream capture of gpu/cuda/prefill.rs:52-108)
+    def capture_begin(self):
+        self._enter()
+        check(self.L.apk_capture_begin(self.h))
+        self._recording = True
+
+    def capture_end(self):
+        g = C.c_void_p()
+        self._recording = False
+        check(self.L.apk_capture_end(self.h, C.byref(g)))
+        return Graph(self, g)
+
+    def capture_abort(self):
+        self._recording = False
+        check(self.L.apk_capture_abort(self.h))
+
+    @contextlib.contextmanager
+    def record(self):
+        """`with be.record() as rec: <ops>` -> `rec.graph` replays them with one submission."""
+        rec = _Recording()
+        self.capture_begin()
+        try:
+            yield rec
+        except BaseException:
+            self.capture_abort()
+            raise
+        rec.graph = self.capture_end()
+
     # ---- ops::* (crates/allpaka-backend/src/ops)
     def rmsnorm(self, x, weight, eps):
         """ops::rmsnorm (norm.rs:115): in place over ONE row."""
@@ -111,7 +147,7 @@ class Backend:
         assert dst.numel() >= rows * n, "dst holds fewer rows than src"
         self._enter()
         check(self.L.apk_add_rmsnorm_rows(self.h, _ptr(src), None, _ptr(dst), _ptr(weight), n, rows, eps, _dt(src)))
-        self.sync()
+        self._leave()
 
     def add_assign_slice(self, a, b):
         """ops::add_assign_slice (blas.rs:105) -- on the device this op only exists
@@ -136,7 +172,7 @@ class Backend:
         assert gamma.dtype == torch.float32
         self._enter()
         check(self.L.apk_add_rmsnorm_rows(self.h, _ptr(x), _ptr(delta), _ptr(h), _ptr(gamma), n, rows, eps, _dt(x)))
-        self.sync()
+        self._leave()
 
     def rope_table(self, positions, inv_freq):
         """ops::rope_sin_cos per position -> [rows, half, 2] = [sin, cos] (rope.rs:18-22)."""
@@ -145,7 +181,7 @@ class Backend:
         table = torch.empty((rows, half, 2), dtype=torch.float32, device=self.device)
         self._enter()
         check(self.L.apk_rope_table(self.h, _ptr(positions), _ptr(inv_freq), rows, half, _ptr(table)))
-        self.sync()
+        self._leave()
         return table
 
     def qknorm_rope_neox(self, q, k, q_norm, k_norm, rope_flat, n_q, n_kv, head_dim, eps, rot_dim=None):
@@ -161,7 +197,7 @@ class Backend:
         self._enter()
         check(self.L.apk_qknorm_rope_neox(self.h, _ptr(q), _ptr(k), _ptr(q_norm), _ptr(k_norm), _ptr(rope_flat), rows,
                                           n_q, n_kv, head_dim, rot, eps, _dt(q)))
-        self.sync()
+        self._leave()
 
     def qknorm_rope_kv_store(self, q, k, v, q_norm, k_norm, rope_flat, cache_pos, k_cache, v_cache, n_q, n_kv, head_dim, eps):
         """qknorm_rope_neox, then KvCache::store_at of every row's k and v as f16 at cache row
@@ -175,7 +211,7 @@ class Backend:
         check(self.L.apk_qknorm_rope_kv_store(self.h, _ptr(q), _ptr(k), _ptr(v), _ptr(q_norm), _ptr(k_norm), _ptr(rope_flat),
                                               _ptr(cache_pos), _ptr(k_cache), _ptr(v_cache), k_cache.shape[0], rows, n_q, n_kv,
                                               head_dim, head_dim, eps, _dt(q)))
-        self.sync()
+        self._leave()
         if self.take_faults() & _l.FAULT_CACHE_RANGE:
             raise AssertionError("position past capacity")
 
@@ -190,7 +226,7 @@ class Backend:
         self._enter()
         check(self.L.apk_layer_prologue(self.h, _ptr(x), _ptr(delta), _ptr(h), _ptr(gamma), n, _ptr(q), _ptr(k), _ptr(q_norm),
                                         _ptr(k_norm), _ptr(rope_flat), rows, n_q, n_kv, head_dim, head_dim, eps, _dt(x)))
-        self.sync()
+        self._leave()
 
     def rope_neox_cached_from_array(self, x, table):
         """ops::rope_neox_cached_from_array (rope.rs:70) on one head."""
@@ -203,7 +239,7 @@ class Backend:
         assert gate.dtype == up.dtype
         self._enter()
         check(self.L.apk_swiglu(self.h, _ptr(gate), _ptr(up), gate.numel(), _dt(gate)))
-        self.sync()
+        self._leave()
 
     # ---- model::route_gated (crates/allpaka-model/src/model/moe.rs:601)
     def route_rows(self, logits, k, gating=Gating.Softmax, norm=True, scale=1.0, bias=None):
@@ -218,7 +254,7 @@ class Backend:
         self._enter()
         check(self.L.apk_route_topk(self.h, _ptr(logits), _ptr(bias), rows, n, k, int(norm), scale,
                                     int(gating == Gating.Sigmoid), _ptr(ids), _ptr(w)))
-        self.sync()
+        self._leave()
         return ids, w
 
     def route_gated(self, logits, k, gating=Gating.Softmax, norm=True, scale=1.0, bias=None):
@@ -239,7 +275,7 @@ class Backend:
         self._enter()
         check(self.L.apk_moe_permute(self.h, _ptr(ids), _ptr(w), rows, k, n_expert, _ptr(table), _ptr(n_used), _ptr(tok),
                                      _ptr(tok_off), _ptr(hit_row), _ptr(hit_w)))
-        self.sync()
+        self._leave()
         return table[: int(n_used.item())], tok, tok_off, hit_row, hit_w
 
     def gather_rows(self, src, tok):
@@ -248,7 +284,7 @@ class Backend:
         dst = torch.empty((total, src.shape[1]), dtype=src.dtype, device=self.device)
         self._enter()
         check(self.L.apk_gather_rows(self.h, _ptr(src), _ptr(tok), src.shape[0], total, src.shape[1], _ptr(dst), _dt(src)))
-        self.sync()
+        self._leave()
         return dst
 
     def scatter_rows(self, src, hit_row, k):
@@ -258,7 +294,7 @@ class Backend:
         dst = torch.empty((total, src.shape[1]), dtype=src.dtype, device=self.device)
         self._enter()
         check(self.L.apk_scatter_rows(self.h, _ptr(src), _ptr(hit_row), rows, k, total, src.shape[1], _ptr(dst), _dt(src)))
-        self.sync()
+        self._leave()
         return dst
 
     def moe_combine_add_rmsnorm(self, x, flat, tok_off, hit_row, hit_w, h, gamma, eps):
@@ -271,17 +307,47 @@ class Backend:
         self._enter()
         check(self.L.apk_moe_combine_add_rmsnorm(self.h, _ptr(x), _ptr(flat), _ptr(tok_off), _ptr(hit_row), _ptr(hit_w),
                                                  flat.shape[0], _ptr(h), _ptr(gamma), n, rows, eps, _dt(x)))
-        self.sync()
+        self._leave()
 
     def argmax_rows(self, logits):
         """Greedy pick per row: (0..n).max_by(total_cmp) of forward_greedy (decode.rs:628-630)."""
+        out = torch.empty(logits.shape[0], dtype=torch.int32, device=self.device)
+        self.argmax_rows_into(logits, out)
+        self._leave()
+        return out
+
+    def argmax_rows_into(self, logits, out):
+        """The same into a caller's int32 tensor, enqueued only (no wait)."""
         rows, n = logits.shape
-        assert logits.dtype == torch.float32
-        out = torch.empty(rows, dtype=torch.int32, device=self.device)
+        assert logits.dtype == torch.float32 and out.dtype == torch.int32 and out.numel() >= rows
         self._enter()
         check(self.L.apk_argmax_rows(self.h, _ptr(logits), rows, n, _ptr(out)))
-        self.sync()
-        return out
+
+
+class _Recording:
+    graph = None
+
+
+class Graph:
+    """A recorded chain of ops (`apk_graph`); every pointer and size is baked in, so the
+    tensors the ops were recorded with must stay alive and in place."""
+
+    def __init__(self, backend, handle):
+        self.be, self.g = backend, handle
+
+    @property
+    def nodes(self):
+        n = C.c_size_t()
+        check(self.be.L.apk_graph_nodes(self.g, C.byref(n)))
+        return n.value
+
+    def launch(self):
+        check(self.be.L.apk_graph_launch(self.be.h, self.g))
+
+    def destroy(self):
+        if self.g:
+            check(self.be.L.apk_graph_destroy(self.be.h, self.g))
+            self.g = None
 
 
 class QuantMat:

@@ -93,9 +93,20 @@ struct apk_ctx {
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     void* argmax_scratch = nullptr;  // one 128-byte line per row: u64 running best + u32 arrivals; zero between calls
     size_t argmax_rows_cap = 0;
+    bool capturing = false;        // between apk_capture_begin and apk_capture_end / _abort
+    size_t capture_nodes = 0;      // launches recorded so far
+    bool capture_argmax = false;   // the recording holds the argmax scratch address
+    size_t graphs_with_argmax = 0; // live graphs that do: the scratch must not move under them
     std::mutex mu;
     std::map<uintptr_t, Mapping> attached;
     std::atomic<uint64_t> calls{0}, dispatches{0}, encode_ns{0}, wait_ns{0};
+};
+
+struct apk_graph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    size_t nodes = 0;
+    bool uses_argmax = false;
 };
 
 namespace {
@@ -114,9 +125,16 @@ int launch(apk_ctx* c, const std::string& k, unsigned grid, unsigned block, unsi
     if (it == c->fn.end()) return fail(APK_DECLINE_UNSUPPORTED, "no kernel %s in the code object", k.c_str());
     hipError_t e = hipModuleLaunchKernel(it->second, grid, 1, 1, block, 1, 1, shmem, c->stream, args, nullptr);
     if (e != hipSuccess) return hip_fail(e, k.c_str());
-    c->dispatches++;
+    if (c->capturing) c->capture_nodes++;  // recorded, not run: counted when the graph is replayed
+    else c->dispatches++;
     return APK_OK;
 }
+
+// Entries that allocate, copy to or from the host, or wait cannot run inside a recording.
+#define NOT_WHILE_CAPTURING(c, name)                                                              \
+    do {                                                                                          \
+        if ((c)->capturing) return fail(APK_DECLINE_CAPTURE, name ": not possible while recording"); \
+    } while (0)
 
 bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 int elem_size(int dtype) { return dtype == APK_F32 ? 4 : (dtype == APK_F16 ? 2 : 0); }
@@ -197,6 +215,12 @@ int apk_init(int device, apk_ctx** out) {
 int apk_shutdown(apk_ctx* c) {
     if (!c) return APK_OK;
     (void)hipSetDevice(c->device);
+    if (c->capturing) {
+        hipGraph_t g = nullptr;
+        (void)hipStreamEndCapture(c->stream, &g);
+        if (g) (void)hipGraphDestroy(g);
+        c->capturing = false;
+    }
     if (c->stream) (void)hipStreamSynchronize(c->stream);
     for (auto& kv : c->attached) (void)hipFree(kv.second.dev);
     if (c->ids_stage_dev) (void)hipFree(c->ids_stage_dev);
@@ -214,6 +238,7 @@ int apk_shutdown(apk_ctx* c) {
 int apk_sync(apk_ctx* c) {
     if (!c) return fail(APK_DECLINE_NULL, "apk_sync: ctx is NULL");
     std::lock_guard<std::mutex> lock(c->mu);
+    NOT_WHILE_CAPTURING(c, "apk_sync");
     uint64_t t0 = now_ns();
     hipError_t e = hipStreamSynchronize(c->stream);
     c->wait_ns += now_ns() - t0;
@@ -235,6 +260,7 @@ int apk_stats(apk_ctx* c, uint64_t* calls, uint64_t* dispatches, uint64_t* encod
 int apk_take_faults(apk_ctx* c, uint32_t* faults) {
     if (!c || !faults) return fail(APK_DECLINE_NULL, "apk_take_faults: NULL argument");
     std::lock_guard<std::mutex> lock(c->mu);
+    NOT_WHILE_CAPTURING(c, "apk_take_faults");
     if (int rc = set_device(c)) return rc;
     uint32_t v = 0;
     HIP_TRY(hipMemcpyAsync(&v, c->fault_dev, 4, hipMemcpyDeviceToHost, c->stream));
@@ -252,6 +278,7 @@ int apk_take_faults(apk_ctx* c, uint32_t* faults) {
 int apk_malloc(apk_ctx* c, size_t bytes, void** dev_out) {
     if (!c || !dev_out) return fail(APK_DECLINE_NULL, "apk_malloc: NULL argument");
     std::lock_guard<std::mutex> lock(c->mu);
+    NOT_WHILE_CAPTURING(c, "apk_malloc");
     if (int rc = set_device(c)) return rc;
     HIP_TRY(hipMalloc(dev_out, bytes ? bytes : 16));
     return APK_OK;
@@ -259,6 +286,7 @@ int apk_malloc(apk_ctx* c, size_t bytes, void** dev_out) {
 int apk_free(apk_ctx* c, void* dev) {
     if (!c) return fail(APK_DECLINE_NULL, "apk_free: ctx is NULL");
     std::lock_guard<std::mutex> lock(c->mu);
+    NOT_WHILE_CAPTURING(c, "apk_free");
     if (int rc = set_device(c)) return rc;
     HIP_TRY(hipStreamSynchronize(c->stream));
     HIP_TRY(hipFree(dev));
@@ -267,6 +295,7 @@ int apk_free(apk_ctx* c, void* dev) {
 int apk_h2d(apk_ctx* c, void* dev_dst, const void* host_src, size_t bytes) {
     if (!c || (bytes && (!dev_dst || !host_src))) return fail(APK_DECLINE_NULL, "apk_h2d: NULL argument");
     CallScope s(c);
+    NOT_WHILE_CAPTURING(c, "apk_h2d");
     if (int rc = set_device(c)) return rc;
     if (bytes) HIP_TRY(hipMemcpyAsync(dev_dst, host_src, bytes, hipMemcpyHostToDevice, c->stream));
     return APK_OK;
@@ -274,6 +303,7 @@ int apk_h2d(apk_ctx* c, void* dev_dst, const void* host_src, size_t bytes) {
 int apk_d2h(apk_ctx* c, void* host_dst, const void* dev_src, size_t bytes) {
     if (!c || (bytes && (!host_dst || !dev_src))) return fail(APK_DECLINE_NULL, "apk_d2h: NULL argument");
     CallScope s(c);
+    NOT_WHILE_CAPTURING(c, "apk_d2h");
     if (int rc = set_device(c)) return rc;
     if (bytes) HIP_TRY(hipMemcpyAsync(host_dst, dev_src, bytes, hipMemcpyDeviceToHost, c->stream));
     return APK_OK;
@@ -282,6 +312,7 @@ int apk_d2h(apk_ctx* c, void* host_dst, const void* dev_src, size_t bytes) {
 int apk_attach(apk_ctx* c, const void* host_base, size_t len) {
     if (!c || !host_base || !len) return fail(APK_DECLINE_NULL, "apk_attach: NULL or empty mapping");
     std::lock_guard<std::mutex> lock(c->mu);
+    NOT_WHILE_CAPTURING(c, "apk_attach");
     if (int rc = set_device(c)) return rc;
     if (c->attached.count((uintptr_t)host_base)) return APK_OK;  // already resident
     void* dev = nullptr;
@@ -297,6 +328,7 @@ int apk_attach(apk_ctx* c, const void* host_base, size_t len) {
 int apk_detach(apk_ctx* c, const void* host_base) {
     if (!c) return fail(APK_DECLINE_NULL, "apk_detach: ctx is NULL");
     std::lock_guard<std::mutex> lock(c->mu);
+    NOT_WHILE_CAPTURING(c, "apk_detach");
     auto it = c->attached.find((uintptr_t)host_base);
     if (it == c->attached.end()) return fail(APK_DECLINE_NOT_ATTACHED, "apk_detach: mapping is not attached");
     if (int rc = set_device(c)) return rc;
@@ -324,17 +356,107 @@ int apk_resolve(apk_ctx* c, const void* host_ptr, size_t len, void** dev_out) {
 int apk_timer_begin(apk_ctx* c) {
     if (!c) return fail(APK_DECLINE_NULL, "apk_timer_begin: ctx is NULL");
     std::lock_guard<std::mutex> lock(c->mu);
+    NOT_WHILE_CAPTURING(c, "apk_timer_begin");
     HIP_TRY(hipEventRecord(c->ev0, c->stream));
     return APK_OK;
 }
 int apk_timer_end(apk_ctx* c, float* ms_out) {
     if (!c || !ms_out) return fail(APK_DECLINE_NULL, "apk_timer_end: NULL argument");
     std::lock_guard<std::mutex> lock(c->mu);
+    NOT_WHILE_CAPTURING(c, "apk_timer_end");
     HIP_TRY(hipEventRecord(c->ev1, c->stream));
     uint64_t t0 = now_ns();
     HIP_TRY(hipEventSynchronize(c->ev1));
     c->wait_ns += now_ns() - t0;
     HIP_TRY(hipEventElapsedTime(ms_out, c->ev0, c->ev1));
+    return APK_OK;
+}
+
+/* ------------------------------------------------------- record / replay */
+
+int apk_capture_begin(apk_ctx* c) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_capture_begin: ctx is NULL");
+    std::lock_guard<std::mutex> lock(c->mu);
+    if (c->capturing) return fail(APK_DECLINE_CAPTURE, "apk_capture_begin: already recording");
+    if (int rc = set_device(c)) return rc;
+    // relaxed: other threads of the process stay free to allocate (the mode the reference uses)
+    HIP_TRY(hipStreamBeginCapture(c->stream, hipStreamCaptureModeRelaxed));
+    c->capturing = true;
+    c->capture_nodes = 0;
+    c->capture_argmax = false;
+    return APK_OK;
+}
+
+static int end_capture(apk_ctx* c, hipGraph_t* g) {
+    *g = nullptr;
+    c->capturing = false;
+    HIP_TRY(hipStreamEndCapture(c->stream, g));
+    return APK_OK;
+}
+
+int apk_capture_end(apk_ctx* c, apk_graph** out) {
+    if (!c || !out) return fail(APK_DECLINE_NULL, "apk_capture_end: NULL argument");
+    *out = nullptr;
+    std::lock_guard<std::mutex> lock(c->mu);
+    if (!c->capturing) return fail(APK_DECLINE_CAPTURE, "apk_capture_end: not recording");
+    if (int rc = set_device(c)) return rc;
+    hipGraph_t g = nullptr;
+    if (int rc = end_capture(c, &g)) return rc;
+    if (!g) return fail(-(int)hipErrorStreamCaptureInvalidated, "apk_capture_end: the recording was invalidated");
+    hipGraphExec_t exec = nullptr;
+    hipError_t e = hipGraphInstantiate(&exec, g, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGraphDestroy(g);
+        return hip_fail(e, "hipGraphInstantiate");
+    }
+    apk_graph* gr = new apk_graph();
+    gr->graph = g;
+    gr->exec = exec;
+    gr->nodes = c->capture_nodes;
+    gr->uses_argmax = c->capture_argmax;
+    if (gr->uses_argmax) c->graphs_with_argmax++;
+    *out = gr;
+    return APK_OK;
+}
+
+int apk_capture_abort(apk_ctx* c) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_capture_abort: ctx is NULL");
+    std::lock_guard<std::mutex> lock(c->mu);
+    if (!c->capturing) return APK_OK;
+    if (int rc = set_device(c)) return rc;
+    hipGraph_t g = nullptr;
+    const int rc = end_capture(c, &g);
+    if (g) (void)hipGraphDestroy(g);
+    return rc;
+}
+
+int apk_graph_launch(apk_ctx* c, apk_graph* g) {
+    if (!c || !g) return fail(APK_DECLINE_NULL, "apk_graph_launch: NULL argument");
+    CallScope s(c);
+    NOT_WHILE_CAPTURING(c, "apk_graph_launch");
+    if (int rc = set_device(c)) return rc;
+    HIP_TRY(hipGraphLaunch(g->exec, c->stream));
+    c->dispatches += g->nodes;
+    return APK_OK;
+}
+
+int apk_graph_nodes(apk_graph* g, size_t* nodes) {
+    if (!g || !nodes) return fail(APK_DECLINE_NULL, "apk_graph_nodes: NULL argument");
+    *nodes = g->nodes;
+    return APK_OK;
+}
+
+int apk_graph_destroy(apk_ctx* c, apk_graph* g) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_graph_destroy: ctx is NULL");
+    if (!g) return APK_OK;
+    std::lock_guard<std::mutex> lock(c->mu);
+    NOT_WHILE_CAPTURING(c, "apk_graph_destroy");
+    if (int rc = set_device(c)) return rc;
+    HIP_TRY(hipStreamSynchronize(c->stream));  // a replay may still be running
+    if (g->uses_argmax && c->graphs_with_argmax) c->graphs_with_argmax--;
+    if (g->exec) (void)hipGraphExecDestroy(g->exec);
+    if (g->graph) (void)hipGraphDestroy(g->graph);
+    delete g;
     return APK_OK;
 }
 
@@ -575,6 +697,7 @@ int apk_embed_rows_host_ids(apk_ctx* c, int fmt, const void* table, size_t vocab
                             const uint32_t* ids_host, size_t t, void* out, int out_dtype) {
     if (!c) return fail(APK_DECLINE_NULL, "apk_embed_rows_host_ids: ctx is NULL");
     CallScope s(c);
+    NOT_WHILE_CAPTURING(c, "apk_embed_rows_host_ids");
     if (t == 0) return APK_OK;
     if (!ids_host) return fail(APK_DECLINE_NULL, "apk_embed_rows_host_ids: ids is NULL");
     for (size_t i = 0; i < t; i++)
@@ -715,6 +838,10 @@ int apk_argmax_rows(apk_ctx* c, const float* logits, size_t rows, size_t n, uint
     if (n == 0 || n > 0xffffffffu || rows > (1u << 20)) return fail(APK_DECLINE_SHAPE, "apk_argmax_rows: sizes out of range");
     if (int rc = set_device(c)) return rc;
     if (rows > c->argmax_rows_cap) {
+        if (c->capturing || c->graphs_with_argmax)
+            return fail(APK_DECLINE_CAPTURE, "apk_argmax_rows: the scratch would have to grow %s",
+                        c->capturing ? "inside a recording (run once unrecorded first)"
+                                     : "while a recorded graph holds its address (destroy the graph first)");
         HIP_TRY(hipStreamSynchronize(c->stream));  // a previous launch may still use the old scratch
         if (c->argmax_scratch) (void)hipFree(c->argmax_scratch);
         c->argmax_scratch = nullptr;
@@ -733,6 +860,7 @@ int apk_argmax_rows(apk_ctx* c, const float* logits, size_t rows, size_t n, uint
     uint64_t n64 = n;
     int parts_i = (int)parts;
     void* args[] = {&logits, &n64, &parts_i, &c->argmax_scratch, &out};
+    if (c->capturing) c->capture_argmax = true;
     return launch(c, "apk_argmax_rows", (unsigned)(rows * parts), 256, 0, args);
 }
 

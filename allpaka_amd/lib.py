@@ -32,6 +32,12 @@ SYMBOLS = {
     "apk_resolve": (_i, [_vp, _vp, _sz, C.POINTER(_vp)]),
     "apk_timer_begin": (_i, [_vp]),
     "apk_timer_end": (_i, [_vp, C.POINTER(_f)]),
+    "apk_capture_begin": (_i, [_vp]),
+    "apk_capture_end": (_i, [_vp, C.POINTER(_vp)]),
+    "apk_capture_abort": (_i, [_vp]),
+    "apk_graph_launch": (_i, [_vp, _vp]),
+    "apk_graph_nodes": (_i, [_vp, C.POINTER(_sz)]),
+    "apk_graph_destroy": (_i, [_vp, _vp]),
     "apk_embed_rows": (_i, [_vp, _i, _vp, _sz, _sz, _vp, _sz, _vp, _i]),
     "apk_embed_rows_host_ids": (_i, [_vp, _i, _vp, _sz, _sz, _vp, _sz, _vp, _i]),
     "apk_add_rmsnorm_rows": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _f, _i]),

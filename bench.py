@@ -182,6 +182,39 @@ def main():
                 p(qk[i % len(qk)]["q"]), p(qk[i % len(qk)]["k"]), p(qw), p(kw), p(rope), rows, NQ, NKV, HD, HD, EPS, F16)), 200)
             record("layer_prologue (add_rmsnorm || qknorm_rope, one launch)", sh, us,
                    4 * rows * H * b + 4 * H + 2 * rows * (NQ + NKV) * HD * b + rows * (HD // 2) * 8 + 2 * HD * 4, note="launch-bound")
+        # the decode chain of a whole model (64 layers x 4 launches) issued op by op, and recorded once
+        # and replayed with one submission; and the 3-launch form with the fused prologue
+        NL = 64
+        for rows, label in ((1, "decode T=1"), (6, "verify T=6"), (64, "batched decode, 64 rows")):
+            sh = f"qwen3-32b {label} f16, {NL} layers"
+            lb = 2 * (4 * rows * H * b + 4 * H) + 2 * rows * (NQ + NKV) * HD * b + rows * (HD // 2) * 8 + 2 * HD * 4 + 3 * rows * FF * b
+
+            def chain4(j):
+                for l in range(NL):
+                    op_addnorm(2 * (j * NL + l), rows=rows)
+                    op_qkrope(j * NL + l, rows=rows)
+                    op_addnorm(2 * (j * NL + l) + 1, gamma2, rows=rows)
+                    op_swiglu(j * NL + l, rows=rows)
+
+            def chain3(j):
+                for l in range(NL):
+                    i = j * NL + l
+                    apklib.check(L.apk_layer_prologue(
+                        h, p(an[(2 * i) % len(an)]["x"]), p(an[(2 * i) % len(an)]["d"]), p(an[(2 * i) % len(an)]["h"]), p(gamma1), H,
+                        p(qk[i % len(qk)]["q"]), p(qk[i % len(qk)]["k"]), p(qw), p(kw), p(rope), rows, NQ, NKV, HD, HD, EPS, F16))
+                    op_addnorm(2 * i + 1, gamma2, rows=rows)
+                    op_swiglu(i, rows=rows)
+
+            for chain, nl, name in ((chain4, 4, "layer chain"), (chain3, 3, "layer chain with fused prologue")):
+                us = timed(chain, 6) / NL
+                record(f"{name}, op by op", sh, us, lb, launches=nl, note="launch-bound; us per layer")
+                g = C.c_void_p()
+                apklib.check(L.apk_capture_begin(h))
+                chain(0)
+                apklib.check(L.apk_capture_end(h, C.byref(g)))
+                us = timed(lambda i: apklib.check(L.apk_graph_launch(h, g)), 12) / NL
+                record(f"{name}, recorded once and replayed", sh, us, lb, launches=nl, note="launch-bound; us per layer")
+                apklib.check(L.apk_graph_destroy(h, g))
         # QK-norm + RoPE with the K/V cache store fused in (one launch; the cache planes of one layer, capacity T)
         kvp = [dict(v=randn((T, NKV * HD)), kc=torch.empty((T, NKV * HD), dtype=torch.float16, device=dev),
                     vc=torch.empty((T, NKV * HD), dtype=torch.float16, device=dev)) for _ in range(len(qk))]

@@ -49,7 +49,8 @@ enum apk_decline {
     APK_DECLINE_NULL = 3,        /* a required pointer is NULL                                         */
     APK_DECLINE_RANGE = 4,       /* an index is out of range (host-checked ids)                        */
     APK_DECLINE_NO_DEVICE = 5,   /* no usable GPU / disabled by ALLPAKA_NO_GPU (capability.rs:58-61)   */
-    APK_DECLINE_NOT_ATTACHED = 6 /* host address is not inside an attached mapping                    */
+    APK_DECLINE_NOT_ATTACHED = 6, /* host address is not inside an attached mapping                   */
+    APK_DECLINE_CAPTURE = 7       /* not possible while (or: only while) the stream is being recorded  */
 };
 
 /* Unified dequant format codes -- the exact integers of gpu::common::dq_fmt
@@ -113,6 +114,34 @@ int apk_resolve(apk_ctx* ctx, const void* host_ptr, size_t len, void** dev_out);
 /* Elapsed device time between two points of the stream (hipEvent based). */
 int apk_timer_begin(apk_ctx* ctx);
 int apk_timer_end(apk_ctx* ctx, float* ms_out);
+
+/* ------------------------------------------------------ record / replay ---- */
+
+/* Records the ops enqueued between begin and end into a HIP graph instead of
+ * running them, and replays the whole chain with ONE submission: the launch-bound
+ * decode chain (a few small kernels per layer, tens of layers) pays the host's
+ * per-launch cost once.  Replaces the stream capture of the reference's CUDA host
+ * (begin_capture in prefill_begin, gpu/cuda/prefill.rs:52-66; `graph.launch()` in
+ * prefill_replay, :71-108; drop_pf_graph, gpu/cuda/runtime/device.rs:626-631).
+ * As there, a graph bakes in every pointer and size its ops were called with, and
+ * nothing may allocate, copy to or from the host, or wait inside a recording:
+ * apk_sync, apk_malloc, apk_free, apk_h2d, apk_d2h, apk_attach, apk_detach,
+ * apk_take_faults, apk_timer_*, apk_embed_rows_host_ids and an apk_argmax_rows that
+ * would have to grow its scratch return APK_DECLINE_CAPTURE and record nothing
+ * (run the chain once unrecorded first, as the reference does).  A declined op
+ * leaves the recording intact.  One recording per context at a time. */
+typedef struct apk_graph apk_graph;
+int apk_capture_begin(apk_ctx* ctx);
+/* Ends the recording and instantiates it; *out is NULL on any non-zero status. */
+int apk_capture_end(apk_ctx* ctx, apk_graph** out);
+/* Ends the recording and throws it away (prefill_abort, gpu/cuda/prefill.rs:180). */
+int apk_capture_abort(apk_ctx* ctx);
+/* Enqueues one replay on the context's stream (asynchronous, ordered like an op). */
+int apk_graph_launch(apk_ctx* ctx, apk_graph* graph);
+/* Number of kernel launches one replay performs. */
+int apk_graph_nodes(apk_graph* graph, size_t* nodes);
+/* Waits for the stream, then frees the graph. */
+int apk_graph_destroy(apk_ctx* ctx, apk_graph* graph);
 
 /* ----------------------------------------------------------------- ops ------ */
 
