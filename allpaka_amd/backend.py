@@ -184,9 +184,21 @@ class Backend:
         self._leave()
         return table
 
-    def qknorm_rope_neox(self, q, k, q_norm, k_norm, rope_flat, n_q, n_kv, head_dim, eps, rot_dim=None):
+    def qknorm_rope_norm(self, q, k, q_norm, k_norm, rope_flat, n_q, n_kv, head_dim, eps, rot_dim=None):
+        """The same loop for RopeStyle::Norm models: adjacent pairs (2i, 2i+1) rotate
+        (rope_norm_cached_from_array, rope.rs:52-64; attention.rs:62-67)."""
+        self.qknorm_rope_neox(q, k, q_norm, k_norm, rope_flat, n_q, n_kv, head_dim, eps, rot_dim, _entry="apk_qknorm_rope_norm")
+
+    def rope_norm_cached_from_array(self, x, table):
+        """ops::rope_norm_cached_from_array (rope.rs:52) on one head."""
+        assert x.numel() >= table.shape[0] * 2
+        self.qknorm_rope_norm(x, x[:0], None, None, table, 1, 0, x.numel(), 0.0, rot_dim=table.shape[0] * 2)
+
+    def qknorm_rope_neox(self, q, k, q_norm, k_norm, rope_flat, n_q, n_kv, head_dim, eps, rot_dim=None,
+                         _entry="apk_qknorm_rope_neox"):
         """The QK-norm + RoPE loop of run_cpu_attention_from_qkv (attention.rs:131-165):
-        q [rows, n_q*head_dim], k [rows, n_kv*head_dim] in place; rope_flat [rows, half, 2]."""
+        q [rows, n_q*head_dim], k [rows, n_kv*head_dim] in place; rope_flat [rows, half, 2]
+        (half = rot_dim/2 <= head_dim/2: partial rotary leaves the tail of a head unrotated)."""
         rows = q.numel() // (n_q * head_dim) if n_q else k.numel() // (n_kv * head_dim)
         assert q.numel() == rows * n_q * head_dim and k.numel() == rows * n_kv * head_dim
         rot = head_dim if rot_dim is None else rot_dim
@@ -195,8 +207,8 @@ class Backend:
         for w in (q_norm, k_norm):
             assert w is None or (w.numel() == head_dim and w.dtype == torch.float32)
         self._enter()
-        check(self.L.apk_qknorm_rope_neox(self.h, _ptr(q), _ptr(k), _ptr(q_norm), _ptr(k_norm), _ptr(rope_flat), rows,
-                                          n_q, n_kv, head_dim, rot, eps, _dt(q)))
+        check(getattr(self.L, _entry)(self.h, _ptr(q), _ptr(k), _ptr(q_norm), _ptr(k_norm), _ptr(rope_flat), rows,
+                                      n_q, n_kv, head_dim, rot, eps, _dt(q)))
         self._leave()
 
     def qknorm_rope_kv_store(self, q, k, v, q_norm, k_norm, rope_flat, cache_pos, k_cache, v_cache, n_q, n_kv, head_dim, eps):

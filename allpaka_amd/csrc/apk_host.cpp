@@ -64,7 +64,8 @@ const int kQkHeadDims[] = {64, 128, 256};
 std::vector<std::string> all_kernel_names() {
     std::vector<std::string> v = {"apk_swiglu_f32", "apk_swiglu_f16", "apk_rope_table", "apk_embed_q4k_f32",
                                   "apk_embed_q4k_f16", "apk_embed_q8_0_f32", "apk_embed_q8_0_f16", "apk_route_topk",
-                                  "apk_moe_permute", "apk_gather_rows", "apk_scatter_rows", "apk_argmax_rows", "apk_add_rmsnorm_ragged_f32", "apk_copy"};
+                                  "apk_moe_permute", "apk_gather_rows", "apk_scatter_rows", "apk_argmax_rows", "apk_add_rmsnorm_ragged_f32", "apk_copy",
+                                  "apk_qknorm_rope_generic_f32", "apk_qknorm_rope_generic_f16"};
     for (const char* t : {"f32", "f16"}) {
         for (const char* f : {"q5k", "q6k", "q2k", "q3k", "q5_0", "f16", "f32", "bf16"}) v.push_back(std::string("apk_embed_") + f + "_" + t);
         for (int c : kAddnormTiles) v.push_back(std::string("apk_add_rmsnorm_") + t + "_c" + std::to_string(c));
@@ -537,19 +538,23 @@ struct KvStore {  // the fused K/V cache store of apk_qknorm_rope_kv_store (all 
     size_t capacity = 0;
 };
 
+// style: 0 = NeoX pairs (i, i + rot_dim/2), 1 = adjacent pairs (2i, 2i+1).  validate_only: every
+// check, no launch (so a caller that chains two ops can decline before the first one runs).
 static int qknorm_rope_common(apk_ctx* c, void* q, void* k, const float* qw, const float* kw, const float* rope, size_t rows,
                               size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim, float eps, int dtype,
-                              const KvStore* kv) {
+                              const KvStore* kv, int style = 0, bool validate_only = false) {
     const int es = elem_size(dtype);
-    if (!es) return fail(APK_DECLINE_UNSUPPORTED, "apk_qknorm_rope_neox: dtype %d", dtype);
-    if (head_dim != 64 && head_dim != 128 && head_dim != 256)
-        return fail(APK_DECLINE_UNSUPPORTED, "apk_qknorm_rope_neox: head_dim %zu", head_dim);
-    if (rot_dim != head_dim)
-        return fail(APK_DECLINE_UNSUPPORTED, "apk_qknorm_rope_neox: partial rotary (rot_dim %zu of %zu)", rot_dim, head_dim);
+    if (!es) return fail(APK_DECLINE_UNSUPPORTED, "apk_qknorm_rope: dtype %d", dtype);
+    if (head_dim == 0 || head_dim > 65536 || rot_dim % 2 || rot_dim > head_dim)
+        return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope: head_dim %zu, rot_dim %zu", head_dim, rot_dim);
+    const bool tiled = style == 0 && rot_dim == head_dim && (head_dim == 64 || head_dim == 128 || head_dim == 256);
+    if (kv && !tiled)
+        return fail(APK_DECLINE_UNSUPPORTED, "apk_qknorm_rope_kv_store: NeoX over a whole head of 64/128/256 only (head_dim %zu, rot_dim %zu)",
+                    head_dim, rot_dim);
     if (rows == 0 || n_q + n_kv == 0) return APK_OK;
-    if ((n_q && !q) || (n_kv && !k) || !rope) return fail(APK_DECLINE_NULL, "apk_qknorm_rope_neox: NULL tensor");
+    if ((n_q && !q) || (n_kv && !k) || (!rope && rot_dim)) return fail(APK_DECLINE_NULL, "apk_qknorm_rope: NULL tensor");
     if ((q && !aligned16(q)) || (k && !aligned16(k)) || !aligned16(rope) || (qw && !aligned16(qw)) || (kw && !aligned16(kw)))
-        return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_neox: tensors must be 16-byte aligned");
+        return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope: tensors must be 16-byte aligned");
     if (kv) {
         if (n_kv == 0) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_kv_store: no k heads");
         if (!kv->v || !kv->cache_pos || !kv->k_cache || !kv->v_cache) return fail(APK_DECLINE_NULL, "apk_qknorm_rope_kv_store: NULL tensor");
@@ -557,7 +562,18 @@ static int qknorm_rope_common(apk_ctx* c, void* q, void* k, const float* qw, con
             return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_kv_store: tensors must be 16-byte aligned");
         if (kv->capacity == 0 || kv->capacity > 0xffffffffu) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_kv_store: capacity");
     }
-    if (rows > 0x7fffffffu || n_q > 65535 || n_kv > 65535) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_neox: too large");
+    if (rows > 0x7fffffffu || n_q > 65535 || n_kv > 65535) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope: too large");
+    int rows_i = (int)rows, nq_i = (int)n_q, nkv_i = (int)n_kv;
+    if (!tiled) {
+        // a wave per head, element-wise: any head_dim, partial rotary, either pairing
+        const uint64_t grid = ((uint64_t)rows * (n_q + n_kv) + 3) / 4;
+        if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope: too large");
+        if (validate_only) return APK_OK;
+        if (int rc = set_device(c)) return rc;
+        int hd_i = (int)head_dim, half_i = (int)(rot_dim / 2);
+        void* gargs[] = {&q, &k, &qw, &kw, &rope, &rows_i, &nq_i, &nkv_i, &hd_i, &half_i, &style, &eps};
+        return launch(c, dtype == APK_F32 ? "apk_qknorm_rope_generic_f32" : "apk_qknorm_rope_generic_f16", (unsigned)grid, 256, 0, gargs);
+    }
     // A wave owns (row, q or k, group of HPW*ITER heads), HPW = heads per wave pass; k waves
     // take one pass.  The largest ITER for q that still leaves >= 1536 waves (6 per CU)
     // amortises the row's [sin, cos] tile and the norm weight over the most heads; small
@@ -573,11 +589,11 @@ static int qknorm_rope_common(apk_ctx* c, void* q, void* k, const float* qw, con
     const uint64_t waves = (uint64_t)rows * ((n_q + hpw * iter - 1) / (hpw * iter) + gk);
     const unsigned block = iter >= 4 ? 64 : 256;
     const uint64_t grid = (waves * 64 + block - 1) / block;
-    if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_neox: too large");
+    if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope: too large");
+    if (validate_only) return APK_OK;
     const std::string which = std::string(kv ? "apk_qknorm_rope_kv_" : "apk_qknorm_rope_") + (dtype == APK_F32 ? "f32" : "f16") +
                               "_hd" + std::to_string(head_dim) + "_i" + std::to_string(iter);
     if (int rc = set_device(c)) return rc;
-    int rows_i = (int)rows, nq_i = (int)n_q, nkv_i = (int)n_kv;
     if (kv) {
         uint32_t cap32 = (uint32_t)kv->capacity;
         void* kargs[] = {&q, &k, (void*)&kv->v, &qw, &kw, &rope, (void*)&kv->cache_pos, (void*)&kv->k_cache, (void*)&kv->v_cache,
@@ -592,7 +608,14 @@ int apk_qknorm_rope_neox(apk_ctx* c, void* q, void* k, const float* qw, const fl
                          size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim, float eps, int dtype) {
     if (!c) return fail(APK_DECLINE_NULL, "apk_qknorm_rope_neox: ctx is NULL");
     CallScope s(c);
-    return qknorm_rope_common(c, q, k, qw, kw, rope, rows, n_q, n_kv, head_dim, rot_dim, eps, dtype, nullptr);
+    return qknorm_rope_common(c, q, k, qw, kw, rope, rows, n_q, n_kv, head_dim, rot_dim, eps, dtype, nullptr, 0);
+}
+
+int apk_qknorm_rope_norm(apk_ctx* c, void* q, void* k, const float* qw, const float* kw, const float* rope,
+                         size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim, float eps, int dtype) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_qknorm_rope_norm: ctx is NULL");
+    CallScope s(c);
+    return qknorm_rope_common(c, q, k, qw, kw, rope, rows, n_q, n_kv, head_dim, rot_dim, eps, dtype, nullptr, 1);
 }
 
 int apk_qknorm_rope_kv_store(apk_ctx* c, void* q, void* k, const void* v, const float* qw, const float* kw,
@@ -624,6 +647,9 @@ int apk_layer_prologue(apk_ctx* c, void* x, const void* delta, void* h, const fl
     if (!fused) {
         // outside the single-launch shape (large batches are bandwidth-bound, not launch-bound):
         // the same result as two launches; every check and decline is theirs
+        // (the second op is validated before the first runs: a decline leaves nothing half done)
+        if (int rc = qknorm_rope_common(c, q, k, qw, kw, rope, rows, n_q, n_kv, head_dim, rot_dim, eps, dtype, nullptr, 0, true))
+            return rc;
         if (int rc = apk_add_rmsnorm_rows(c, x, delta, h, gamma, n, rows, eps, dtype)) return rc;
         return apk_qknorm_rope_neox(c, q, k, qw, kw, rope, rows, n_q, n_kv, head_dim, rot_dim, eps, dtype);
     }

@@ -704,6 +704,57 @@ APK_QKROPE_ALL(f16_t, f16)
 APK_QKROPE_KV_ALL(float, f32)
 APK_QKROPE_KV_ALL(f16_t, f16)
 
+// Any other head geometry: head_dim not 64/128/256, a rotary table that covers only the
+// leading rot_half pairs of a head (partial rotary: channels >= 2*rot_half are normalised
+// and pass through, rope.rs:52-81), or the adjacent-pair style (RopeStyle::Norm, pairs
+// (2i, 2i+1), rope.rs:52-64; chosen per model in attention.rs:62-67).  A wave per head,
+// element-wise; same arithmetic as the tiled kernels minus the coefficient folding.
+template <typename T>
+DEV void qknorm_rope_generic_body(T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q,
+                                  int n_kv, int hd, int rot_half, int norm_style, float eps) {
+    typedef typename stat<T>::acc_t acc_t;
+    const int lane = threadIdx.x & 63;
+    const uint64_t wid = ((uint64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const uint64_t heads = (uint64_t)n_q + n_kv;
+    if (wid >= (uint64_t)rows * heads) return;  // whole wave
+    const uint64_t row = wid / heads;
+    const int hh = (int)(wid % heads);
+    const bool isq = hh < n_q;
+    T* x = isq ? q + (row * n_q + hh) * (uint64_t)hd : k + (row * n_kv + (hh - n_q)) * (uint64_t)hd;
+    const float* w = isq ? qw : kw;
+    const float* t = rope + row * (uint64_t)rot_half * 2;
+    acc_t scale = 1;
+    if (w) {
+        acc_t ss = 0;
+        for (int i = lane; i < hd; i += 64) ss = stat<T>::sq(ss, (float)x[i]);
+        ss = group_sum<64>(ss);  // every lane's loads are consumed here, before any store below
+        scale = stat<T>::rscale(ss, hd, eps);
+    }
+    for (int i = lane; i < rot_half; i += 64) {
+        const int ia = norm_style ? 2 * i : i, ib = norm_style ? 2 * i + 1 : i + rot_half;
+        float a = (float)x[ia], b = (float)x[ib];
+        if (w) {
+            a = stat<T>::apply(a, scale, w[ia]);
+            b = stat<T>::apply(b, scale, w[ib]);
+        }
+        const float sn = t[2 * i], cs = t[2 * i + 1];
+        x[ia] = (T)(a * cs - b * sn);
+        x[ib] = (T)(a * sn + b * cs);
+    }
+    if (w)
+        for (int i = 2 * rot_half + lane; i < hd; i += 64) x[i] = (T)stat<T>::apply((float)x[i], scale, w[i]);
+}
+extern "C" __global__ __launch_bounds__(256) void apk_qknorm_rope_generic_f32(
+    float* q, float* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv, int hd,
+    int rot_half, int norm_style, float eps) {
+    qknorm_rope_generic_body<float>(q, k, qw, kw, rope, rows, n_q, n_kv, hd, rot_half, norm_style, eps);
+}
+extern "C" __global__ __launch_bounds__(256) void apk_qknorm_rope_generic_f16(
+    f16_t* q, f16_t* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv, int hd,
+    int rot_half, int norm_style, float eps) {
+    qknorm_rope_generic_body<f16_t>(q, k, qw, kw, rope, rows, n_q, n_kv, hd, rot_half, norm_style, eps);
+}
+
 // Layer prologue for small decode batches: the residual add + RMSNorm of the hidden
 // rows and the QK-norm + RoPE of the q/k rows as ONE launch.  They are two independent
 // jobs sharing a grid (workgroups [0, rows) normalise one hidden row each, the rest

@@ -8,7 +8,7 @@ _SO = os.path.join(_HERE, "libapk_hip.so")
 
 F32, F16 = 0, 1
 FMT_Q4K, FMT_Q5K, FMT_Q6K, FMT_Q8_0, FMT_Q2K, FMT_Q3K, FMT_Q5_0, FMT_F16, FMT_F32, FMT_BF16 = range(10)
-DECLINE_UNSUPPORTED, DECLINE_SHAPE, DECLINE_NULL, DECLINE_RANGE, DECLINE_NO_DEVICE, DECLINE_NOT_ATTACHED = range(1, 7)
+DECLINE_UNSUPPORTED, DECLINE_SHAPE, DECLINE_NULL, DECLINE_RANGE, DECLINE_NO_DEVICE, DECLINE_NOT_ATTACHED, DECLINE_CAPTURE = range(1, 8)
 FAULT_TOKEN_RANGE, FAULT_EXPERT_RANGE, FAULT_ROW_RANGE, FAULT_CACHE_RANGE = 1, 2, 4, 8
 
 # every symbol include/apk_hip.h declares: (restype, argtypes)
@@ -42,6 +42,7 @@ SYMBOLS = {
     "apk_embed_rows_host_ids": (_i, [_vp, _i, _vp, _sz, _sz, _vp, _sz, _vp, _i]),
     "apk_add_rmsnorm_rows": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _f, _i]),
     "apk_qknorm_rope_neox": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _f, _i]),
+    "apk_qknorm_rope_norm": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _f, _i]),
     "apk_qknorm_rope_kv_store": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _sz, _f, _i]),
     "apk_layer_prologue": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _f, _i]),
     "apk_rope_table": (_i, [_vp, _vp, _vp, _sz, _sz, _vp]),

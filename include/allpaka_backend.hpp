@@ -146,6 +146,15 @@ inline void rope_neox_cached_from_array(std::vector<float>& x, const std::vector
     dx.read_back(x.data());
 }
 
+// ops::rope_norm_cached_from_array(x, table): adjacent pairs (2i, 2i+1) rotate (rope.rs:52).
+inline void rope_norm_cached_from_array(std::vector<float>& x, const std::vector<std::array<float, 2>>& table) {
+    if (x.size() < table.size() * 2) throw Panic("assertion failed: x.len() >= table.len() * 2");
+    Dev<float> dx(x.data(), x.size()), dt(&table[0][0], table.size() * 2);
+    check(apk_qknorm_rope_norm(Gpu::get().ctx(), dx.ptr(), nullptr, nullptr, nullptr, dt.ptr(), 1, 1, 0, x.size(), table.size() * 2,
+                               0.0f, APK_F32));
+    dx.read_back(x.data());
+}
+
 // The QK-norm + RoPE loop of run_cpu_attention_from_qkv (attention.rs:131-165) over rows of q and k.
 inline void qknorm_rope_rows(std::vector<float>& q, std::vector<float>& k, const std::vector<float>* q_norm,
                              const std::vector<float>* k_norm, const std::vector<std::array<float, 2>>& rope_flat, size_t rows,

@@ -176,10 +176,19 @@ int apk_add_rmsnorm_rows(apk_ctx* ctx, void* x, const void* delta, void* h, cons
  * over every q and k head of every row (model/attention.rs:131-165,
  * ops/norm.rs:115-187, ops/rope.rs:70-81).
  * q: [rows][n_q*head_dim], k: [rows][n_kv*head_dim] of dtype; qw, kw: f32[head_dim]
- * or NULL (no norm for that tensor); rope: f32 [rows][head_dim/2][2] = [sin, cos]
+ * or NULL (no norm for that tensor); rope: f32 [rows][rot_dim/2][2] = [sin, cos]
  * per row (the session table rows, model/session.rs:34-50).
- * head_dim in {64,128,256}; rot_dim must equal head_dim (else declined). */
+ * rot_dim (even, <= head_dim) is the rotary width: pairs (i, i + rot_dim/2) rotate and
+ * channels >= rot_dim are normalised and pass through (partial rotary, rope.rs:66-81).
+ * head_dim in {64,128,256} with rot_dim == head_dim takes the tiled kernels; any other
+ * geometry takes an element-wise kernel (a wave per head). */
 int apk_qknorm_rope_neox(apk_ctx* ctx, void* q, void* k, const float* qw, const float* kw, const float* rope,
+                         size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim, float eps,
+                         int dtype);
+/* The same with the adjacent-pair rotation (2i, 2i+1) of RopeStyle::Norm models:
+ * ops::rope_norm_cached_from_array (ops/rope.rs:52-64), selected per model in
+ * rope_from_arrays (model/attention.rs:62-67).  Element-wise kernel for every geometry. */
+int apk_qknorm_rope_norm(apk_ctx* ctx, void* q, void* k, const float* qw, const float* kw, const float* rope,
                          size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim, float eps,
                          int dtype);
 
@@ -193,7 +202,8 @@ int apk_qknorm_rope_neox(apk_ctx* ctx, void* q, void* k, const float* qw, const 
  * v: [rows][n_kv*head_dim] of dtype (read only); cache_pos: u32[rows] on the device;
  * k_cache, v_cache: fp16 [capacity][n_kv*head_dim] (one layer's K and V planes).
  * A position >= capacity skips that row's cache store and raises APK_FAULT_CACHE_RANGE
- * (the reference asserts "position past capacity"). */
+ * (the reference asserts "position past capacity").  NeoX over a whole head of
+ * 64/128/256 only; other geometries are declined (run the two steps separately). */
 int apk_qknorm_rope_kv_store(apk_ctx* ctx, void* q, void* k, const void* v, const float* qw, const float* kw,
                              const float* rope, const uint32_t* cache_pos, void* k_cache, void* v_cache,
                              size_t capacity, size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim,

@@ -66,6 +66,8 @@ def lib():
         L.ora_rope_norm.argtypes = [vp, sz, u32, f32]
         L.ora_qknorm_rope_rows.argtypes = [vp, vp, sz, sz, sz, sz, vp, vp, vp, sz, f32]
         L.ora_qknorm_rope_rows_f16.argtypes = [vp, vp, sz, sz, sz, sz, vp, vp, vp, sz, f32]
+        L.ora_qknorm_rope_rows_style.argtypes = [vp, vp, sz, sz, sz, sz, vp, vp, vp, sz, f32, C.c_int]
+        L.ora_qknorm_rope_rows_style_f16.argtypes = [vp, vp, sz, sz, sz, sz, vp, vp, vp, sz, f32, C.c_int]
         L.ora_silu.restype = f32
         L.ora_silu.argtypes = [f32]
         L.ora_swiglu.argtypes = [vp, sz, vp, sz]
@@ -277,16 +279,17 @@ def rope_norm(x, pos, base):
     lib().ora_rope_norm(_p(x), x.size, int(pos), base)
 
 
-def qknorm_rope_rows(q, k, n_q, n_kv, head_dim, qw, kw, rope_flat, eps):
-    """OP-C: q [rows, n_q*hd], k [rows, n_kv*hd] in place; rope_flat [rows, half, 2]."""
+def qknorm_rope_rows(q, k, n_q, n_kv, head_dim, qw, kw, rope_flat, eps, style=0):
+    """OP-C: q [rows, n_q*hd], k [rows, n_kv*hd] in place; rope_flat [rows, half, 2];
+    style 0 = NeoX pairs, 1 = adjacent (NORM) pairs."""
     rows = q.shape[0]
     half = rope_flat.shape[1]
     _chk(rope_flat, np.float32)
     if q.dtype == np.float32:
-        lib().ora_qknorm_rope_rows(_p(q), _p(k), rows, n_q, n_kv, head_dim, _p(qw), _p(kw), _p(rope_flat), half, eps)
+        lib().ora_qknorm_rope_rows_style(_p(q), _p(k), rows, n_q, n_kv, head_dim, _p(qw), _p(kw), _p(rope_flat), half, eps, style)
     else:
         _chk(q, np.uint16)
-        lib().ora_qknorm_rope_rows_f16(_p(q), _p(k), rows, n_q, n_kv, head_dim, _p(qw), _p(kw), _p(rope_flat), half, eps)
+        lib().ora_qknorm_rope_rows_style_f16(_p(q), _p(k), rows, n_q, n_kv, head_dim, _p(qw), _p(kw), _p(rope_flat), half, eps, style)
 
 
 # ---- activation

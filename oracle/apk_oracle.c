@@ -527,14 +527,17 @@ ORA_API void ora_rope_norm(float *x, size_t d, uint32_t pos, float base) {
  * crates/allpaka-model/src/model/attention.rs:131-165: for row i, every head of
  * q then of k gets rmsnorm(head, w, eps) (when a weight is given) followed by
  * the NeoX rotation with that row's table rope_flat[i*half .. (i+1)*half]. */
-ORA_API void ora_qknorm_rope_rows(float *q, float *k, size_t rows, size_t n_q, size_t n_kv, size_t head_dim,
-                                  const float *qw, const float *kw, const float *rope_flat, size_t half, float eps) {
+/* style 0: RopeStyle::Neox, 1: RopeStyle::Norm (rope_from_arrays, attention.rs:62-67) */
+ORA_API void ora_qknorm_rope_rows_style(float *q, float *k, size_t rows, size_t n_q, size_t n_kv, size_t head_dim,
+                                        const float *qw, const float *kw, const float *rope_flat, size_t half, float eps,
+                                        int style) {
     for (size_t i = 0; i < rows; i++) {
         const float *rope = rope_flat + i * half * 2;
         for (size_t h = 0; h < n_q; h++) {
             float *head = q + (i * n_q + h) * head_dim;
             if (qw) ora_rmsnorm(head, qw, head_dim, eps);
-            ora_rope_neox_cached_from_array(head, head_dim, rope, half);
+            if (style) ora_rope_norm_cached_from_array(head, head_dim, rope, half);
+            else ora_rope_neox_cached_from_array(head, head_dim, rope, half);
         }
     }
     for (size_t i = 0; i < rows; i++) {
@@ -542,9 +545,14 @@ ORA_API void ora_qknorm_rope_rows(float *q, float *k, size_t rows, size_t n_q, s
         for (size_t h = 0; h < n_kv; h++) {
             float *head = k + (i * n_kv + h) * head_dim;
             if (kw) ora_rmsnorm(head, kw, head_dim, eps);
-            ora_rope_neox_cached_from_array(head, head_dim, rope, half);
+            if (style) ora_rope_norm_cached_from_array(head, head_dim, rope, half);
+            else ora_rope_neox_cached_from_array(head, head_dim, rope, half);
         }
     }
+}
+ORA_API void ora_qknorm_rope_rows(float *q, float *k, size_t rows, size_t n_q, size_t n_kv, size_t head_dim,
+                                  const float *qw, const float *kw, const float *rope_flat, size_t half, float eps) {
+    ora_qknorm_rope_rows_style(q, k, rows, n_q, n_kv, head_dim, qw, kw, rope_flat, half, eps, 0);
 }
 
 /* ------------------------------------------------------------- activation */
@@ -771,16 +779,21 @@ ORA_API void ora_add_rmsnorm_rows_f16(uint16_t *x, const uint16_t *delta, uint16
     }
     free(v); free(o);
 }
-ORA_API void ora_qknorm_rope_rows_f16(uint16_t *q, uint16_t *k, size_t rows, size_t n_q, size_t n_kv, size_t head_dim,
-                                      const float *qw, const float *kw, const float *rope_flat, size_t half, float eps) {
+ORA_API void ora_qknorm_rope_rows_style_f16(uint16_t *q, uint16_t *k, size_t rows, size_t n_q, size_t n_kv, size_t head_dim,
+                                            const float *qw, const float *kw, const float *rope_flat, size_t half, float eps,
+                                            int style) {
     size_t nq = rows * n_q * head_dim, nk = rows * n_kv * head_dim;
     float *qf = (float *)malloc(sizeof(float) * (nq ? nq : 1)), *kf = (float *)malloc(sizeof(float) * (nk ? nk : 1));
     ora_f16_to_f32_slice(q, qf, nq);
     ora_f16_to_f32_slice(k, kf, nk);
-    ora_qknorm_rope_rows(qf, kf, rows, n_q, n_kv, head_dim, qw, kw, rope_flat, half, eps);
+    ora_qknorm_rope_rows_style(qf, kf, rows, n_q, n_kv, head_dim, qw, kw, rope_flat, half, eps, style);
     ora_f32_to_f16_slice(qf, q, nq);
     ora_f32_to_f16_slice(kf, k, nk);
     free(qf); free(kf);
+}
+ORA_API void ora_qknorm_rope_rows_f16(uint16_t *q, uint16_t *k, size_t rows, size_t n_q, size_t n_kv, size_t head_dim,
+                                      const float *qw, const float *kw, const float *rope_flat, size_t half, float eps) {
+    ora_qknorm_rope_rows_style_f16(q, k, rows, n_q, n_kv, head_dim, qw, kw, rope_flat, half, eps, 0);
 }
 ORA_API void ora_swiglu_f16(uint16_t *gate, const uint16_t *up, size_t n) {
     for (size_t i = 0; i < n; i++)

@@ -99,8 +99,28 @@ static void rope_neox_pairs_split_channels() {  // :206-221
     x[0] = 1.0f;
     ops::rope_neox_cached_from_array(x, table_for(1, 128, 10000.0f));
     CHECK(close(x[64], std::sin(1.0f)) && x[1] == 0.0f);
-    // a head the device path does not take (partial rotary) is declined, not mis-rotated
-    CHECK(throws<Declined>([] { std::vector<float> x(128, 1.0f); ops::rope_neox_cached_from_array(x, table_for(1, 64, 10000.0f)); }));
+    // adjacent-pair style: channel 0 pairs with channel 1 (rope.rs:90-101)
+    std::vector<float> y(128, 0.0f);
+    y[0] = 1.0f;
+    ops::rope_norm_cached_from_array(y, table_for(1, 128, 10000.0f));
+    CHECK(close(y[1], std::sin(1.0f)) && y[64] == 0.0f);
+}
+static void partial_rotary_rotates_the_head_and_passes_the_tail() {  // :367-391 (12-wide head, 8 rotating channels)
+    std::vector<float> orig(12);
+    for (size_t i = 0; i < 12; i++) orig[i] = 0.25f * (float)i - 1.0f;
+    auto table = table_for(5, 8, 10000.0f);
+    std::vector<float> a(orig), b(orig);
+    ops::rope_neox_cached_from_array(a, table);
+    ops::rope_norm_cached_from_array(b, table);
+    for (size_t i = 8; i < 12; i++) CHECK(a[i] == orig[i] && b[i] == orig[i]);
+    // the rotating channels are those of an 8-wide head on its own
+    std::vector<float> a8(orig.begin(), orig.begin() + 8), b8(a8);
+    ops::rope_neox_cached_from_array(a8, table);
+    ops::rope_norm_cached_from_array(b8, table);
+    for (size_t i = 0; i < 8; i++) CHECK(a[i] == a8[i] && b[i] == b8[i]);
+    CHECK(a8 != b8);
+    // a table longer than the head is the reference's assertion
+    CHECK(throws<Panic>([] { std::vector<float> x(8, 1.0f); ops::rope_neox_cached_from_array(x, table_for(1, 16, 10000.0f)); }));
 }
 static void device_rope_rows_match_the_host_table() {  // session.rs:34-50
     std::vector<float> inv(64);
@@ -150,6 +170,7 @@ int main() {
         {"swiglu_is_silu_of_gate_times_up", swiglu_is_silu_of_gate_times_up},
         {"rope_is_norm_preserving_and_identity_at_position_zero", rope_is_norm_preserving_and_identity_at_position_zero},
         {"rope_neox_pairs_split_channels", rope_neox_pairs_split_channels},
+        {"partial_rotary_rotates_the_head_and_passes_the_tail", partial_rotary_rotates_the_head_and_passes_the_tail},
         {"device_rope_rows_match_the_host_table", device_rope_rows_match_the_host_table},
         {"q8_0_is_scale_times_value", q8_0_is_scale_times_value},
         {"route_picks_the_top_k_and_renormalises", route_picks_the_top_k_and_renormalises},

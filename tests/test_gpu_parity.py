@@ -306,8 +306,66 @@ def test_rope_only_and_reference_vectors(be, ora):
     assert abs(h[64] - np.sin(np.float32(1.0))) < 1e-6 and h[1] == 0.0
     import allpaka_amd as apk
 
-    with pytest.raises(apk.Declined):  # partial rotary is declined, not mis-rotated
-        be.qknorm_rope_neox(tq, tk, None, None, dev(ropes[:, :32].copy()), n_q, n_kv, hd, 1e-6, rot_dim=64)
+    tr = dev(ropes)
+    for bad_hd, bad_rot in ((128, 63), (64, 128), (0, 0)):  # odd rotary width; wider than the head; no head
+        rc = be.L.apk_qknorm_rope_neox(be.h, tq.data_ptr(), tk.data_ptr(), None, None, tr.data_ptr(), 2, n_q, n_kv, bad_hd, bad_rot,
+                                       1e-6, apk.lib.F32)
+        assert rc == apk.lib.DECLINE_SHAPE, (bad_hd, bad_rot)
+    be.sync()
+    assert np.array_equal(host(tq), wq)  # declined: nothing touched
+    # adjacent-pair style: a one-hot channel 0 moves energy to channel 1 (rope.rs:90-101)
+    x = torch.zeros(128, device="cuda")
+    x[0] = 1.0
+    be.rope_norm_cached_from_array(x, dev(t1))
+    h = host(x)
+    assert abs(h[1] - np.sin(np.float32(1.0))) < 1e-6 and h[64] == 0.0
+    # the reference's partial-rotary vector: a 12-wide head rotating its first 8 channels (ops/mod.rs:367-391)
+    inv4 = ora.rope_inv_freq(8, 10000.0)
+    t4 = ora.rope_sin_cos(5, inv4)
+    for name in ("rope_neox_cached_from_array", "rope_norm_cached_from_array"):
+        a = (np.arange(12, dtype=np.float32) * 0.25 - 1.0).astype(np.float32)
+        want = a.copy()
+        getattr(ora, name)(want, t4)
+        ta = dev(a)
+        getattr(be, name)(ta, dev(t4))
+        assert np.array_equal(host(ta), want)
+        assert np.array_equal(want[8:], a[8:])  # the tail passes through
+
+
+@pytest.mark.parametrize("rows,n_q,n_kv,hd,rot", [
+    (5, 4, 2, 128, 64),   # partial rotary on a tiled head size (GLM style)
+    (3, 6, 2, 96, 96), (7, 5, 1, 80, 32), (2, 2, 2, 192, 192), (4, 3, 3, 32, 16), (1, 1, 1, 576, 64), (3, 2, 1, 128, 0),
+])
+@pytest.mark.parametrize("style", [0, 1])
+@pytest.mark.parametrize("f16", [False, True])
+@pytest.mark.parametrize("normed", [True, False])
+def test_qknorm_rope_any_geometry(be, ora, rows, n_q, n_kv, hd, rot, style, f16, normed):
+    """Head sizes outside 64/128/256, partial rotary and the adjacent-pair style: the reference's caller loop
+    (attention.rs:131-165 with rope_from_arrays :62-67) through the element-wise kernel."""
+    s = synth()
+    g = s.rng(3, rows * 977 + hd * 13 + rot + style)
+    q, k = s.normal_f32(g, (rows, n_q * hd)), s.normal_f32(g, (rows, n_kv * hd))
+    qw, kw = (s.normal_f32(g, hd, 1.0, 0.05), s.normal_f32(g, hd, 1.0, 0.05)) if normed else (None, None)
+    if f16:
+        q, k = s.to_f16_bits(q), s.to_f16_bits(k)
+    positions = [int(v) for v in g.integers(0, 32768, size=rows)]
+    if rot:
+        ropes = ora.rope_table(positions, ora.rope_inv_freq(rot, 1e6))
+    else:
+        ropes = np.zeros((rows, 0, 2), np.float32)
+    wq, wk = q.copy(), k.copy()
+    ora.qknorm_rope_rows(wq, wk, n_q, n_kv, hd, qw, kw, ropes, 1e-6, style=style)
+    tq, tk = dev(q), dev(k)
+    fn = be.qknorm_rope_norm if style else be.qknorm_rope_neox
+    rt = dev(ropes) if rot else torch.zeros((rows, 0, 2), device="cuda")
+    fn(tq, tk, None if qw is None else dev(qw), None if kw is None else dev(kw), rt, n_q, n_kv, hd, 1e-6, rot_dim=rot)
+    for got, want in ((host(tq), wq), (host(tk), wk)):
+        if f16:
+            assert f16_ulp_diff(got, want) <= TOL_F16_ULP
+        elif not normed:
+            assert np.array_equal(got, want)  # rotation only: the same f32 operations
+        else:
+            assert rel_err_f32(got, want) <= TOL_F32 and close_idiom(got, want)
 
 
 def test_rope_table_on_device(be, ora):
