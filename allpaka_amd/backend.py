@@ -391,13 +391,18 @@ class QuantMat:
         check(self.b.L.apk_embed_rows_host_ids(self.b.h, self.ty, _ptr(self.data), self.n_out, self.n_in, ids, 1, _ptr(dst), _dt(dst)))
         self.b.sync()
 
-    def rows_into(self, ids, dst):
-        """The embedding loop of forward_batch (prefill.rs:92-106) as one launch; ids on the device."""
+    def rows_into(self, ids, dst, embed_scale=1.0):
+        """The embedding loop of forward_batch (prefill.rs:92-109) as one launch; ids on the device;
+        embed_scale: the multiplier of models that scale their token embeddings."""
         t = ids.numel()
         if dst.numel() != t * self.n_in:
             raise ValueError("destination size")
         self.b._enter()
-        check(self.b.L.apk_embed_rows(self.b.h, self.ty, _ptr(self.data), self.n_out, self.n_in, _ptr(ids), t, _ptr(dst), _dt(dst)))
+        if embed_scale == 1.0:
+            check(self.b.L.apk_embed_rows(self.b.h, self.ty, _ptr(self.data), self.n_out, self.n_in, _ptr(ids), t, _ptr(dst), _dt(dst)))
+        else:
+            check(self.b.L.apk_embed_rows_scaled(self.b.h, self.ty, _ptr(self.data), self.n_out, self.n_in, _ptr(ids), t,
+                                                 embed_scale, _ptr(dst), _dt(dst)))
         self.b.sync()
         if self.b.take_faults() & _l.FAULT_TOKEN_RANGE:
             raise ValueError("token id out of vocab")

@@ -681,7 +681,7 @@ int apk_rope_table(apk_ctx* c, const uint32_t* positions, const float* inv_freq,
 }
 
 static int embed_common(apk_ctx* c, int fmt, const void* table, size_t vocab, size_t n_in, const uint32_t* ids_dev,
-                        size_t t, void* out, int out_dtype) {
+                        size_t t, void* out, int out_dtype, float scale = 1.0f) {
     if (!apk_can_embed(fmt, n_in)) return fail(APK_DECLINE_UNSUPPORTED, "apk_embed_rows: fmt %d / n_in %zu", fmt, n_in);
     if (!elem_size(out_dtype)) return fail(APK_DECLINE_UNSUPPORTED, "apk_embed_rows: out_dtype %d", out_dtype);
     if (t == 0) return APK_OK;
@@ -696,7 +696,7 @@ static int embed_common(apk_ctx* c, int fmt, const void* table, size_t vocab, si
         // one workgroup per row, 8 lanes per 256-element super-block
         size_t threads = (n_in / 256 * 8 + 63) / 64 * 64;
         if (threads > 256) threads = 256;
-        void* args[] = {&table, &vocab32, &n_i, &ids_dev, &out, &c->fault_dev};
+        void* args[] = {&table, &vocab32, &n_i, &ids_dev, &out, &c->fault_dev, &scale};
         return launch(c, out_dtype == APK_F32 ? "apk_embed_q4k_f32" : "apk_embed_q4k_f16", (unsigned)t, (unsigned)threads, 0, args);
     }
     // every other format: one workgroup per row, the row staged in LDS
@@ -707,7 +707,7 @@ static int embed_common(apk_ctx* c, int fmt, const void* table, size_t vocab, si
     const size_t max_threads = fmt == APK_FMT_Q8_0 ? 1024 : 256;
     if (threads > max_threads) threads = max_threads;
     uint64_t table_bytes = (uint64_t)vocab * row_bytes;
-    void* args[] = {&table, &table_bytes, &vocab32, &n_i, &ids_dev, &out, &c->fault_dev};
+    void* args[] = {&table, &table_bytes, &vocab32, &n_i, &ids_dev, &out, &c->fault_dev, &scale};
     const std::string which = std::string("apk_embed_") + kFmtName[fmt] + (out_dtype == APK_F32 ? "_f32" : "_f16");
     return launch(c, which, (unsigned)t, (unsigned)threads, (unsigned)shmem, args);
 }
@@ -717,6 +717,13 @@ int apk_embed_rows(apk_ctx* c, int fmt, const void* table, size_t vocab, size_t 
     if (!c) return fail(APK_DECLINE_NULL, "apk_embed_rows: ctx is NULL");
     CallScope s(c);
     return embed_common(c, fmt, table, vocab, n_in, ids, t, out, out_dtype);
+}
+
+int apk_embed_rows_scaled(apk_ctx* c, int fmt, const void* table, size_t vocab, size_t n_in, const uint32_t* ids, size_t t,
+                          float scale, void* out, int out_dtype) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_embed_rows_scaled: ctx is NULL");
+    CallScope s(c);
+    return embed_common(c, fmt, table, vocab, n_in, ids, t, out, out_dtype, scale);
 }
 
 int apk_embed_rows_host_ids(apk_ctx* c, int fmt, const void* table, size_t vocab, size_t n_in,

@@ -819,8 +819,18 @@ DEV void k4_scale_min(const u32x4 hdr, int s, float& sc, float& mn) {
     mn = (float)b;
 }
 
+// The embedding multiplier of models that scale their token embeddings (`*v *= embed_scale`
+// after the dequant, only when it is not 1: model/prefill.rs:107-109, model/decode.rs:427-429).
+template <int N> DEV void embed_scale(float* v, float scale) {
+    if (scale != 1.0f) {
+#pragma unroll
+        for (int i = 0; i < N; i++) v[i] *= scale;
+    }
+}
+
 template <typename TO>
-DEV void embed_q4k_body(const uint8_t* table, uint32_t vocab, int n_in, const uint32_t* ids, TO* out, uint32_t* fault) {
+DEV void embed_q4k_body(const uint8_t* table, uint32_t vocab, int n_in, const uint32_t* ids, TO* out, uint32_t* fault,
+                        float scale) {
     const int nsb = n_in / 256;
     const uint64_t t = blockIdx.x;
     const uint32_t id = ids[t];
@@ -854,6 +864,7 @@ DEV void embed_q4k_body(const uint8_t* table, uint32_t vocab, int n_in, const ui
                         const uint32_t qv = hi ? (byte >> 4) : (byte & 0xfu);
                         v[4 * w + b] = dl * (float)qv - ml;
                     }
+                embed_scale<8>(v, scale);
                 io<f16_t>::store_nt((f16_t*)orow + (uint64_t)sb * 256 + k * 64 + L * 8, v);
             }
         } else {
@@ -872,18 +883,21 @@ DEV void embed_q4k_body(const uint8_t* table, uint32_t vocab, int n_in, const ui
                     const uint32_t qv = (k & 1) ? (byte >> 4) : (byte & 0xfu);
                     v[b] = dl * (float)qv - ml;
                 }
+                embed_scale<4>(v, scale);
                 io<float>::store_nt((float*)orow + (uint64_t)sb * 256 + k * 32 + L * 4, v);
             }
         }
     }
 }
 extern "C" __global__ __launch_bounds__(256) void apk_embed_q4k_f32(const uint8_t* table, uint32_t vocab, int n_in,
-                                                                   const uint32_t* ids, float* out, uint32_t* fault) {
-    embed_q4k_body<float>(table, vocab, n_in, ids, out, fault);
+                                                                   const uint32_t* ids, float* out, uint32_t* fault,
+                                                                   float scale) {
+    embed_q4k_body<float>(table, vocab, n_in, ids, out, fault, scale);
 }
 extern "C" __global__ __launch_bounds__(256) void apk_embed_q4k_f16(const uint8_t* table, uint32_t vocab, int n_in,
-                                                                   const uint32_t* ids, f16_t* out, uint32_t* fault) {
-    embed_q4k_body<f16_t>(table, vocab, n_in, ids, out, fault);
+                                                                   const uint32_t* ids, f16_t* out, uint32_t* fault,
+                                                                   float scale) {
+    embed_q4k_body<f16_t>(table, vocab, n_in, ids, out, fault, scale);
 }
 
 // Q8_0 (dequant.rs:94-126): 34-byte block = f16 scale + 32 int8; out = d * q.
@@ -893,7 +907,7 @@ extern "C" __global__ __launch_bounds__(256) void apk_embed_q4k_f16(const uint8_
 // from LDS, consecutive lanes writing consecutive tiles.
 template <typename TO>
 DEV void embed_q8_0_body(const uint8_t* table, uint64_t table_bytes, uint32_t vocab, int n_in, const uint32_t* ids,
-                         TO* out, uint32_t* fault) {
+                         TO* out, uint32_t* fault, float scale) {
     extern __shared__ __attribute__((aligned(16))) uint8_t stage[];
     constexpr int OPT = io<TO>::VEC;  // outputs per tile
     const uint64_t t = blockIdx.x;
@@ -935,18 +949,19 @@ DEV void embed_q8_0_body(const uint8_t* table, uint64_t table_bytes, uint32_t vo
             o[2 * i] = d * (float)(int8_t)(two & 0xffu);
             o[2 * i + 1] = d * (float)(int8_t)(two >> 8);
         }
+        embed_scale<OPT>(o, scale);
         io<TO>::store_nt(out + t * (uint64_t)n_in + (uint64_t)g * OPT, o);
     }
 }
 extern "C" __global__ __launch_bounds__(1024) void apk_embed_q8_0_f32(const uint8_t* table, uint64_t table_bytes,
                                                                      uint32_t vocab, int n_in, const uint32_t* ids,
-                                                                     float* out, uint32_t* fault) {
-    embed_q8_0_body<float>(table, table_bytes, vocab, n_in, ids, out, fault);
+                                                                     float* out, uint32_t* fault, float scale) {
+    embed_q8_0_body<float>(table, table_bytes, vocab, n_in, ids, out, fault, scale);
 }
 extern "C" __global__ __launch_bounds__(1024) void apk_embed_q8_0_f16(const uint8_t* table, uint64_t table_bytes,
                                                                      uint32_t vocab, int n_in, const uint32_t* ids,
-                                                                     f16_t* out, uint32_t* fault) {
-    embed_q8_0_body<f16_t>(table, table_bytes, vocab, n_in, ids, out, fault);
+                                                                     f16_t* out, uint32_t* fault, float scale) {
+    embed_q8_0_body<f16_t>(table, table_bytes, vocab, n_in, ids, out, fault, scale);
 }
 
 // ---- the other GGUF formats of the unified dequant codes (gpu/common.rs:47-61) -------
@@ -1046,7 +1061,7 @@ template <> struct dq<8> {  // F32 (rows are 4-byte aligned)
 // writing consecutive tiles.
 template <int FMT, typename TO>
 DEV void embed_staged_body(const uint8_t* table, uint64_t table_bytes, uint32_t vocab, int n_in, const uint32_t* ids,
-                           TO* out, uint32_t* fault) {
+                           TO* out, uint32_t* fault, float scale) {
     extern __shared__ __attribute__((aligned(16))) uint8_t stage[];
     constexpr int OPT = io<TO>::VEC, BE = dq<FMT>::BE, BB = dq<FMT>::BB;
     const uint64_t t = blockIdx.x;
@@ -1083,19 +1098,20 @@ DEV void embed_staged_body(const uint8_t* table, uint64_t table_bytes, uint32_t 
             const int e = e0 + i;
             o[i] = dq<FMT>::elem(stage + mis + (e / BE) * BB, e % BE);
         }
+        embed_scale<OPT>(o, scale);
         io<TO>::store_nt(out + t * (uint64_t)n_in + e0, o);
     }
 }
 #define APK_EMBED_GEN(NAME, FMT)                                                                                          \
     extern "C" __global__ __launch_bounds__(256) void apk_embed_##NAME##_f32(                                             \
         const uint8_t* table, uint64_t table_bytes, uint32_t vocab, int n_in, const uint32_t* ids, float* out,            \
-        uint32_t* fault) {                                                                                                \
-        embed_staged_body<FMT, float>(table, table_bytes, vocab, n_in, ids, out, fault);                                  \
+        uint32_t* fault, float scale) {                                                                                   \
+        embed_staged_body<FMT, float>(table, table_bytes, vocab, n_in, ids, out, fault, scale);                           \
     }                                                                                                                     \
     extern "C" __global__ __launch_bounds__(256) void apk_embed_##NAME##_f16(                                             \
         const uint8_t* table, uint64_t table_bytes, uint32_t vocab, int n_in, const uint32_t* ids, f16_t* out,            \
-        uint32_t* fault) {                                                                                                \
-        embed_staged_body<FMT, f16_t>(table, table_bytes, vocab, n_in, ids, out, fault);                                  \
+        uint32_t* fault, float scale) {                                                                                   \
+        embed_staged_body<FMT, f16_t>(table, table_bytes, vocab, n_in, ids, out, fault, scale);                           \
     }
 APK_EMBED_GEN(q5k, 1) APK_EMBED_GEN(q6k, 2) APK_EMBED_GEN(q2k, 4) APK_EMBED_GEN(q3k, 5) APK_EMBED_GEN(q5_0, 6)
 APK_EMBED_GEN(f16, 7) APK_EMBED_GEN(f32, 8) APK_EMBED_GEN(bf16, 9)

@@ -39,6 +39,7 @@ SYMBOLS = {
     "apk_graph_nodes": (_i, [_vp, C.POINTER(_sz)]),
     "apk_graph_destroy": (_i, [_vp, _vp]),
     "apk_embed_rows": (_i, [_vp, _i, _vp, _sz, _sz, _vp, _sz, _vp, _i]),
+    "apk_embed_rows_scaled": (_i, [_vp, _i, _vp, _sz, _sz, _vp, _sz, _f, _vp, _i]),
     "apk_embed_rows_host_ids": (_i, [_vp, _i, _vp, _sz, _sz, _vp, _sz, _vp, _i]),
     "apk_add_rmsnorm_rows": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _f, _i]),
     "apk_qknorm_rope_neox": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _f, _i]),

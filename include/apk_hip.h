@@ -156,6 +156,12 @@ int apk_graph_destroy(apk_ctx* ctx, apk_graph* graph);
  * multiple of 8 and a row must fit 64 KiB (apk_can_embed tells). */
 int apk_embed_rows(apk_ctx* ctx, int fmt, const void* table, size_t vocab, size_t n_in, const uint32_t* ids,
                    size_t t, void* out, int out_dtype);
+/* The same followed by `*v *= scale` in f32 when scale != 1 (before the narrowing of an
+ * fp16 output): the embedding multiplier of models that scale their token embeddings
+ * (model/prefill.rs:107-109, model/decode.rs:427-429; the reference keeps such models on
+ * the CPU gather, model/decode.rs:93). */
+int apk_embed_rows_scaled(apk_ctx* ctx, int fmt, const void* table, size_t vocab, size_t n_in, const uint32_t* ids,
+                          size_t t, float scale, void* out, int out_dtype);
 /* Same with the ids on the host: range-checked BEFORE anything is enqueued
  * (APK_DECLINE_RANGE), as the reference's callers reject token >= vocab first. */
 int apk_embed_rows_host_ids(apk_ctx* ctx, int fmt, const void* table, size_t vocab, size_t n_in,

@@ -170,9 +170,14 @@ def quantmat_row(data, fmt, n_out, n_in, j, dst_len=None):
     return dst
 
 
-def embed_rows(data, fmt, vocab, n_in, ids, out_f16=False):
+def embed_rows(data, fmt, vocab, n_in, ids, out_f16=False, scale=1.0):
+    """QuantMat::row_into over ids; scale != 1: the `*v *= embed_scale` of model/prefill.rs:107-109
+    (one f32 multiply per element after the dequant), then the optional narrowing to fp16."""
     data = np.ascontiguousarray(data, dtype=np.uint8)
     ids = np.ascontiguousarray(ids, dtype=np.uint32)
+    if scale != 1.0:
+        rows = embed_rows(data, fmt, vocab, n_in, ids) * np.float32(scale)
+        return f32_to_f16_bits(rows) if out_f16 else rows
     out = np.zeros((ids.size, n_in), np.uint16 if out_f16 else np.float32)
     fn = lib().ora_embed_rows_f16 if out_f16 else lib().ora_embed_rows
     rc = fn(_p(data), data.size, fmt, vocab, n_in, _p(ids), ids.size, _p(out))

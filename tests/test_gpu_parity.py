@@ -126,6 +126,14 @@ def test_embed_all_ten_formats_bit_exact(be, ora, fmt_name, out_f16):
     got = host(out)
     assert np.array_equal(got.view(np.uint16 if out_f16 else np.uint32), want.view(np.uint16 if out_f16 else np.uint32))
     assert np.array_equal(host(qm.row(3, dtype=out.dtype)), want[0])  # token 3 of 6, as the reference's test
+    # models that scale their token embeddings: one f32 multiply after the dequant (prefill.rs:107-109;
+    # Gemma's factor is sqrt(hidden), here of a 3584-wide model)
+    scale = float(np.sqrt(np.float32(3584.0)))
+    want_s = ora.embed_rows(raw, fmt, vocab, hidden, ids, out_f16=out_f16, scale=scale)
+    assert not np.array_equal(want_s, want)
+    qm.rows_into(dev(ids), out, embed_scale=scale)
+    got = host(out)
+    assert np.array_equal(got.view(np.uint16 if out_f16 else np.uint32), want_s.view(np.uint16 if out_f16 else np.uint32))
 
 
 def test_embed_subnormal_scales_and_reference_vectors(be, ora):
