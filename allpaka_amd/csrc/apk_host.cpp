@@ -65,7 +65,7 @@ std::vector<std::string> all_kernel_names() {
     std::vector<std::string> v = {"apk_swiglu_f32", "apk_swiglu_f16", "apk_rope_table", "apk_embed_q4k_f32",
                                   "apk_embed_q4k_f16", "apk_embed_q8_0_f32", "apk_embed_q8_0_f16", "apk_route_topk",
                                   "apk_moe_permute", "apk_gather_rows", "apk_scatter_rows", "apk_argmax_rows", "apk_add_rmsnorm_ragged_f32", "apk_copy",
-                                  "apk_qknorm_rope_generic_f32", "apk_qknorm_rope_generic_f16"};
+                                  "apk_qknorm_rope_generic_f32", "apk_qknorm_rope_generic_f16", "apk_route_topk_wide"};
     for (const char* t : {"f32", "f16"}) {
         for (const char* f : {"q5k", "q6k", "q2k", "q3k", "q5_0", "f16", "f32", "bf16"}) v.push_back(std::string("apk_embed_") + f + "_" + t);
         for (int c : kAddnormTiles) v.push_back(std::string("apk_add_rmsnorm_") + t + "_c" + std::to_string(c));
@@ -762,7 +762,7 @@ int apk_route_topk(apk_ctx* c, const float* logits, const float* bias, size_t ro
                    float scale, int sigmoid, uint32_t* ids, float* w) {
     if (!c) return fail(APK_DECLINE_NULL, "apk_route_topk: ctx is NULL");
     CallScope s(c);
-    if (n_expert == 0 || n_expert > 256) return fail(APK_DECLINE_UNSUPPORTED, "apk_route_topk: n_expert %zu (1..256)", n_expert);
+    if (n_expert == 0 || n_expert > 1024) return fail(APK_DECLINE_UNSUPPORTED, "apk_route_topk: n_expert %zu (1..1024)", n_expert);
     if (k == 0 || k > n_expert || k > 64) return fail(APK_DECLINE_UNSUPPORTED, "apk_route_topk: k %zu", k);
     if (rows == 0) return APK_OK;
     if (!logits || !ids || !w) return fail(APK_DECLINE_NULL, "apk_route_topk: NULL tensor");
@@ -772,7 +772,7 @@ int apk_route_topk(apk_ctx* c, const float* logits, const float* bias, size_t ro
     const unsigned block = 256, per_block = block / 64;
     const uint64_t grid = (rows + per_block - 1) / per_block;
     void* args[] = {&logits, &bias, &rows_i, &ne_i, &k_i, &norm, &scale, &sigmoid, &ids, &w};
-    return launch(c, "apk_route_topk", (unsigned)grid, block, 0, args);
+    return launch(c, n_expert <= 256 ? "apk_route_topk" : "apk_route_topk_wide", (unsigned)grid, block, 0, args);
 }
 
 int apk_moe_permute(apk_ctx* c, const uint32_t* ids, const float* w, size_t rows, size_t k, size_t n_expert,

@@ -1117,10 +1117,10 @@ APK_EMBED_GEN(q5k, 1) APK_EMBED_GEN(q6k, 2) APK_EMBED_GEN(q2k, 4) APK_EMBED_GEN(
 APK_EMBED_GEN(f16, 7) APK_EMBED_GEN(f32, 8) APK_EMBED_GEN(bf16, 9)
 
 // =========================================================================
-// MoE router: per token softmax (or sigmoid) over n_expert <= 256 logits, top-k
+// MoE router: per token softmax (or sigmoid) over n_expert <= 64*EPL logits, top-k
 // by descending selection score with the LOWER INDEX winning ties, winners
 // renormalised (moe.rs:524-594).  One wave per token; lane l holds experts
-// l, l+64, l+128, l+192.  For softmax without bias the selection runs on the
+// l, l+64, l+128, ... (EPL of them).  For softmax without bias the selection runs on the
 // raw logits (same order as the probabilities, no dependence on exp rounding).
 // =========================================================================
 DEV float wave_max_f32(float v) {
@@ -1130,21 +1130,21 @@ DEV float wave_max_f32(float v) {
     return fmaxf(v, __shfl_xor(v, 32, 64));
 }
 DEV float wave_sum_f32(float v) { return group_sum<64>(v); }
-extern "C" __global__ __launch_bounds__(256) void apk_route_topk(const float* logits, const float* bias, int rows,
-                                                                int n_expert, int k, int norm, float scale,
-                                                                int sigmoid, uint32_t* ids, float* wout) {
+template <int EPL>  // experts per lane: the wave covers 64*EPL experts
+DEV void route_topk_body(const float* logits, const float* bias, int rows, int n_expert, int k, int norm, float scale,
+                         int sigmoid, uint32_t* ids, float* wout) {
     const int lane = threadIdx.x & 63;
     const uint64_t t = (uint64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (t >= (uint64_t)rows) return;  // whole wave exits together
     const float* lr = logits + t * (uint64_t)n_expert;
-    float lg[4], score[4];
-    uint32_t key[4];
+    float lg[EPL], score[EPL];
+    uint32_t key[EPL];
     float mx = -INFINITY;
-    float raw[4];
+    float raw[EPL];
 #pragma unroll
-    for (int j = 0; j < 4; j++) raw[j] = lr[min(lane + 64 * j, n_expert - 1)];  // all four loads in flight, no branch
+    for (int j = 0; j < EPL; j++) raw[j] = lr[min(lane + 64 * j, n_expert - 1)];  // every load in flight, no branch
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
+    for (int j = 0; j < EPL; j++) {
         const int e = lane + 64 * j;
         lg[j] = e < n_expert ? raw[j] : -INFINITY;
         if (e < n_expert) mx = fmaxf(mx, lg[j]);
@@ -1153,7 +1153,7 @@ extern "C" __global__ __launch_bounds__(256) void apk_route_topk(const float* lo
         mx = wave_max_f32(mx);
         float sum = 0.0f;
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int j = 0; j < EPL; j++) {
             const int e = lane + 64 * j;
             score[j] = e < n_expert ? expf(lg[j] - mx) : 0.0f;
             sum += score[j];
@@ -1161,28 +1161,28 @@ extern "C" __global__ __launch_bounds__(256) void apk_route_topk(const float* lo
         sum = wave_sum_f32(sum);
         const float inv = 1.0f / sum;
 #pragma unroll
-        for (int j = 0; j < 4; j++) score[j] *= inv;
+        for (int j = 0; j < EPL; j++) score[j] *= inv;
     } else {
 #pragma unroll
-        for (int j = 0; j < 4; j++) score[j] = 1.0f / (1.0f + expf(-lg[j]));
+        for (int j = 0; j < EPL; j++) score[j] = 1.0f / (1.0f + expf(-lg[j]));
     }
     const bool on_logits = !sigmoid && bias == nullptr;
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
+    for (int j = 0; j < EPL; j++) {
         const int e = lane + 64 * j;
         float sel = on_logits ? lg[j] : (bias != nullptr && e < n_expert ? score[j] + bias[e] : score[j]);
         key[j] = total_order_key(sel);
     }
     uint32_t taken = 0;
 #pragma unroll
-    for (int j = 0; j < 4; j++)
+    for (int j = 0; j < EPL; j++)
         if (lane + 64 * j >= n_expert) taken |= 1u << j;
     uint32_t my_id = 0;
     float my_score = 0.0f, total = 0.0f;
     for (int r = 0; r < k; r++) {
         uint64_t best = 0;  // (key << 32) | ~index; 0 = nothing left on this lane
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int j = 0; j < EPL; j++) {
             if (!(taken & (1u << j))) {
                 uint64_t cand = ((uint64_t)key[j] << 32) | (uint64_t)(0xffffffffu - (uint32_t)(lane + 64 * j));
                 best = cand > best ? cand : best;
@@ -1194,7 +1194,8 @@ extern "C" __global__ __launch_bounds__(256) void apk_route_topk(const float* lo
         float s = 0.0f;
         if (lane == owner) {
             taken |= 1u << slot;
-            s = slot == 0 ? score[0] : (slot == 1 ? score[1] : (slot == 2 ? score[2] : score[3]));
+#pragma unroll
+            for (int j = 0; j < EPL; j++) s = slot == j ? score[j] : s;  // selects, not an indexed (scratch) read
         }
         s = __shfl(s, owner, 64);
         total += s;  // best-first sequential f32 sum, as the reference's iterator sum
@@ -1208,6 +1209,18 @@ extern "C" __global__ __launch_bounds__(256) void apk_route_topk(const float* lo
         ids[t * (uint64_t)k + lane] = my_id;
         wout[t * (uint64_t)k + lane] = w * scale;
     }
+}
+
+extern "C" __global__ __launch_bounds__(256) void apk_route_topk(const float* logits, const float* bias, int rows,
+                                                                int n_expert, int k, int norm, float scale,
+                                                                int sigmoid, uint32_t* ids, float* wout) {
+    route_topk_body<4>(logits, bias, rows, n_expert, k, norm, scale, sigmoid, ids, wout);
+}
+// routers wider than 256 experts (the reference's heap path, moe.rs:536-545): up to 1024
+extern "C" __global__ __launch_bounds__(256) void apk_route_topk_wide(const float* logits, const float* bias, int rows,
+                                                                     int n_expert, int k, int norm, float scale,
+                                                                     int sigmoid, uint32_t* ids, float* wout) {
+    route_topk_body<16>(logits, bias, rows, n_expert, k, norm, scale, sigmoid, ids, wout);
 }
 
 // =========================================================================

@@ -243,7 +243,7 @@ int apk_swiglu(apk_ctx* ctx, void* gate, const void* up, size_t n, int dtype);
  * weights renormalised over the winners when norm != 0, then * scale.  Replaces
  * model::route_gated / route_gated_into_slice per token (model/moe.rs:524-616,
  * token loop :204-227).  logits: f32[rows][n_expert]; ids: u32[rows][k];
- * w: f32[rows][k], both best-first.  n_expert <= 256, 1 <= k <= min(n_expert, 64). */
+ * w: f32[rows][k], both best-first.  n_expert <= 1024, 1 <= k <= min(n_expert, 64). */
 int apk_route_topk(apk_ctx* ctx, const float* logits, const float* bias, size_t rows, size_t n_expert, size_t k,
                    int norm, float scale, int sigmoid, uint32_t* ids, float* w);
 

@@ -513,7 +513,8 @@ def _ref_logits(n):
     return np.float32([((i * 37 % 331) - 165.0) * 0.03 for i in range(n)])
 
 
-@pytest.mark.parametrize("rows,n_expert,k", [(1024, 128, 8), (1, 128, 8), (7, 64, 4), (33, 256, 8), (5, 60, 6), (3, 4, 4), (9, 200, 1)])
+@pytest.mark.parametrize("rows,n_expert,k", [(1024, 128, 8), (1, 128, 8), (7, 64, 4), (33, 256, 8), (5, 60, 6), (3, 4, 4), (9, 200, 1),
+                                            (40, 257, 8), (17, 384, 6), (5, 1024, 8), (3, 1000, 64)])
 @pytest.mark.parametrize("norm,scale", [(True, 1.0), (False, 1.5)])
 def test_route_topk(be, ora, rows, n_expert, k, norm, scale):
     s = synth()
@@ -558,10 +559,27 @@ def test_route_reference_vectors_ties_sigmoid_bias(be, ora):
     # route(probs, k) of the reference's test (gpu_eligible_forward.rs:88-97) through log-probabilities
     got = be.route_gated(dev(np.log(np.float32([0.1, 0.5, 0.15, 0.25]))), 2)
     assert [e for e, _ in got] == [1, 3] and abs(got[0][1] - 2 / 3) < 1e-6 and abs(got[1][1] - 1 / 3) < 1e-6
-    # k clamps to n; more than 256 experts is declined
+    # k clamps to n
     assert len(be.route_gated(dev(t[:4].copy()), 8)) == 4
+    # the reference's stack/heap boundary (moe.rs:680-715): a 257th expert that can never win leaves
+    # the picks and weights of the 256-expert router as they were, for every gating
+    wide = np.append(base, np.float32(-np.inf))
+    for gating, norm in [(apk.Gating.Softmax, True), (apk.Gating.Softmax, False), (apk.Gating.Sigmoid, True)]:
+        for k in (1, 8):
+            a, b = be.route_gated(dev(base), k, gating, norm, 1.5), be.route_gated(dev(wide), k, gating, norm, 1.5)
+            assert [e for e, _ in a] == [e for e, _ in b]
+            assert np.allclose([x for _, x in a], [x for _, x in b], rtol=0, atol=1e-6)
+    wide_bias = np.append(bias, np.float32(0.0))
+    a = be.route_gated(dev(base), 8, apk.Gating.Sigmoid, True, 2.5, dev(bias))
+    b = be.route_gated(dev(wide), 8, apk.Gating.Sigmoid, True, 2.5, dev(wide_bias))
+    assert [e for e, _ in a] == [e for e, _ in b] and np.allclose([x for _, x in a], [x for _, x in b], rtol=0, atol=1e-6)
+    # wide routers pick the true top-k, best first (moe.rs:719-726)
+    w320 = _ref_logits(320)
+    got = be.route_gated(dev(w320), 4, apk.Gating.Softmax, False, 1.0)
+    assert [e for e, _ in got] == list(np.argsort(-w320, kind="stable")[:4]) == list(ora.route_gated(w320, 4, ora.SOFTMAX, False, 1.0)[0])
+    # more than 1024 experts is declined
     with pytest.raises(apk.Declined):
-        be.route_gated(dev(_ref_logits(320)), 4)
+        be.route_gated(dev(np.zeros(1025, np.float32)), 4)
 
 
 # ------------------------------------------------------- grouping and gather
