@@ -150,10 +150,21 @@ class Backend:
         self._leave()
 
     def add_assign_slice(self, a, b):
-        """ops::add_assign_slice (blas.rs:105) -- on the device this op only exists
-        fused in front of a norm; see add_rmsnorm_rows."""
+        """ops::add_assign_slice (blas.rs:105): a += b.  Where a norm follows, add_rmsnorm_rows
+        does both in one pass."""
         assert a.numel() == b.numel()
-        raise Declined(_l.DECLINE_UNSUPPORTED, "residual add is fused into add_rmsnorm_rows on the device")
+        assert a.dtype == b.dtype
+        self._enter()
+        check(self.L.apk_add_assign(self.h, _ptr(a), _ptr(b), a.numel(), _dt(a)))
+        self._leave()
+
+    def softmax(self, x):
+        """ops::softmax (activation.rs:5) over each row of x (or over a 1-D x), in place."""
+        assert x.dtype == torch.float32
+        rows, n = (1, x.numel()) if x.dim() == 1 else (x.shape[0], x.shape[1])
+        self._enter()
+        check(self.L.apk_softmax_rows(self.h, _ptr(x), rows, n))
+        self._leave()
 
     def add_rmsnorm_rows(self, x, delta, h, gamma, eps):
         """x += delta; h = rmsnorm(x) * gamma, rows = x.len() / gamma.len()

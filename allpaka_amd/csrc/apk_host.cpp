@@ -65,7 +65,7 @@ std::vector<std::string> all_kernel_names() {
     std::vector<std::string> v = {"apk_swiglu_f32", "apk_swiglu_f16", "apk_rope_table", "apk_embed_q4k_f32",
                                   "apk_embed_q4k_f16", "apk_embed_q8_0_f32", "apk_embed_q8_0_f16", "apk_route_topk",
                                   "apk_moe_permute", "apk_gather_rows", "apk_scatter_rows", "apk_argmax_rows", "apk_add_rmsnorm_ragged_f32", "apk_copy",
-                                  "apk_qknorm_rope_generic_f32", "apk_qknorm_rope_generic_f16", "apk_route_topk_wide"};
+                                  "apk_qknorm_rope_generic_f32", "apk_qknorm_rope_generic_f16", "apk_route_topk_wide", "apk_add_assign_f32", "apk_add_assign_f16", "apk_softmax_rows"};
     for (const char* t : {"f32", "f16"}) {
         for (const char* f : {"q5k", "q6k", "q2k", "q3k", "q5_0", "f16", "f32", "bf16"}) v.push_back(std::string("apk_embed_") + f + "_" + t);
         for (int c : kAddnormTiles) v.push_back(std::string("apk_add_rmsnorm_") + t + "_c" + std::to_string(c));
@@ -480,6 +480,39 @@ int apk_swiglu(apk_ctx* c, void* gate, const void* up, size_t n, int dtype) {
     uint64_t n64 = n;
     void* args[] = {&gate, &up, &n64};
     return launch(c, dtype == APK_F32 ? "apk_swiglu_f32" : "apk_swiglu_f16", (unsigned)grid, block, 0, args);
+}
+
+int apk_add_assign(apk_ctx* c, void* a, const void* b, size_t n, int dtype) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_add_assign: ctx is NULL");
+    CallScope s(c);
+    const int es = elem_size(dtype);
+    if (!es) return fail(APK_DECLINE_UNSUPPORTED, "apk_add_assign: dtype %d", dtype);
+    if (n == 0) return APK_OK;
+    if (!a || !b) return fail(APK_DECLINE_NULL, "apk_add_assign: NULL tensor");
+    if (!aligned16(a) || !aligned16(b)) return fail(APK_DECLINE_SHAPE, "apk_add_assign: tensors must be 16-byte aligned");
+    if (int rc = set_device(c)) return rc;
+    const uint64_t nvec = n / (16 / es);
+    uint64_t grid = (nvec + 255) / 256;
+    if (grid == 0) grid = 1;
+    if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_add_assign: n too large");
+    uint64_t n64 = n;
+    void* args[] = {&a, &b, &n64};
+    return launch(c, dtype == APK_F32 ? "apk_add_assign_f32" : "apk_add_assign_f16", (unsigned)grid, 256, 0, args);
+}
+
+int apk_softmax_rows(apk_ctx* c, float* x, size_t rows, size_t n) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_softmax_rows: ctx is NULL");
+    CallScope s(c);
+    if (rows == 0 || n == 0) return APK_OK;
+    if (!x) return fail(APK_DECLINE_NULL, "apk_softmax_rows: NULL tensor");
+    // the reference sums a row's exponentials one after the other in f32; a parallel sum stays
+    // within 1e-5 of that only while rows are short (router widths), so longer rows are declined
+    if (n > 4096) return fail(APK_DECLINE_UNSUPPORTED, "apk_softmax_rows: rows of %zu (at most 4096)", n);
+    if (rows > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_softmax_rows: too large");
+    if (int rc = set_device(c)) return rc;
+    int rows_i = (int)rows, n_i = (int)n;
+    void* args[] = {&x, &rows_i, &n_i};
+    return launch(c, "apk_softmax_rows", (unsigned)((rows + 3) / 4), 256, 0, args);
 }
 
 int apk_add_rmsnorm_rows(apk_ctx* c, void* x, const void* delta, void* h, const float* gamma, size_t n, size_t rows,

@@ -210,6 +210,51 @@ extern "C" __global__ __launch_bounds__(256) void apk_swiglu_f16(f16_t* gate, co
     swiglu_body<f16_t, APK_SWIGLU_UNR>(gate, up, n);
 }
 
+// Residual add on its own: a[i] += b[i] (ops::add_assign_slice, blas.rs:105-178), for the
+// places where no norm follows.  One 16-byte tile per lane, a scalar tail for ragged n.
+template <typename T> DEV void add_assign_body(T* a, const T* b, uint64_t n) {
+    constexpr int VEC = io<T>::VEC;
+    const uint64_t nvec = n / VEC, c = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c < nvec) {
+        float x[VEC], y[VEC];
+        io<T>::load_nt(a + c * VEC, x);
+        io<T>::load_nt(b + c * VEC, y);
+#pragma unroll
+        for (int i = 0; i < VEC; i++) x[i] += y[i];
+        io<T>::store_nt(a + c * VEC, x);
+    }
+    if (blockIdx.x == gridDim.x - 1)
+        for (uint64_t i = nvec * VEC + threadIdx.x; i < n; i += blockDim.x) a[i] = (T)((float)a[i] + (float)b[i]);
+}
+extern "C" __global__ __launch_bounds__(256) void apk_add_assign_f32(float* a, const float* b, uint64_t n) {
+    add_assign_body<float>(a, b, n);
+}
+extern "C" __global__ __launch_bounds__(256) void apk_add_assign_f16(f16_t* a, const f16_t* b, uint64_t n) {
+    add_assign_body<f16_t>(a, b, n);
+}
+
+// Softmax over rows in place (ops::softmax, activation.rs:5-16): max, exp(v - max), sum,
+// times 1/sum.  A wave per row, any row length; the sum runs in lane order, not index order.
+extern "C" __global__ __launch_bounds__(256) void apk_softmax_rows(float* x, int rows, int n) {
+    const int lane = threadIdx.x & 63;
+    const uint64_t r = ((uint64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    if (r >= (uint64_t)rows) return;  // whole wave
+    float* row = x + r * (uint64_t)n;
+    float mx = -INFINITY;
+    for (int i = lane; i < n; i += 64) mx = fmaxf(mx, row[i]);
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    float sum = 0.0f;
+    for (int i = lane; i < n; i += 64) {
+        const float e = expf(row[i] - mx);
+        row[i] = e;
+        sum += e;
+    }
+    sum = group_sum<64>(sum);
+    const float inv = 1.0f / sum;
+    for (int i = lane; i < n; i += 64) row[i] *= inv;  // each lane re-reads only what it wrote
+}
+
 // =========================================================================
 // Residual add + RMSNorm over rows (blas.rs:105-178 then norm.rs:193-269):
 //   x' = x + delta  (written back when delta != null)

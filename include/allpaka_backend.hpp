@@ -146,6 +146,21 @@ inline void rope_neox_cached_from_array(std::vector<float>& x, const std::vector
     dx.read_back(x.data());
 }
 
+// ops::add_assign_slice(a, b): a += b (blas.rs:105); a shorter or longer b panics.
+inline void add_assign_slice(std::vector<float>& a, const std::vector<float>& b) {
+    if (a.size() != b.size()) throw Panic("assertion `left == right` failed: a.len() == b.len()");
+    Dev<float> da(a.data(), a.size()), db(b.data(), b.size());
+    check(apk_add_assign(Gpu::get().ctx(), da.ptr(), db.ptr(), a.size(), APK_F32));
+    da.read_back(a.data());
+}
+
+// ops::softmax(x) in place (activation.rs:5).
+inline void softmax(std::vector<float>& x) {
+    Dev<float> dx(x.data(), x.size());
+    check(apk_softmax_rows(Gpu::get().ctx(), dx.ptr(), 1, x.size()));
+    dx.read_back(x.data());
+}
+
 // ops::rope_norm_cached_from_array(x, table): adjacent pairs (2i, 2i+1) rotate (rope.rs:52).
 inline void rope_norm_cached_from_array(std::vector<float>& x, const std::vector<std::array<float, 2>>& table) {
     if (x.size() < table.size() * 2) throw Panic("assertion failed: x.len() >= table.len() * 2");

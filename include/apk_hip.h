@@ -167,6 +167,16 @@ int apk_embed_rows_scaled(apk_ctx* ctx, int fmt, const void* table, size_t vocab
 int apk_embed_rows_host_ids(apk_ctx* ctx, int fmt, const void* table, size_t vocab, size_t n_in,
                             const uint32_t* ids_host, size_t t, void* out, int out_dtype);
 
+/* Residual add on its own: a[i] += b[i].  Replaces ops::add_assign_slice / add_assign_par
+ * (ops/blas.rs:105-213) where no norm follows (where one does, apk_add_rmsnorm_rows does
+ * both in one pass).  Any n; bit-exact (fp16: widen, add in f32, one rounding). */
+int apk_add_assign(apk_ctx* ctx, void* a, const void* b, size_t n, int dtype);
+/* Softmax over rows of f32 in place.  Replaces ops::softmax (ops/activation.rs:5-16) per
+ * row; the router's softmax is fused into apk_route_topk, this is the op on its own.
+ * Rows of at most 4096 (router widths): the reference adds the exponentials one after the
+ * other in f32, which a parallel sum matches to 1e-5 only for short rows; longer declined. */
+int apk_softmax_rows(apk_ctx* ctx, float* x, size_t rows, size_t n);
+
 /* Residual add + RMSNorm over rows: x += delta (skipped when delta is NULL), then
  * h = rmsnorm(x) * gamma.  Replaces ops::add_assign_slice followed by
  * ops::rmsnorm_into / rmsnorm_rows_into (ops/blas.rs:105-178, ops/norm.rs:193-304;

@@ -75,6 +75,20 @@ static void swiglu_is_silu_of_gate_times_up() {  // :172-185, silu fixed points 
     CHECK(g[0] == 0.0f && close(g[1], 1.0f / (1.0f + std::exp(-1.0f))) && std::fabs(g[2]) < 1e-7f && close(g[3], 20.0f));
     CHECK(throws<Panic>([] { std::vector<float> g(4), u(3); ops::swiglu(g, u); }));
 }
+static void softmax_sums_to_one_and_survives_huge_logits() {  // ops/mod.rs:147-161
+    std::vector<float> x = {1.0f, 3.0f, 2.0f};
+    ops::softmax(x);
+    CHECK(close(x[0] + x[1] + x[2], 1.0f) && x[1] > x[2] && x[2] > x[0]);
+    std::vector<float> y = {1000.0f, 999.0f};
+    ops::softmax(y);
+    CHECK(std::isfinite(y[0]) && std::isfinite(y[1]) && close(y[0] + y[1], 1.0f));
+}
+static void add_assign_slice_adds_and_rejects_length_mismatch() {  // ops/mod.rs:394-408
+    std::vector<float> a = {1.0f, 2.0f, 3.0f, 4.0f, 5.0f}, b = {0.5f, -2.0f, 10.0f, 0.25f, -5.0f};
+    ops::add_assign_slice(a, b);
+    CHECK((a == std::vector<float>{1.5f, 0.0f, 13.0f, 4.25f, 0.0f}));
+    CHECK(throws<Panic>([] { std::vector<float> a(8), b(7); ops::add_assign_slice(a, b); }));
+}
 static std::vector<std::array<float, 2>> table_for(uint32_t pos, size_t head_dim, float base) {  // rope.rs:8-22
     std::vector<std::array<float, 2>> t(head_dim / 2);
     for (size_t i = 0; i < head_dim / 2; i++) {
@@ -168,6 +182,8 @@ int main() {
         {"rmsnorm_rows_into_rejects_a_short_destination", rmsnorm_rows_into_rejects_a_short_destination},
         {"add_assign_then_norm_matches_the_two_ops", add_assign_then_norm_matches_the_two_ops},
         {"swiglu_is_silu_of_gate_times_up", swiglu_is_silu_of_gate_times_up},
+        {"softmax_sums_to_one_and_survives_huge_logits", softmax_sums_to_one_and_survives_huge_logits},
+        {"add_assign_slice_adds_and_rejects_length_mismatch", add_assign_slice_adds_and_rejects_length_mismatch},
         {"rope_is_norm_preserving_and_identity_at_position_zero", rope_is_norm_preserving_and_identity_at_position_zero},
         {"rope_neox_pairs_split_channels", rope_neox_pairs_split_channels},
         {"partial_rotary_rotates_the_head_and_passes_the_tail", partial_rotary_rotates_the_head_and_passes_the_tail},

@@ -508,6 +508,54 @@ def test_swiglu_reference_sweep_and_assert(be, ora):
         be.swiglu(torch.zeros(4, device="cuda"), torch.zeros(3, device="cuda"))
 
 
+# ------------------------------------------------- residual add, softmax alone
+@pytest.mark.parametrize("n", [1, 3, 8, 1024, 5120 * 6 + 5, 65536 * 3 + 1])
+@pytest.mark.parametrize("f16", [False, True])
+def test_add_assign_slice_bit_exact(be, ora, n, f16):
+    s = synth()
+    g = s.rng(1, n)
+    a, b = s.normal_f32(g, n), s.normal_f32(g, n)
+    if f16:
+        a16, b16 = s.to_f16_bits(a), s.to_f16_bits(b)
+        want = ora.f32_to_f16_bits(ora.f16_bits_to_f32(a16) + ora.f16_bits_to_f32(b16))
+        ta, tb = dev(a16), dev(b16)
+    else:
+        want = a.copy()
+        ora.add_assign_slice(want, b)
+        ta, tb = dev(a), dev(b)
+    be.add_assign_slice(ta, tb)
+    assert np.array_equal(host(ta), want)
+    assert np.array_equal(host(tb), b16 if f16 else b)  # the addend is only read
+    with pytest.raises(AssertionError):  # blas.rs: a shorter source panics (ops/mod.rs:394-408)
+        be.add_assign_slice(ta, tb[:-1])
+
+
+@pytest.mark.parametrize("rows,n", [(1, 3), (1, 128), (5, 256), (1024, 128), (3, 1000), (2, 4096)])
+def test_softmax_rows(be, ora, rows, n):
+    s = synth()
+    x = s.normal_f32(s.rng(4, rows * 7 + n), (rows, n), 0.0, 3.0)
+    want = x.copy()
+    for r in range(rows):
+        ora.softmax(want[r])
+    t = dev(x)
+    be.softmax(t)
+    got = host(t)
+    assert rel_err_f32(got, want) <= TOL_F32
+    assert np.allclose(got.sum(axis=1, dtype=np.float64), 1.0, atol=1e-5)
+    # the reference's vectors (ops/mod.rs:147-161): order kept, sums to 1; huge logits stay finite
+    v = dev(np.float32([1.0, 3.0, 2.0]))
+    be.softmax(v)
+    h = host(v)
+    assert h[1] > h[2] > h[0] and abs(h.sum() - 1.0) < 1e-6
+    v = dev(np.float32([1000.0, 999.0]))
+    be.softmax(v)
+    assert np.all(np.isfinite(host(v))) and abs(host(v).sum() - 1.0) < 1e-6
+    import allpaka_amd as apk
+
+    with pytest.raises(apk.Declined):  # vocabulary-sized rows: the sequential f32 sum is not reproducible to 1e-5
+        be.softmax(torch.zeros(4097, device="cuda"))
+
+
 # --------------------------------------------------------------------- router
 def _ref_logits(n):
     return np.float32([((i * 37 % 331) - 165.0) * 0.03 for i in range(n)])
