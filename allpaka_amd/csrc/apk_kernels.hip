@@ -609,21 +609,19 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
         io<float>::load(wp + HALF + EPL * l + i, wb + i);
     }
     typename io<T>::raw_t araw[ITER], braw[ITER], varaw[ITER], vbraw[ITER];
-    T* hp[ITER];
-    int hoff[ITER];
-    bool live[ITER];
+    // head of pass `it` and its element offset: recomputed where needed (a few integer
+    // operations) rather than kept in registers across the loads
+    const int hh_first = g * ITER * HPW + sub;
+    auto head_off = [&](int it) { return min(hh_first + it * HPW, nheads - 1) * HD + EPL * l; };
 #pragma unroll
     for (int it = 0; it < ITER; it++) {
-        const int hh0 = (g * ITER + it) * HPW + sub;
-        live[it] = hh0 < nheads;
-        hoff[it] = min(hh0, nheads - 1) * HD;
-        hp[it] = base + hoff[it];
+        const int off = head_off(it);
         __builtin_amdgcn_sched_barrier(0);  // loads stay in program order (returns are in order)
-        araw[it] = io<T>::ldraw_nt(hp[it] + EPL * l);
-        braw[it] = io<T>::ldraw_nt(hp[it] + HALF + EPL * l);
+        araw[it] = io<T>::ldraw_nt(base + off);
+        braw[it] = io<T>::ldraw_nt(base + off + HALF);
         if constexpr (KV) {
-            varaw[it] = io<T>::ldraw_nt(vrow + hoff[it] + EPL * l);
-            vbraw[it] = io<T>::ldraw_nt(vrow + hoff[it] + HALF + EPL * l);
+            varaw[it] = io<T>::ldraw_nt(vrow + off);
+            vbraw[it] = io<T>::ldraw_nt(vrow + off + HALF);
         }
     }
     __builtin_amdgcn_sched_barrier(0);  // every load above; all uses below
@@ -670,19 +668,21 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
                 ob[i] = x * s + y * c;
             }
         }
-        if (live[it]) {
-            io<T>::store_nt(hp[it] + EPL * l, oa);
-            io<T>::store_nt(hp[it] + HALF + EPL * l, ob);
+        const bool live = hh_first + it * HPW < nheads;
+        const int off = head_off(it);
+        if (live) {
+            io<T>::store_nt(base + off, oa);
+            io<T>::store_nt(base + off + HALF, ob);
         }
         if constexpr (KV) {
-            if (live[it] && kc != nullptr) {  // kc == nullptr: cache position out of range, row skipped
+            if (live && kc != nullptr) {  // kc == nullptr: cache position out of range, row skipped
                 float va[EPL], vb[EPL];
                 io<T>::widen(varaw[it], va);
                 io<T>::widen(vbraw[it], vb);
-                store_f16_tile<T>(kc + hoff[it] + EPL * l, oa);
-                store_f16_tile<T>(kc + hoff[it] + HALF + EPL * l, ob);
-                store_f16_tile<T>(vc + hoff[it] + EPL * l, va);
-                store_f16_tile<T>(vc + hoff[it] + HALF + EPL * l, vb);
+                store_f16_tile<T>(kc + off, oa);
+                store_f16_tile<T>(kc + off + HALF, ob);
+                store_f16_tile<T>(vc + off, va);
+                store_f16_tile<T>(vc + off + HALF, vb);
             }
         }
         __builtin_amdgcn_sched_barrier(0);  // pass by pass: pass it+1 waits only for its own tiles
@@ -721,8 +721,11 @@ DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const fl
         }
     }
 }
+// At most 128 VGPRs (4 waves per SIMD): the q waves of a 2048-row batch are 8 per CU and the k
+// waves another 8, so at 16 resident waves per CU the whole launch is one round with no tail.
+#define APK_QK_OCC __attribute__((amdgpu_waves_per_eu(4)))
 #define APK_QKROPE(T, TN, HD, ITER)                                                                          \
-    extern "C" __global__ __launch_bounds__(256) void apk_qknorm_rope_##TN##_hd##HD##_i##ITER(              \
+    extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void apk_qknorm_rope_##TN##_hd##HD##_i##ITER(   \
         T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv, float eps) { \
         qknorm_rope_body<T, HD, ITER>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, blockIdx.x);                  \
     }
@@ -736,7 +739,7 @@ APK_QKROPE_ALL(f16_t, f16)
 // The same with the K/V cache store fused in: rotated k and the row's v narrowed to fp16
 // at cache row cache_pos[row] (one launch instead of QK-norm+RoPE, then two narrowing copies).
 #define APK_QKROPE_KV(T, TN, HD, ITER)                                                                            \
-    extern "C" __global__ __launch_bounds__(256) void apk_qknorm_rope_kv_##TN##_hd##HD##_i##ITER(                \
+    extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void apk_qknorm_rope_kv_##TN##_hd##HD##_i##ITER(     \
         T* q, T* k, const T* v, const float* qw, const float* kw, const float* rope, const uint32_t* cache_pos,  \
         f16_t* k_cache, f16_t* v_cache, uint32_t capacity, int rows, int n_q, int n_kv, float eps, uint32_t* fault) { \
         qknorm_rope_body<T, HD, ITER, true>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, blockIdx.x, v, cache_pos,   \

@@ -169,6 +169,18 @@ def main():
     record("copy (plain stream)", f"{cp_bytes >> 20} MiB -> {cp_bytes >> 20} MiB",
            timed(lambda i: apklib.check(L.apk_copy(h, p(sw[i % len(sw)]["up"]), p(sw[i % len(sw)]["gate"]), cp_bytes)), reps), 2 * cp_bytes)
 
+    # The practical ceiling at each op's size: a plain copy (one 16-byte tile per lane, out of place) moving
+    # the same number of bytes.  Every launch pays a fixed ~2 us before it streams at ~6.8 TB/s, so a
+    # ~76 MB op cannot reach the fraction of peak a 300 MB op does.
+    cp_pool = torch.zeros(int(COLD_BYTES * 1.1), dtype=torch.uint8, device=dev)
+    torch.cuda.synchronize()
+    for name, nb in (("add_rmsnorm", bytes_addnorm), ("qknorm_rope_neox", bytes_qkrope), ("embed_rows Q4_K->f16", T * (2880 + 4 + H * 2))):
+        half = nb // 2 // 4096 * 4096
+        nset = cp_pool.numel() // (2 * half)
+        us = timed(lambda i: apklib.check(L.apk_copy(h, p(cp_pool) + (i % nset) * 2 * half, p(cp_pool) + (i % nset) * 2 * half + half, half)), reps)
+        record(f"copy (plain stream) of the bytes of {name}", f"{2 * half / 1e6:.1f} MB moved", us, 2 * half, note="ceiling at this size")
+    del cp_pool
+
     if args.shapes == "all":
         # small-T shapes of the same model: launch-latency bound, reported as us/launch
         for rows, label in ((1, "decode T=1"), (6, "verify T=6"), (64, "batched decode, 64 rows with own positions")):
