@@ -495,6 +495,33 @@ def test_swiglu(be, ora, n, f16):
         assert rel_err_f32(got, want) <= TOL_F32 and close_idiom(got, want)
 
 
+def test_swiglu_f32_strict_relative_error_over_the_whole_range(be, ora):
+    """Element by element (no floor): every normal result within 1e-5 of the reference's
+    g / (1 + exp(-g)) * u, from the underflow edge of exp to its overflow edge, and the same
+    zeros / infinities / NaNs outside it."""
+    g = np.concatenate([np.linspace(-104.0, 104.0, 400001), synth().normal_f32(synth().rng(4, 1), 300000, 0.0, 4.0),
+                        [0.0, -0.0, 1e-30, -1e-30, 88.7, -88.7, 88.73, -88.73, -87.3, 120.0, -120.0, 3e38, -3e38, np.inf, -np.inf,
+                         np.nan, 0.0]]).astype(np.float32)
+    up = np.ones_like(g)
+    up[-1] = np.nan
+    want = g.copy()
+    with np.errstate(all="ignore"):
+        ora.swiglu(want, up)
+    tg = dev(g)
+    be.swiglu(tg, dev(up))
+    got = host(tg)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    ok = ~np.isnan(want)
+    normal = ok & (np.abs(want) >= np.float32(1.17549435e-38)) & np.isfinite(want)
+    rel = np.abs(got[normal].astype(np.float64) - want[normal]) / np.abs(want[normal].astype(np.float64))
+    assert rel.max() <= TOL_F32, (rel.max(), g[normal][rel.argmax()])
+    rest = ok & ~normal  # zeros, subnormal results, infinities: equal up to one subnormal step
+    assert np.all(np.isinf(got[rest]) == np.isinf(want[rest]))
+    fin = rest & np.isfinite(want)
+    assert np.max(np.abs(got[fin].astype(np.float64) - want[fin])) <= 2e-38
+    assert np.array_equal(np.signbit(got[fin & (want == 0)]), np.signbit(want[fin & (want == 0)]))
+
+
 def test_swiglu_reference_sweep_and_assert(be, ora):
     # ops/mod.rs:172-185
     gate = np.float32([i * 0.7 for i in range(-25, 26)])
