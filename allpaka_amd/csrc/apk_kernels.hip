@@ -414,9 +414,9 @@ APK_ADDNORM_ALL(f16_t, f16)
 //   (ops::add_scaled_slice, blas.rs:25-102, x86 arm: one rounding per hit);
 //   x += out;  h = rmsnorm(x) * gamma  (skipped when h is null).
 // Same row layout as add+RMSNorm: W waves per row, NCH tiles per lane; the k
-// expert rows of a token are streamed two hits at a time.
+// expert rows of a token are fetched HB hits at a time, all in flight together.
 // =========================================================================
-template <typename T, int NCH>
+template <typename T, int NCH, int HB>
 DEV void combine_add_rmsnorm_body(T* x, const T* flat, const uint32_t* tok_off, const uint32_t* hit_row,
                                   const float* hit_w, uint32_t total_rows, T* h, const float* gamma, int n, float eps,
                                   uint32_t* fault) {
@@ -439,29 +439,42 @@ DEV void combine_add_rmsnorm_body(T* x, const T* flat, const uint32_t* tok_off, 
     for (int j = 0; j < NCH; j++)
 #pragma unroll
         for (int i = 0; i < VEC; i++) acc[j][i] = 0.0f;
-    for (uint32_t k = h0; k < h1; k += 2) {  // uniform for the workgroup
-        const bool two = k + 1 < h1;
-        uint32_t r0 = hit_row[k], r1 = two ? hit_row[k + 1] : 0u;
-        const float w0 = hit_w[k], w1 = two ? hit_w[k + 1] : 0.0f;
-        const bool ok0 = r0 < total_rows, ok1 = two && r1 < total_rows;
-        if ((!ok0 || (two && !ok1)) && threadIdx.x == 0) atomicOr(fault, APK_FAULT_ROW_RANGE);
-        r0 = ok0 ? r0 : 0u;
-        r1 = ok1 ? r1 : 0u;
-        typename io<T>::raw_t d0[NCH], d1[NCH];
+    // HB hits at a time: their row numbers and weights first (uniform for the workgroup), then
+    // every tile of all HB expert rows in flight at once, then the multiply-adds in hit order (the
+    // order is the contract: one rounding per hit).  Slots past the token's last hit re-read its
+    // last row (a cache hit) and add nothing.
+    for (uint32_t kb = h0; kb < h1; kb += HB) {
+        uint32_t r[HB];
+        float w[HB];
+        bool use[HB];
+        bool bad = false;
 #pragma unroll
-        for (int j = 0; j < NCH; j++) {
-            d0[j] = io<T>::ldraw_nt(flat + (uint64_t)r0 * n + cidx[j] * VEC);
-            d1[j] = io<T>::ldraw_nt(flat + (uint64_t)r1 * n + cidx[j] * VEC);
+        for (int j = 0; j < HB; j++) {
+            const uint32_t kk = min(kb + (uint32_t)j, h1 - 1u);
+            r[j] = hit_row[kk];
+            w[j] = hit_w[kk];
+            const bool in_range = r[j] < total_rows;
+            use[j] = kb + (uint32_t)j < h1 && in_range;
+            bad |= !in_range;
+            r[j] = in_range ? r[j] : 0u;
         }
+        if (bad && threadIdx.x == 0) atomicOr(fault, APK_FAULT_ROW_RANGE);
+        typename io<T>::raw_t d[HB][NCH];
 #pragma unroll
-        for (int j = 0; j < NCH; j++) {
-            float a[VEC], b[VEC];
-            io<T>::widen(d0[j], a);
-            io<T>::widen(d1[j], b);
+        for (int j = 0; j < HB; j++)
 #pragma unroll
-            for (int i = 0; i < VEC; i++) {
-                if (ok0) acc[j][i] = __builtin_fmaf(a[i], w0, acc[j][i]);
-                if (ok1) acc[j][i] = __builtin_fmaf(b[i], w1, acc[j][i]);
+            for (int c = 0; c < NCH; c++) d[j][c] = io<T>::ldraw_nt(flat + (uint64_t)r[j] * n + cidx[c] * VEC);
+        __builtin_amdgcn_sched_barrier(0);  // every load above, every use below
+#pragma unroll
+        for (int j = 0; j < HB; j++) {
+            if (use[j]) {  // uniform
+#pragma unroll
+                for (int c = 0; c < NCH; c++) {
+                    float a[VEC];
+                    io<T>::widen(d[j][c], a);
+#pragma unroll
+                    for (int i = 0; i < VEC; i++) acc[c][i] = __builtin_fmaf(a[i], w[j], acc[c][i]);
+                }
             }
         }
     }
@@ -503,11 +516,13 @@ DEV void combine_add_rmsnorm_body(T* x, const T* flat, const uint32_t* tok_off, 
         }
     }
 }
+// 4 hits in flight: with 4 tiles per lane that is 16 loads per lane, the register budget of a
+// 1024-thread workgroup (8 hits in flight with 2 tiles per lane measured slower).
 #define APK_COMBINE(T, TN, NCH)                                                                                        \
     extern "C" __global__ __launch_bounds__(1024) void apk_combine_add_rmsnorm_##TN##_c##NCH(                         \
         T* x, const T* flat, const uint32_t* tok_off, const uint32_t* hit_row, const float* hit_w, uint32_t total_rows, \
         T* h, const float* gamma, int n, float eps, uint32_t* fault) {                                                 \
-        combine_add_rmsnorm_body<T, NCH>(x, flat, tok_off, hit_row, hit_w, total_rows, h, gamma, n, eps, fault);       \
+        combine_add_rmsnorm_body<T, NCH, 4>(x, flat, tok_off, hit_row, hit_w, total_rows, h, gamma, n, eps, fault);    \
     }
 APK_COMBINE(float, f32, 1) APK_COMBINE(float, f32, 2) APK_COMBINE(float, f32, 4)
 APK_COMBINE(f16_t, f16, 1) APK_COMBINE(f16_t, f16, 2) APK_COMBINE(f16_t, f16, 4)
