@@ -87,6 +87,7 @@ struct apk_ctx {
     hipModule_t module = nullptr;
     hipStream_t stream = nullptr;
     std::unordered_map<std::string, hipFunction_t> fn;
+    std::unordered_map<uint32_t, hipFunction_t> fn_by_key;  // (op, variant) -> function: no name building on the hot path
     uint32_t* fault_dev = nullptr;  // device status word
     uint32_t* ids_stage_host = nullptr;  // pinned staging for host-side token ids
     uint32_t* ids_stage_dev = nullptr;
@@ -120,15 +121,38 @@ struct CallScope {  // counts one ABI call and its host-side encode time
     ~CallScope() { c->encode_ns += now_ns() - t0; }
 };
 
+int launch_fn(apk_ctx* c, hipFunction_t f, const char* what, unsigned grid, unsigned block, unsigned shmem, void** args) {
+    hipError_t e = hipModuleLaunchKernel(f, grid, 1, 1, block, 1, 1, shmem, c->stream, args, nullptr);
+    if (e != hipSuccess) return hip_fail(e, what);
+    if (c->capturing) c->capture_nodes++;  // recorded, not run: counted when the graph is replayed
+    else c->dispatches++;
+    return APK_OK;
+}
+
 int launch(apk_ctx* c, const std::string& k, unsigned grid, unsigned block, unsigned shmem, void** args) {
     if (grid == 0) return APK_OK;
     auto it = c->fn.find(k);
     if (it == c->fn.end()) return fail(APK_DECLINE_UNSUPPORTED, "no kernel %s in the code object", k.c_str());
-    hipError_t e = hipModuleLaunchKernel(it->second, grid, 1, 1, block, 1, 1, shmem, c->stream, args, nullptr);
-    if (e != hipSuccess) return hip_fail(e, k.c_str());
-    if (c->capturing) c->capture_nodes++;  // recorded, not run: counted when the graph is replayed
-    else c->dispatches++;
-    return APK_OK;
+    return launch_fn(c, it->second, k.c_str(), grid, block, shmem, args);
+}
+
+// The same for the ops of the decode chain, where the host's cost per launch is what bounds
+// the chain: the kernel of an (op, variant) pair is looked up by an integer; its name is built
+// only the first time.
+enum OpId : uint32_t { OP_SWIGLU = 1, OP_ADDNORM, OP_QKROPE, OP_QKROPE_KV, OP_PROLOGUE, OP_ADD_ASSIGN, OP_EMBED, OP_ARGMAX };
+template <typename NameFn>
+int launch_keyed(apk_ctx* c, OpId op, uint32_t variant, NameFn&& name, unsigned grid, unsigned block, unsigned shmem,
+                 void** args) {
+    if (grid == 0) return APK_OK;
+    const uint32_t key = ((uint32_t)op << 24) | (variant & 0xffffffu);
+    auto it = c->fn_by_key.find(key);
+    if (it == c->fn_by_key.end()) {
+        const std::string k = name();
+        auto byname = c->fn.find(k);
+        if (byname == c->fn.end()) return fail(APK_DECLINE_UNSUPPORTED, "no kernel %s in the code object", k.c_str());
+        it = c->fn_by_key.emplace(key, byname->second).first;
+    }
+    return launch_fn(c, it->second, "hipModuleLaunchKernel", grid, block, shmem, args);
 }
 
 // Entries that allocate, copy to or from the host, or wait cannot run inside a recording.
@@ -479,7 +503,8 @@ int apk_swiglu(apk_ctx* c, void* gate, const void* up, size_t n, int dtype) {
     if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_swiglu: n too large");
     uint64_t n64 = n;
     void* args[] = {&gate, &up, &n64};
-    return launch(c, dtype == APK_F32 ? "apk_swiglu_f32" : "apk_swiglu_f16", (unsigned)grid, block, 0, args);
+    return launch_keyed(c, OP_SWIGLU, (uint32_t)dtype, [&] { return std::string(dtype == APK_F32 ? "apk_swiglu_f32" : "apk_swiglu_f16"); },
+                        (unsigned)grid, block, 0, args);
 }
 
 int apk_add_assign(apk_ctx* c, void* a, const void* b, size_t n, int dtype) {
@@ -497,7 +522,8 @@ int apk_add_assign(apk_ctx* c, void* a, const void* b, size_t n, int dtype) {
     if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_add_assign: n too large");
     uint64_t n64 = n;
     void* args[] = {&a, &b, &n64};
-    return launch(c, dtype == APK_F32 ? "apk_add_assign_f32" : "apk_add_assign_f16", (unsigned)grid, 256, 0, args);
+    return launch_keyed(c, OP_ADD_ASSIGN, (uint32_t)dtype,
+                        [&] { return std::string(dtype == APK_F32 ? "apk_add_assign_f32" : "apk_add_assign_f16"); }, (unsigned)grid, 256, 0, args);
 }
 
 int apk_softmax_rows(apk_ctx* c, float* x, size_t rows, size_t n) {
@@ -556,11 +582,12 @@ int apk_add_rmsnorm_rows(apk_ctx* c, void* x, const void* delta, void* h, const 
     }
     if (!nch) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: row of %zu elements is too long", n);
     const size_t threads = waves * 64;
-    const std::string which = std::string("apk_add_rmsnorm_") + (dtype == APK_F32 ? "f32" : "f16") + "_c" + std::to_string(nch);
     if (int rc = set_device(c)) return rc;
     int n_i = (int)n;
     void* args[] = {&x, &delta, &h, &gamma, &n_i, &eps};
-    return launch(c, which, (unsigned)rows, (unsigned)threads, 0, args);
+    return launch_keyed(c, OP_ADDNORM, (uint32_t)dtype << 8 | (uint32_t)nch,
+                        [&] { return std::string("apk_add_rmsnorm_") + (dtype == APK_F32 ? "f32" : "f16") + "_c" + std::to_string(nch); },
+                        (unsigned)rows, (unsigned)threads, 0, args);
 }
 
 struct KvStore {  // the fused K/V cache store of apk_qknorm_rope_kv_store (all NULL/0: plain op)
@@ -624,17 +651,20 @@ static int qknorm_rope_common(apk_ctx* c, void* q, void* k, const float* qw, con
     const uint64_t grid = (waves * 64 + block - 1) / block;
     if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope: too large");
     if (validate_only) return APK_OK;
-    const std::string which = std::string(kv ? "apk_qknorm_rope_kv_" : "apk_qknorm_rope_") + (dtype == APK_F32 ? "f32" : "f16") +
-                              "_hd" + std::to_string(head_dim) + "_i" + std::to_string(iter);
+    auto which = [&] {
+        return std::string(kv ? "apk_qknorm_rope_kv_" : "apk_qknorm_rope_") + (dtype == APK_F32 ? "f32" : "f16") + "_hd" +
+               std::to_string(head_dim) + "_i" + std::to_string(iter);
+    };
+    const uint32_t variant = (uint32_t)dtype << 16 | (uint32_t)head_dim << 4 | (uint32_t)iter;
     if (int rc = set_device(c)) return rc;
     if (kv) {
         uint32_t cap32 = (uint32_t)kv->capacity;
         void* kargs[] = {&q, &k, (void*)&kv->v, &qw, &kw, &rope, (void*)&kv->cache_pos, (void*)&kv->k_cache, (void*)&kv->v_cache,
                          &cap32, &rows_i, &nq_i, &nkv_i, &eps, &c->fault_dev};
-        return launch(c, which, (unsigned)grid, block, 0, kargs);
+        return launch_keyed(c, OP_QKROPE_KV, variant, which, (unsigned)grid, block, 0, kargs);
     }
     void* args[] = {&q, &k, &qw, &kw, &rope, &rows_i, &nq_i, &nkv_i, &eps};
-    return launch(c, which, (unsigned)grid, block, 0, args);
+    return launch_keyed(c, OP_QKROPE, variant, which, (unsigned)grid, block, 0, args);
 }
 
 int apk_qknorm_rope_neox(apk_ctx* c, void* q, void* k, const float* qw, const float* kw, const float* rope,
@@ -693,10 +723,11 @@ int apk_layer_prologue(apk_ctx* c, void* x, const void* delta, void* h, const fl
     const uint64_t wpb = threads / 64;
     const uint64_t grid = rows + (qk_waves + wpb - 1) / wpb;
     if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_layer_prologue: too large");
-    const std::string which = std::string("apk_layer_prologue_") + (dtype == APK_F32 ? "f32" : "f16") + "_hd" + std::to_string(head_dim);
     int n_i = (int)n, rows_i = (int)rows, nq_i = (int)n_q, nkv_i = (int)n_kv;
     void* args[] = {&x, &delta, &h, &gamma, &n_i, &q, &k, &qw, &kw, &rope, &rows_i, &nq_i, &nkv_i, &eps};
-    return launch(c, which, (unsigned)grid, (unsigned)threads, 0, args);
+    return launch_keyed(c, OP_PROLOGUE, (uint32_t)dtype << 16 | (uint32_t)head_dim,
+                        [&] { return std::string("apk_layer_prologue_") + (dtype == APK_F32 ? "f32" : "f16") + "_hd" + std::to_string(head_dim); },
+                        (unsigned)grid, (unsigned)threads, 0, args);
 }
 
 int apk_rope_table(apk_ctx* c, const uint32_t* positions, const float* inv_freq, size_t rows, size_t half, float* table) {
@@ -730,7 +761,9 @@ static int embed_common(apk_ctx* c, int fmt, const void* table, size_t vocab, si
         size_t threads = (n_in / 256 * 8 + 63) / 64 * 64;
         if (threads > 256) threads = 256;
         void* args[] = {&table, &vocab32, &n_i, &ids_dev, &out, &c->fault_dev, &scale};
-        return launch(c, out_dtype == APK_F32 ? "apk_embed_q4k_f32" : "apk_embed_q4k_f16", (unsigned)t, (unsigned)threads, 0, args);
+        return launch_keyed(c, OP_EMBED, (uint32_t)fmt << 8 | (uint32_t)out_dtype,
+                            [&] { return std::string(out_dtype == APK_F32 ? "apk_embed_q4k_f32" : "apk_embed_q4k_f16"); }, (unsigned)t,
+                            (unsigned)threads, 0, args);
     }
     // every other format: one workgroup per row, the row staged in LDS
     static const char* const kFmtName[10] = {"q4k", "q5k", "q6k", "q8_0", "q2k", "q3k", "q5_0", "f16", "f32", "bf16"};
@@ -741,8 +774,9 @@ static int embed_common(apk_ctx* c, int fmt, const void* table, size_t vocab, si
     if (threads > max_threads) threads = max_threads;
     uint64_t table_bytes = (uint64_t)vocab * row_bytes;
     void* args[] = {&table, &table_bytes, &vocab32, &n_i, &ids_dev, &out, &c->fault_dev, &scale};
-    const std::string which = std::string("apk_embed_") + kFmtName[fmt] + (out_dtype == APK_F32 ? "_f32" : "_f16");
-    return launch(c, which, (unsigned)t, (unsigned)threads, (unsigned)shmem, args);
+    return launch_keyed(c, OP_EMBED, (uint32_t)fmt << 8 | (uint32_t)out_dtype,
+                        [&] { return std::string("apk_embed_") + kFmtName[fmt] + (out_dtype == APK_F32 ? "_f32" : "_f16"); }, (unsigned)t,
+                        (unsigned)threads, (unsigned)shmem, args);
 }
 
 int apk_embed_rows(apk_ctx* c, int fmt, const void* table, size_t vocab, size_t n_in, const uint32_t* ids, size_t t,
@@ -927,7 +961,7 @@ int apk_argmax_rows(apk_ctx* c, const float* logits, size_t rows, size_t n, uint
     int parts_i = (int)parts;
     void* args[] = {&logits, &n64, &parts_i, &c->argmax_scratch, &out};
     if (c->capturing) c->capture_argmax = true;
-    return launch(c, "apk_argmax_rows", (unsigned)(rows * parts), 256, 0, args);
+    return launch_keyed(c, OP_ARGMAX, 0, [] { return std::string("apk_argmax_rows"); }, (unsigned)(rows * parts), 256, 0, args);
 }
 
 int apk_copy(apk_ctx* c, const void* src, void* dst, size_t bytes) {
