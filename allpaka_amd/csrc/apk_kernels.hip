@@ -115,14 +115,36 @@ DEV float dpp_step(float v, int s) {
 DEV double dpp_step(double v, int s) {
     return s == 0 ? dpp_f64<DPP_XOR1>(v) : s == 1 ? dpp_f64<DPP_XOR2>(v) : s == 2 ? dpp_f64<DPP_HALF_MIRROR>(v) : dpp_f64<DPP_MIRROR>(v);
 }
+// The value of lane `lane` (a constant) as a wave-uniform scalar: v_readlane, no LDS round trip.
+template <int LANE> DEV float lane_value(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), LANE));
+}
+template <int LANE> DEV double lane_value(double v) {
+    const uint64_t b = __builtin_bit_cast(uint64_t, v);
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)b, LANE);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(b >> 32), LANE);
+    return __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);
+}
 // Sum over aligned groups of WIDTH lanes (4, 8, 16, 32 or 64); every lane gets the sum.
+// Inside a 16-lane row: DPP butterflies.  Across the four rows: each row's sum read as a scalar
+// and added as (row0 + row1) + (row2 + row3), the value the xor-16 / xor-32 butterfly gives
+// every lane, without its two LDS-crossbar round trips.
 template <int WIDTH, typename A> DEV A group_sum(A v) {
 #pragma unroll
     for (int s = 0; s < 4; s++)
         if ((1 << (s + 1)) <= WIDTH) v += dpp_step(v, s);
-    if (WIDTH >= 32) v += __shfl_xor(v, 16, 64);
-    if (WIDTH >= 64) v += __shfl_xor(v, 32, 64);
+    if constexpr (WIDTH >= 32) {
+        const A lo = lane_value<0>(v) + lane_value<16>(v), hi = lane_value<32>(v) + lane_value<48>(v);
+        if constexpr (WIDTH >= 64) v = lo + hi;
+        else v = (threadIdx.x & 32) ? hi : lo;
+    }
     return v;
+}
+
+DEV float wave_max_f32(float v) {
+#pragma unroll
+    for (int s = 0; s < 4; s++) v = fmaxf(v, dpp_step(v, s));
+    return fmaxf(fmaxf(lane_value<0>(v), lane_value<16>(v)), fmaxf(lane_value<32>(v), lane_value<48>(v)));
 }
 
 // One tile of activations narrowed to fp16 (RNE) for the KV cache: 16 bytes from an
@@ -257,8 +279,7 @@ extern "C" __global__ __launch_bounds__(256) void apk_softmax_rows(float* x, int
     float* row = x + r * (uint64_t)n;
     float mx = -INFINITY;
     for (int i = lane; i < n; i += 64) mx = fmaxf(mx, row[i]);
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    mx = wave_max_f32(mx);
     float sum = 0.0f;
     for (int i = lane; i < n; i += 64) {
         const float e = expf(row[i] - mx);
@@ -312,7 +333,21 @@ DEV void add_rmsnorm_impl(T* x, const T* delta, T* h, const float* gamma, int n,
 
     // Every load of the lane is issued before the first use: no branch and no
     // conversion in this loop (a lane past the end of the row re-reads the last tile).
+    // With one or two tiles per lane (decode-sized batches: many waves per row, the kernel is a
+    // chain of latencies, not a stream) the norm weights are fetched here too, so that nothing is
+    // loaded after the cross-wave reduction; with more tiles they are read after it (they sit in
+    // L2, the other resident waves cover the latency, and the registers go to the row instead).
+    constexpr bool PRE_GAMMA = NCH <= 2;
     typename io<T>::raw_t xraw[NCH], draw[NCH];
+    float gpre[PRE_GAMMA ? NCH : 1][VEC];
+    if constexpr (PRE_GAMMA) {
+#pragma unroll
+        for (int j = 0; j < NCH; j++) {
+            const int c = min((int)(threadIdx.x + j * blockDim.x), nchunks - 1);
+#pragma unroll
+            for (int q = 0; q < VEC; q += 4) io<float>::load(gamma + c * VEC + q, gpre[j] + q);
+        }
+    }
 #pragma unroll
     for (int j = 0; j < NCH; j++) {
         const int c = min((int)(threadIdx.x + j * blockDim.x), nchunks - 1);
@@ -352,8 +387,13 @@ DEV void add_rmsnorm_impl(T* x, const T* delta, T* h, const float* gamma, int n,
         const int c = threadIdx.x + j * blockDim.x;
         if (c < nchunks) {
             float g[VEC], o[VEC];
+            if constexpr (PRE_GAMMA) {
 #pragma unroll
-            for (int q = 0; q < VEC; q += 4) io<float>::load(gamma + c * VEC + q, g + q);
+                for (int i = 0; i < VEC; i++) g[i] = gpre[j][i];
+            } else {
+#pragma unroll
+                for (int q = 0; q < VEC; q += 4) io<float>::load(gamma + c * VEC + q, g + q);
+            }
 #pragma unroll
             for (int i = 0; i < VEC; i++) o[i] = stat<T>::apply(v[j][i], scale, g[i]);
             io<T>::store_nt(hr + c * VEC, o);
@@ -1201,12 +1241,6 @@ APK_EMBED_GEN(f16, 7) APK_EMBED_GEN(f32, 8) APK_EMBED_GEN(bf16, 9)
 // l, l+64, l+128, ... (EPL of them).  For softmax without bias the selection runs on the
 // raw logits (same order as the probabilities, no dependence on exp rounding).
 // =========================================================================
-DEV float wave_max_f32(float v) {
-#pragma unroll
-    for (int s = 0; s < 4; s++) v = fmaxf(v, dpp_step(v, s));
-    v = fmaxf(v, __shfl_xor(v, 16, 64));
-    return fmaxf(v, __shfl_xor(v, 32, 64));
-}
 DEV float wave_sum_f32(float v) { return group_sum<64>(v); }
 template <int EPL>  // experts per lane: the wave covers 64*EPL experts
 DEV void route_topk_body(const float* logits, const float* bias, int rows, int n_expert, int k, int norm, float scale,
@@ -1275,7 +1309,8 @@ DEV void route_topk_body(const float* logits, const float* bias, int rows, int n
 #pragma unroll
             for (int j = 0; j < EPL; j++) s = slot == j ? score[j] : s;  // selects, not an indexed (scratch) read
         }
-        s = __shfl(s, owner, 64);
+        // owner is the same in every lane (it comes out of the wave maximum): a scalar lane select
+        s = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, s), __builtin_amdgcn_readfirstlane(owner)));
         total += s;  // best-first sequential f32 sum, as the reference's iterator sum
         if (lane == r) {
             my_id = e;
