@@ -2,13 +2,13 @@
 """Benchmark of the fused per-layer ops on ONE MI355X.
 
 A "step" is one decoder layer's worth of the hot path at Qwen3-32B shapes,
-T=2048 prefill rows, fp16 activations (BASELINE configs[2]):
+T=2048 prefill rows, fp16 activations (the headline configuration):
     add+RMSNorm (attention norm) -> per-head QK-norm + NeoX RoPE ->
     add+RMSNorm (FFN norm) -> SwiGLU
 i.e. 4 launches per layer, inputs resident in HBM.  Every op cycles through its
 own pool of distinct buffer sets of more than 640 MB, so no launch is served
 from the 256 MB last-level cache ("cold" = HBM numbers).  Every op is also
-timed on its own, at every BASELINE shape, with HIP events on the library's
+timed on its own, at every shape of the five benchmark configurations, with HIP events on the library's
 stream (3 untimed launches first).  The JSON line carries
     value     = microseconds per layer (lower is better),
     roofline  = the dominant kernel (SwiGLU, 300 MiB per launch) against 8 TB/s,
@@ -263,7 +263,7 @@ def main():
         "vs_baseline": None,
         "dtype": "f16",
         "data": "synthetic",
-        "config": {"workload": f"BASELINE configs[2]: Qwen3-32B fused layer ops, T={T} prefill rows, fp16 activations, "
+        "config": {"workload": f"configs[2]: Qwen3-32B fused layer ops, T={T} prefill rows, fp16 activations, "
                                f"hidden {H}, {NQ}q/{NKV}kv heads x {HD}, ffn {FF}; every op rotates through >= 640 MB of "
                                "distinct buffers so every launch streams from HBM",
                    "launches_per_layer": 4, "rows": T},

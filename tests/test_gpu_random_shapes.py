@@ -1,6 +1,6 @@
 """Seeded random shapes for every op through the C ABI against the CPU oracle.
 
-The parametrised parity tests pin the BASELINE shapes and hand-picked edges; this
+The parametrised parity tests pin the benchmark shapes and hand-picked edges; this
 file draws the shapes (row counts, row lengths, head geometry, expert counts, top-k,
 formats) from a fixed-seed generator so that indexing that only breaks off the
 beaten path (a last partial tile, a workgroup tail, a wave that owns no head) is met
