@@ -195,6 +195,16 @@ class Backend:
         self._leave()
         return table
 
+    def rope_table_into(self, positions, inv_freq, table):
+        """rope_table into a caller's [rows, half, 2] tensor: the form a recorded decode step uses
+        (the positions live in a device buffer the caller rewrites between replays)."""
+        rows, half = positions.numel(), inv_freq.numel()
+        assert positions.dtype in (torch.int32, torch.uint32) and inv_freq.dtype == torch.float32
+        assert table.dtype == torch.float32 and table.numel() == rows * half * 2
+        self._enter()
+        check(self.L.apk_rope_table(self.h, _ptr(positions), _ptr(inv_freq), rows, half, _ptr(table)))
+        self._leave()
+
     def qknorm_rope_norm(self, q, k, q_norm, k_norm, rope_flat, n_q, n_kv, head_dim, eps, rot_dim=None):
         """The same loop for RopeStyle::Norm models: adjacent pairs (2i, 2i+1) rotate
         (rope_norm_cached_from_array, rope.rs:52-64; attention.rs:62-67)."""
@@ -235,7 +245,8 @@ class Backend:
                                               _ptr(cache_pos), _ptr(k_cache), _ptr(v_cache), k_cache.shape[0], rows, n_q, n_kv,
                                               head_dim, head_dim, eps, _dt(q)))
         self._leave()
-        if self.take_faults() & _l.FAULT_CACHE_RANGE:
+        # (inside a recording nothing has run yet: the caller reads take_faults() after a replay)
+        if not self._recording and self.take_faults() & _l.FAULT_CACHE_RANGE:
             raise AssertionError("position past capacity")
 
     def layer_prologue(self, x, delta, h, gamma, q, k, q_norm, k_norm, rope_flat, n_q, n_kv, head_dim, eps):

@@ -891,16 +891,20 @@ APK_PROLOGUE(f16_t, f16, 64) APK_PROLOGUE(f16_t, f16, 128) APK_PROLOGUE(f16_t, f
 
 // RoPE table rows from per-row positions (rope.rs:18-22, session.rs:34-50):
 // table[r][i] = [sin, cos]((pos[r] as f32) * inv_freq[i]).  One f32 rounding of
-// the angle, then fully range-reduced sincosf (positions reach 32767 rad).
+// the angle, as the reference; then sine and cosine of that f32 angle in double
+// precision, rounded once to f32: the correctly rounded values, which is what the
+// reference's libm returns in all but rare cases -- a 2-ulp sincosf here would
+// show as 1e-5 in rotated outputs that nearly cancel.  (The table is rows*half
+// values: the cost of the double evaluation does not register.)
 extern "C" __global__ __launch_bounds__(256) void apk_rope_table(const uint32_t* pos, const float* inv_freq, int rows,
                                                                 int half, float* table) {
     const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= (uint64_t)rows * half) return;
     const float ang = (float)pos[i / half] * inv_freq[i % half];
-    float s, c;
-    sincosf(ang, &s, &c);
-    table[2 * i] = s;
-    table[2 * i + 1] = c;
+    double s, c;
+    sincos((double)ang, &s, &c);
+    table[2 * i] = (float)s;
+    table[2 * i + 1] = (float)c;
 }
 
 // =========================================================================

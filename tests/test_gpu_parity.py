@@ -383,7 +383,10 @@ def test_rope_table_on_device(be, ora):
     positions = np.concatenate([np.arange(0, 512), g.integers(0, 32768, size=64)]).astype(np.uint32)
     want = ora.rope_table(positions, inv)
     got = host(be.rope_table(dev(positions), dev(inv)))
-    assert np.max(np.abs(got - want)) <= 2.5e-7  # sin/cos are in [-1,1]: 2 ulp at 1.0
+    # the device rounds the double-precision sine/cosine of the same f32 angle once: the correctly rounded
+    # value, which glibc returns in all but rare cases -- bit-equal almost everywhere, 1 ulp at worst
+    assert np.max(np.abs(got - want)) <= 6e-8
+    assert np.mean(got.view(np.uint32) == want.view(np.uint32)) > 0.98  # glibc sinf/cosf: 0.56 ulp, ~1 % off by one
     # and used end to end on the 64 long-context rows (fp16 config)
     rows, n_q, n_kv, hd = 64, 64, 8, 128
     q, k, qw, kw, _, ropes = _qk_case(ora, 3, rows, n_q, n_kv, hd, True, positions[512:])

@@ -265,3 +265,60 @@ def test_argmax_scratch_cannot_move_under_a_graph(be):
         assert b2.argmax_rows(big).shape[0] == 1000  # free to grow again
     finally:
         b2.close()
+
+
+@pytest.mark.parametrize("f16", [False, True])
+def test_one_recording_serves_every_token_of_a_decode(be, ora, f16):
+    """The reference's graph-replayable decode keeps the token position in device memory
+    (d_pos, gpu/cuda/runtime/device.rs:154; build_rope_freq_dpos + rmsnorm_rope_qk_store_table_dpos,
+    gpu/cuda/kernels.rs:680-765).  Same here: the recorded step builds the rotary row from a position
+    buffer and stores K/V at that position; between replays only the contents of buffers change."""
+    from allpaka_amd import synth as s
+
+    n_q, n_kv, hd, cap = 16, 8, 128, 64
+    g = s.rng(3, 4242)
+    inv = ora.rope_inv_freq(hd, 1e6)
+    qw = (0.88 + 0.001 * np.arange(hd)).astype(np.float32)
+    kw = (0.92 + 0.001 * np.arange(hd)).astype(np.float32)
+    dt = torch.float16 if f16 else torch.float32
+    tq = torch.empty((1, n_q * hd), dtype=dt, device="cuda")
+    tk = torch.empty((1, n_kv * hd), dtype=dt, device="cuda")
+    tv = torch.empty((1, n_kv * hd), dtype=dt, device="cuda")
+    pos = torch.zeros(1, dtype=torch.int32, device="cuda")
+    table = torch.zeros((1, hd // 2, 2), dtype=torch.float32, device="cuda")
+    kc = torch.zeros((cap, n_kv * hd), dtype=torch.float16, device="cuda")
+    vc = torch.zeros((cap, n_kv * hd), dtype=torch.float16, device="cuda")
+    dinv, dqw, dkw = dev(inv), dev(qw), dev(kw)
+    with be.record() as rec:
+        be.rope_table_into(pos, dinv, table)
+        be.qknorm_rope_kv_store(tq, tk, tv, dqw, dkw, table, pos, kc, vc, n_q, n_kv, hd, 1e-6)
+    assert rec.graph.nodes == 2
+    want_kc, want_vc = np.zeros((cap, n_kv * hd), np.uint16), np.zeros((cap, n_kv * hd), np.uint16)
+    for p in (0, 1, 17, 63, 5, 17):  # 17 twice: a position may be rewritten
+        def act(n):
+            a = s.normal_f32(g, (1, n))
+            return s.to_f16_bits(a) if f16 else a
+        q, k, v = act(n_q * hd), act(n_kv * hd), act(n_kv * hd)
+        tq.copy_(dev(q)), tk.copy_(dev(k)), tv.copy_(dev(v))
+        pos.fill_(p)
+        torch.cuda.synchronize()
+        rec.graph.launch()
+        be.sync()
+        assert be.take_faults() == 0
+        wq, wk = q.copy(), k.copy()
+        ora.qknorm_rope_rows(wq, wk, n_q, n_kv, hd, qw, kw, ora.rope_table([p], inv), 1e-6)
+        if f16:
+            assert f16_ulp_diff(host(tq), wq) <= 2 and f16_ulp_diff(host(tk), wk) <= 2
+        else:
+            assert rel_err_f32(host(tq), wq) <= 1e-5 and rel_err_f32(host(tk), wk) <= 1e-5
+        # the cache holds the exact narrowing of the k this launch produced, and of v
+        ora.kv_store_rows(host(tk), v, [p], want_kc, want_vc)
+        assert np.array_equal(host(kc), want_kc) and np.array_equal(host(vc), want_vc)
+    # a position past the capacity: the row's store is skipped and the status word says so
+    pos.fill_(cap)
+    torch.cuda.synchronize()
+    rec.graph.launch()
+    be.sync()
+    assert be.take_faults() == 8  # APK_FAULT_CACHE_RANGE
+    assert np.array_equal(host(kc), want_kc)
+    rec.graph.destroy()
