@@ -236,6 +236,26 @@ def main():
             p(kvp[i % len(qk)]["kc"]), p(kvp[i % len(qk)]["vc"]), T, T, NQ, NKV, HD, HD, EPS, F16)), reps)
         record("qknorm_rope_neox + K/V cache store (one launch)", tag, us, bytes_qkrope + T * NKV * HD * b + 2 * T * NKV * HD * 2 + T * 4)
         del an, qk, sw, kvp
+        # the same headline shape with f32 activations, the reference's own activation type (f64 statistics,
+        # the reference's operation order): twice the bytes per launch
+        f32 = torch.float32
+        an32 = pool(3 * T * H * 4, lambda: dict(x=randn((T, H), f32), d=randn((T, H), f32), h=torch.empty((T, H), dtype=f32, device=dev)))
+        torch.cuda.synchronize()
+        us = timed(lambda i: apklib.check(L.apk_add_rmsnorm_rows(h, p(an32[i % len(an32)]["x"]), p(an32[i % len(an32)]["d"]),
+                                                                 p(an32[i % len(an32)]["h"]), p(gamma1), H, T, EPS, F32)), reps)
+        record("add_rmsnorm", f"qwen3-32b T={T} f32", us, 4 * T * H * 4 + 4 * H)
+        del an32
+        qk32 = pool(T * (NQ + NKV) * HD * 4, lambda: dict(q=randn((T, NQ * HD), f32), k=randn((T, NKV * HD), f32)))
+        torch.cuda.synchronize()
+        us = timed(lambda i: apklib.check(L.apk_qknorm_rope_neox(h, p(qk32[i % len(qk32)]["q"]), p(qk32[i % len(qk32)]["k"]), p(qw), p(kw),
+                                                                 p(rope), T, NQ, NKV, HD, HD, EPS, F32)), reps)
+        record("qknorm_rope_neox", f"qwen3-32b T={T} f32", us, 2 * T * (NQ + NKV) * HD * 4 + T * (HD // 2) * 8 + 2 * HD * 4)
+        del qk32
+        sw32 = pool(2 * T * FF * 4, lambda: dict(gate=randn((T, FF), f32), up=randn((T, FF), f32)))
+        torch.cuda.synchronize()
+        us = timed(lambda i: apklib.check(L.apk_swiglu(h, p(sw32[i % len(sw32)]["gate"]), p(sw32[i % len(sw32)]["up"]), T * FF, F32)), reps)
+        record("swiglu", f"qwen3-32b T={T} f32", us, 3 * T * FF * 4)
+        del sw32
         other_shapes(args, L, h, apklib, synth, torch, gen, dev, randn, pool, p, timed, record, reps, m, qw, kw, rope)
     sync()
 
