@@ -538,6 +538,51 @@ def test_swiglu_reference_sweep_and_assert(be, ora):
         be.swiglu(torch.zeros(4, device="cuda"), torch.zeros(3, device="cuda"))
 
 
+def test_fp16_special_values_follow_the_oracle(be, ora):
+    """fp16 edges: sums that overflow to infinity, subnormal inputs and outputs, all-zero rows, signed zeros."""
+    n = 1024
+    f = lambda a: np.asarray(a, np.float32).astype(np.float16).view(np.uint16)
+    x = np.zeros((6, n), np.float32)
+    d = np.zeros((6, n), np.float32)
+    x[0, :], d[0, :] = 60000.0, 60000.0                    # x + delta = inf in fp16
+    x[1, :] = 6e-8 * (1 + np.arange(n) % 7)                # subnormal inputs (fp16 min subnormal 5.96e-8)
+    d[1, :] = 6e-8
+    x[2, :] = 0.0                                          # zeros + eps: finite, exactly zero
+    x[3, ::2], x[3, 1::2] = -0.0, 0.0
+    d[3, :] = -0.0
+    x[4, :] = np.linspace(-6e-5, 6e-5, n)                  # around the normal/subnormal boundary (6.1e-5)
+    x[5, :] = np.linspace(-65504, 65504, n)
+    d[5, :] = 0.0
+    xb, db = f(x), f(d)
+    gamma = np.ones(n, np.float32)
+    wx, wh = xb.copy(), np.zeros_like(xb)
+    with np.errstate(all="ignore"):
+        ora.add_rmsnorm_rows(wx, db, wh, gamma, 1e-6)
+    tx, th = dev(xb), torch.zeros_like(dev(xb))
+    be.add_rmsnorm_rows(tx, dev(db), th, dev(gamma), 1e-6)
+    assert np.array_equal(host(tx), wx)                    # residual sum incl. inf, subnormals and signed zeros
+    assert np.all(wx[0] == 0x7C00)
+    got = host(th)
+    fin = np.isfinite(wh.view(np.float16)) & np.isfinite(got.view(np.float16))
+    assert np.array_equal(np.isfinite(wh.view(np.float16)), np.isfinite(got.view(np.float16)))
+    assert f16_ulp_diff(got[fin], wh[fin]) <= TOL_F16_ULP
+    assert np.all(got[2] == 0)
+    # SwiGLU over every finite fp16 gate value, up = 1 and up = -2.5
+    gate = np.arange(0x10000, dtype=np.uint32).astype(np.uint16)
+    gate = gate[np.isfinite(gate.view(np.float16))]
+    for upv in (1.0, -2.5):
+        up = f(np.full(gate.size, upv))
+        want = gate.copy()
+        with np.errstate(all="ignore"):
+            ora.swiglu(want, up)
+        tg = dev(gate)
+        be.swiglu(tg, dev(up))
+        g_ = host(tg)
+        assert np.array_equal(np.isfinite(g_.view(np.float16)), np.isfinite(want.view(np.float16)))
+        ok = np.isfinite(want.view(np.float16))
+        assert f16_ulp_diff(g_[ok], want[ok]) <= TOL_F16_ULP, upv
+
+
 # ------------------------------------------------- residual add, softmax alone
 @pytest.mark.parametrize("n", [1, 3, 8, 1024, 5120 * 6 + 5, 65536 * 3 + 1])
 @pytest.mark.parametrize("f16", [False, True])
