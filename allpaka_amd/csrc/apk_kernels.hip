@@ -300,13 +300,16 @@ extern "C" __global__ __launch_bounds__(256) void apk_softmax_rows(float* x, int
 // row is read from HBM once.  The host picks W so that every row of a large
 // batch is resident at once (W = 1: a wave per row, no LDS, no barrier).
 // f32 activations: statistics and scaling in f64, exactly the reference's
-// operations.  fp16 activations: the output keeps 11 bits, so the statistics
-// are f32 (8-element partial sums, then a tree) and the scaling is two f32
-// multiplies; the result stays within 1 ulp of fp16 of the f64 form.
+// operations.  fp16 activations: the output keeps 11 bits and nothing here cancels
+// (h = x * scale * gamma), so f32 statistics (8-element partial sums, then a tree),
+// the hardware rsq and two f32 multiplies differ from the reference's f32 result by
+// parts in 1e7: after the one rounding to fp16 the result is the reference's in all but
+// about 4 in 100 000 elements, and 1 ulp of fp16 away in those.
 // =========================================================================
 template <typename T> struct stat;
 template <> struct stat<float> {
     typedef double acc_t;
+    typedef double scale_t;
     DEV double sq(double a, float v) { return __builtin_fma((double)v, (double)v, a); }
     DEV double wave_sum(double v) { return group_sum<64>(v); }
     DEV double rscale(double ss, int n, float eps) { return 1.0 / sqrt(ss / (double)n + (double)eps); }
@@ -314,10 +317,39 @@ template <> struct stat<float> {
 };
 template <> struct stat<f16_t> {
     typedef float acc_t;
+    typedef float scale_t;
     DEV float sq(float a, float v) { return __builtin_fmaf(v, v, a); }
     DEV float wave_sum(float v) { return group_sum<64>(v); }
     DEV float rscale(float ss, int n, float eps) { return __builtin_amdgcn_rsqf(ss * (1.0f / (float)n) + eps); }
     DEV float apply(float v, float scale, float g) { return v * scale * g; }
+};
+// The per-head norm in front of a rotation is another matter: a rotated output a*cos - b*sin can
+// nearly cancel, and an f32-level difference in the normalised inputs is then many ulps of the
+// fp16 result.  There fp16 activations get the reference's values themselves, at a third of the
+// double-precision work, so that the result is the reference's f32 result rounded once to fp16:
+//   * the sum of squares in f64, as the reference;
+//   * 1/sqrt(mean + eps) by two Newton steps in f64 from the f32 hardware rsq (agrees with the
+//     reference's sqrt-then-divide to about 1e-16);
+//   * (x as f64 * scale) as f32 as an error-free f32 product with scale = hi + lo:
+//     p = fl(x*hi), e = x*hi - p (exact, one fma), result = fl(p + fl(e + x*lo)): the
+//     correctly rounded product unless it lies within 2^-48 of a rounding boundary.
+template <typename T> struct headstat : stat<T> {};
+template <> struct headstat<f16_t> {
+    typedef double acc_t;
+    struct scale_t { float hi, lo; };
+    DEV double sq(double a, float v) { return __builtin_fma((double)v, (double)v, a); }
+    DEV scale_t rscale(double ss, int n, float eps) {
+        const double v = ss / (double)n + (double)eps;  // n a power of two known at compile time: a multiplication
+        double y = (double)__builtin_amdgcn_rsqf((float)v);
+        y = y * __builtin_fma(-0.5 * v, y * y, 1.5);
+        y = y * __builtin_fma(-0.5 * v, y * y, 1.5);
+        const float hi = (float)y;
+        return scale_t{hi, (float)(y - (double)hi)};
+    }
+    DEV float apply(float v, scale_t s, float g) {
+        const float p = v * s.hi;
+        return (p + __builtin_fmaf(v, s.lo, __builtin_fmaf(v, s.hi, -p))) * g;
+    }
 };
 
 template <typename T, int NCH, bool HAS_DELTA>
@@ -381,7 +413,7 @@ DEV void add_rmsnorm_impl(T* x, const T* delta, T* h, const float* gamma, int n,
         ss = 0;
         for (int w = 0; w < nwaves; w++) ss += part[w];
     }
-    const acc_t scale = stat<T>::rscale(ss, n, eps);
+    const typename stat<T>::scale_t scale = stat<T>::rscale(ss, n, eps);
 #pragma unroll
     for (int j = 0; j < NCH; j++) {
         const int c = threadIdx.x + j * blockDim.x;
@@ -541,7 +573,7 @@ DEV void combine_add_rmsnorm_body(T* x, const T* flat, const uint32_t* tok_off, 
         ss = 0;
         for (int w = 0; w < nwaves; w++) ss += part[w];
     }
-    const acc_t scale = stat<T>::rscale(ss, n, eps);
+    const typename stat<T>::scale_t scale = stat<T>::rscale(ss, n, eps);
     T* hr = h + row * (uint64_t)n;
 #pragma unroll
     for (int j = 0; j < NCH; j++) {
@@ -649,10 +681,9 @@ extern "C" __global__ __launch_bounds__(256) void apk_argmax_rows(const float* l
 // the weight are loaded once and reused over ITER passes (q: ITERQ passes,
 // k: 1 pass -- under GQA k has few heads).  The host picks ITERQ so that a
 // large batch is about one resident round of waves.
-// f32 activations: f64 statistics and scaling, no contraction, the reference's
-// operation order.  fp16 activations (output keeps 11 bits): f32 statistics,
-// hardware rsq, and the norm weight folded into the rotation coefficients
-// (out_a = scale*(a*(wa*cos) - b*(wb*sin))): 3 instead of 5 multiplies/element.
+// Arithmetic: the reference's, for both activation types (see `headstat`): f64 statistics,
+// (x as f64 * scale) as f32 * w, then the four products and two sums of the rotation,
+// not contracted.  fp16 results are that f32 result rounded once.
 // =========================================================================
 // KV = true (k items only): the rotated k tiles are also narrowed to fp16 into the cache row
 // kc, and the same tiles of the row's v are narrowed into vc (KvCache::store_at,
@@ -664,7 +695,7 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
     constexpr int HALF = HD / 2;
     constexpr int LPH = HALF / EPL;   // lanes per head
     constexpr int HPW = 64 / LPH;     // heads per wave pass
-    typedef typename stat<T>::acc_t acc_t;
+    typedef typename headstat<T>::acc_t acc_t;
     // Loads return in issue order, so the small cached ones go first and the first pass
     // can start as soon as its own two tiles arrive.  No branch, no conversion here: a
     // lane of a pass beyond the last head re-reads the last head and stores nothing; a
@@ -696,15 +727,6 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
     }
     __builtin_amdgcn_sched_barrier(0);  // every load above; all uses below
     const bool normed = w != nullptr;  // uniform for the wave
-    float P[EPL], Q[EPL], R[EPL], S[EPL];  // fp16 path: rotation coefficients with the weight folded in
-    if constexpr (sizeof(T) == 2) {
-#pragma unroll
-        for (int i = 0; i < EPL; i++) {
-            const float s = sc[2 * i], c = sc[2 * i + 1];
-            const float ga = normed ? wa[i] : 1.0f, gb = normed ? wb[i] : 1.0f;
-            P[i] = ga * c; Q[i] = gb * s; R[i] = ga * s; S[i] = gb * c;
-        }
-    }
 #pragma unroll
     for (int it = 0; it < ITER; it++) {
         float a[EPL], b[EPL], oa[EPL], ob[EPL];
@@ -713,30 +735,21 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
         acc_t ss = 0;
 #pragma unroll
         for (int i = 0; i < EPL; i++) {
-            ss = stat<T>::sq(ss, a[i]);
-            ss = stat<T>::sq(ss, b[i]);
+            ss = headstat<T>::sq(ss, a[i]);
+            ss = headstat<T>::sq(ss, b[i]);
         }
         ss = group_sum<LPH>(ss);
-        const acc_t scale = stat<T>::rscale(ss, HD, eps);
-        if constexpr (sizeof(T) == 2) {
-            const float sf = normed ? (float)scale : 1.0f;
+        const typename headstat<T>::scale_t scale = headstat<T>::rscale(ss, HD, eps);
 #pragma unroll
-            for (int i = 0; i < EPL; i++) {
-                oa[i] = __builtin_fmaf(-b[i], Q[i], a[i] * P[i]) * sf;
-                ob[i] = __builtin_fmaf(b[i], S[i], a[i] * R[i]) * sf;
+        for (int i = 0; i < EPL; i++) {
+            float x = a[i], y = b[i];
+            if (normed) {
+                x = headstat<T>::apply(x, scale, wa[i]);
+                y = headstat<T>::apply(y, scale, wb[i]);
             }
-        } else {
-#pragma unroll
-            for (int i = 0; i < EPL; i++) {
-                float x = a[i], y = b[i];
-                if (normed) {
-                    x = stat<T>::apply(x, scale, wa[i]);
-                    y = stat<T>::apply(y, scale, wb[i]);
-                }
-                const float s = sc[2 * i], c = sc[2 * i + 1];
-                oa[i] = x * c - y * s;
-                ob[i] = x * s + y * c;
-            }
+            const float s = sc[2 * i], c = sc[2 * i + 1];
+            oa[i] = x * c - y * s;  // not contracted: the reference's four products and two sums
+            ob[i] = x * s + y * c;
         }
         const bool live = hh_first + it * HPW < nheads;
         const int off = head_off(it);
@@ -830,7 +843,7 @@ APK_QKROPE_KV_ALL(f16_t, f16)
 template <typename T>
 DEV void qknorm_rope_generic_body(T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q,
                                   int n_kv, int hd, int rot_half, int norm_style, float eps) {
-    typedef typename stat<T>::acc_t acc_t;
+    typedef typename headstat<T>::acc_t acc_t;
     const int lane = threadIdx.x & 63;
     const uint64_t wid = ((uint64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
     const uint64_t heads = (uint64_t)n_q + n_kv;
@@ -841,26 +854,26 @@ DEV void qknorm_rope_generic_body(T* q, T* k, const float* qw, const float* kw, 
     T* x = isq ? q + (row * n_q + hh) * (uint64_t)hd : k + (row * n_kv + (hh - n_q)) * (uint64_t)hd;
     const float* w = isq ? qw : kw;
     const float* t = rope + row * (uint64_t)rot_half * 2;
-    acc_t scale = 1;
+    typename headstat<T>::scale_t scale{};
     if (w) {
         acc_t ss = 0;
-        for (int i = lane; i < hd; i += 64) ss = stat<T>::sq(ss, (float)x[i]);
+        for (int i = lane; i < hd; i += 64) ss = headstat<T>::sq(ss, (float)x[i]);
         ss = group_sum<64>(ss);  // every lane's loads are consumed here, before any store below
-        scale = stat<T>::rscale(ss, hd, eps);
+        scale = headstat<T>::rscale(ss, hd, eps);
     }
     for (int i = lane; i < rot_half; i += 64) {
         const int ia = norm_style ? 2 * i : i, ib = norm_style ? 2 * i + 1 : i + rot_half;
         float a = (float)x[ia], b = (float)x[ib];
         if (w) {
-            a = stat<T>::apply(a, scale, w[ia]);
-            b = stat<T>::apply(b, scale, w[ib]);
+            a = headstat<T>::apply(a, scale, w[ia]);
+            b = headstat<T>::apply(b, scale, w[ib]);
         }
         const float sn = t[2 * i], cs = t[2 * i + 1];
         x[ia] = (T)(a * cs - b * sn);
         x[ib] = (T)(a * sn + b * cs);
     }
     if (w)
-        for (int i = 2 * rot_half + lane; i < hd; i += 64) x[i] = (T)stat<T>::apply((float)x[i], scale, w[i]);
+        for (int i = 2 * rot_half + lane; i < hd; i += 64) x[i] = (T)headstat<T>::apply((float)x[i], scale, w[i]);
 }
 extern "C" __global__ __launch_bounds__(256) void apk_qknorm_rope_generic_f32(
     float* q, float* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv, int hd,

@@ -294,6 +294,26 @@ def test_qknorm_rope(be, ora, rows, n_q, n_kv, hd, pos_kind, f16):
             assert rel_err_f32(got, want) <= TOL_F32 and close_idiom(got, want)
 
 
+@pytest.mark.parametrize("scale", [1.0, 100.0, 1e-3])
+def test_qknorm_rope_fp16_is_the_reference_result_rounded_once(be, ora, scale):
+    """A rotated output a*cos - b*sin can nearly cancel, and an f32-level difference is then many fp16 ulps: the
+    per-head norm in front of the rotation therefore reproduces the reference's f32 values (f64 statistics, the
+    f64 product rounded to f32, uncontracted rotation), and the fp16 result is that value rounded once --
+    bit for bit on these 900 000 elements, many of them in the cancellation zone."""
+    s = synth()
+    g = s.rng(3, int(scale * 1000) + 77)
+    rows, n_q, n_kv, hd = 96, 64, 8, 128
+    q = s.to_f16_bits(s.normal_f32(g, (rows, n_q * hd)) * np.float32(scale))
+    k = s.to_f16_bits(s.normal_f32(g, (rows, n_kv * hd)) * np.float32(scale))
+    qw, kw = s.normal_f32(g, hd, 1.0, 0.05), s.normal_f32(g, hd, 1.0, 0.05)
+    ropes = ora.rope_table([int(v) for v in g.integers(0, 32768, size=rows)], ora.rope_inv_freq(hd, 1e6))
+    wq, wk = q.copy(), k.copy()
+    ora.qknorm_rope_rows(wq, wk, n_q, n_kv, hd, qw, kw, ropes, 1e-6)
+    tq, tk = dev(q), dev(k)
+    be.qknorm_rope_neox(tq, tk, dev(qw), dev(kw), dev(ropes), n_q, n_kv, hd, 1e-6)
+    assert np.array_equal(host(tq), wq) and np.array_equal(host(tk), wk)
+
+
 def test_rope_only_and_reference_vectors(be, ora):
     # no norm weights: rotation only (attention.rs:140-146); bit-exact (same f32 ops, no contraction)
     rows, n_q, n_kv, hd = 9, 4, 2, 128
