@@ -872,8 +872,9 @@ int apk_gather_rows(apk_ctx* c, const void* src, const uint32_t* tok, size_t src
     if (int rc = set_device(c)) return rc;
     uint32_t src_rows32 = (uint32_t)src_rows;
     int row_vecs = (int)(cols * es / 16);
-    void* args[] = {&src, &tok, &src_rows32, &row_vecs, &dst, &c->fault_dev};
-    return launch(c, "apk_gather_rows", (unsigned)total_rows, 256, 0, args);
+    uint32_t total32 = (uint32_t)total_rows;
+    void* args[] = {&src, &tok, &src_rows32, &total32, &row_vecs, &dst, &c->fault_dev};
+    return launch(c, "apk_gather_rows", (unsigned)((total_rows + 3) / 4), 256, 0, args);  // 4 rows per workgroup
 }
 
 int apk_scatter_rows(apk_ctx* c, const void* src, const uint32_t* hit_row, size_t rows, size_t k, size_t total_rows,

@@ -1488,24 +1488,44 @@ extern "C" __global__ __launch_bounds__(APK_PERMUTE_THREADS) void apk_moe_permut
 }
 
 // Gathered activations in tok order (moe.rs:348-352): dst[r,:] = src[tok[r],:].
-// One workgroup per destination row, 16-byte tiles; row_vecs = row bytes / 16.
+// One workgroup per APK_GATHER_ROWS destination rows, 16-byte tiles; row_vecs = row bytes / 16.
+// The source row numbers of the group are read first (uniform for the workgroup), then the
+// tiles of all its rows are in flight together: one index latency per group, not per row.
+#define APK_GATHER_ROWS 4
 extern "C" __global__ __launch_bounds__(256) void apk_gather_rows(const u32x4* src, const uint32_t* tok,
-                                                                 uint32_t src_rows, int row_vecs, u32x4* dst,
-                                                                 uint32_t* fault) {
-    const uint64_t r = blockIdx.x;
-    const uint32_t s = tok[r];
-    if (s >= src_rows) {
-        if (threadIdx.x == 0) atomicOr(fault, APK_FAULT_ROW_RANGE);
-        return;
+                                                                 uint32_t src_rows, uint32_t total_rows, int row_vecs,
+                                                                 u32x4* dst, uint32_t* fault) {
+    const uint32_t r0 = blockIdx.x * APK_GATHER_ROWS;
+    uint32_t s[APK_GATHER_ROWS];
+    bool ok[APK_GATHER_ROWS];
+    bool bad = false;
+#pragma unroll
+    for (int j = 0; j < APK_GATHER_ROWS; j++) {
+        const bool in = r0 + j < total_rows;
+        s[j] = tok[min(r0 + (uint32_t)j, total_rows - 1u)];
+        ok[j] = in && s[j] < src_rows;
+        bad |= in && s[j] >= src_rows;
+        s[j] = s[j] < src_rows ? s[j] : 0u;
     }
-    const u32x4* sp = src + (uint64_t)s * row_vecs;
-    u32x4* dp = dst + r * row_vecs;
+    if (bad && threadIdx.x == 0) atomicOr(fault, APK_FAULT_ROW_RANGE);
     for (int c = threadIdx.x; c < row_vecs; c += 2 * blockDim.x) {
         const int c2 = c + blockDim.x;
-        u32x4 a = sp[c], b;
-        if (c2 < row_vecs) b = sp[c2];
-        __builtin_nontemporal_store(a, dp + c);
-        if (c2 < row_vecs) __builtin_nontemporal_store(b, dp + c2);
+        const bool two = c2 < row_vecs;
+        u32x4 a[APK_GATHER_ROWS], b[APK_GATHER_ROWS];
+#pragma unroll
+        for (int j = 0; j < APK_GATHER_ROWS; j++) {
+            const u32x4* sp = src + (uint64_t)s[j] * row_vecs;
+            a[j] = sp[c];
+            b[j] = sp[two ? c2 : c];
+        }
+#pragma unroll
+        for (int j = 0; j < APK_GATHER_ROWS; j++) {
+            if (ok[j]) {  // uniform
+                u32x4* dp = dst + (uint64_t)(r0 + j) * row_vecs;
+                __builtin_nontemporal_store(a[j], dp + c);
+                if (two) __builtin_nontemporal_store(b[j], dp + c2);
+            }
+        }
     }
 }
 
