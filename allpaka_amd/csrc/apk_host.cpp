@@ -193,11 +193,11 @@ size_t apk_row_bytes(int fmt, size_t n_in) {
 }
 
 int apk_can_embed(int fmt, size_t n_in) {
-    // every format of the unified codes; rows must be whole 16-byte output tiles and
-    // (all but Q4_K, which reads global memory directly) fit the 64 KiB LDS staging
+    // every format of the unified codes; rows must be whole 16-byte output tiles; F16 / BF16 rows
+    // (the two formats still staged through LDS) must fit the 64 KiB staging buffer
     const size_t rb = apk_row_bytes(fmt, n_in);
     if (rb == 0 || n_in == 0 || n_in % 8) return 0;
-    return fmt == APK_FMT_Q4K || rb + 32 <= 64 * 1024;
+    return (fmt == APK_FMT_F16 || fmt == APK_FMT_BF16) ? rb + 32 <= 64 * 1024 : 1;
 }
 
 int apk_init(int device, apk_ctx** out) {
@@ -765,13 +765,41 @@ static int embed_common(apk_ctx* c, int fmt, const void* table, size_t vocab, si
                             [&] { return std::string(out_dtype == APK_F32 ? "apk_embed_q4k_f32" : "apk_embed_q4k_f16"); }, (unsigned)t,
                             (unsigned)threads, 0, args);
     }
-    // every other format: one workgroup per row, the row staged in LDS
     static const char* const kFmtName[10] = {"q4k", "q5k", "q6k", "q8_0", "q2k", "q3k", "q5_0", "f16", "f32", "bf16"};
+    if (fmt == APK_FMT_Q6K || fmt == APK_FMT_Q5K || fmt == APK_FMT_Q2K || fmt == APK_FMT_Q3K) {
+        // decoded straight from global memory, 8 lanes per 256-element super-block (the Q4_K lane layout)
+        const size_t lanes = n_in / 256 * 8;
+        size_t threads = (lanes + 63) / 64 * 64;
+        if (threads > 256) threads = 256;
+        const size_t chunks = (lanes + threads - 1) / threads;
+        const uint64_t grid = (uint64_t)t * chunks;
+        if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_embed_rows: too large");
+        uint32_t chunks32 = (uint32_t)chunks;
+        void* args[] = {&table, &vocab32, &n_i, &ids_dev, &chunks32, &out, &c->fault_dev, &scale};
+        return launch_keyed(c, OP_EMBED, (uint32_t)fmt << 8 | (uint32_t)out_dtype,
+                            [&] { return std::string("apk_embed_") + kFmtName[fmt] + (out_dtype == APK_F32 ? "_f32" : "_f16"); },
+                            (unsigned)grid, (unsigned)threads, 0, args);
+    }
+    if (fmt == APK_FMT_Q8_0 || fmt == APK_FMT_Q5_0 || fmt == APK_FMT_F32) {
+        // decoded straight from global memory: a lane owns 4 of the row's 16-byte output tiles; a row takes
+        // one workgroup of up to 256 lanes, or several chunks of 1024 tiles
+        const size_t tiles_per_row = n_in / (16 / elem_size(out_dtype));
+        size_t threads = ((tiles_per_row + 3) / 4 + 63) / 64 * 64;
+        if (threads > 256) threads = 256;
+        const size_t chunks = (tiles_per_row + threads * 4 - 1) / (threads * 4);
+        const uint64_t grid = (uint64_t)t * chunks;
+        if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_embed_rows: too large");
+        uint32_t chunks32 = (uint32_t)chunks;
+        void* args[] = {&table, &vocab32, &n_i, &ids_dev, &chunks32, &out, &c->fault_dev, &scale};
+        return launch_keyed(c, OP_EMBED, (uint32_t)fmt << 8 | (uint32_t)out_dtype,
+                            [&] { return std::string("apk_embed_") + kFmtName[fmt] + (out_dtype == APK_F32 ? "_f32" : "_f16"); },
+                            (unsigned)grid, (unsigned)threads, 0, args);
+    }
+    // the remaining formats: one workgroup per row, the row staged in LDS
     const size_t row_bytes = apk_row_bytes(fmt, n_in);
     const size_t shmem = row_bytes + 32;
     size_t threads = (n_in / (16 / elem_size(out_dtype)) + 63) / 64 * 64;  // one output tile per lane
-    const size_t max_threads = fmt == APK_FMT_Q8_0 ? 1024 : 256;
-    if (threads > max_threads) threads = max_threads;
+    if (threads > 256) threads = 256;
     uint64_t table_bytes = (uint64_t)vocab * row_bytes;
     void* args[] = {&table, &table_bytes, &vocab32, &n_i, &ids_dev, &out, &c->fault_dev, &scale};
     return launch_keyed(c, OP_EMBED, (uint32_t)fmt << 8 | (uint32_t)out_dtype,

@@ -151,9 +151,9 @@ int apk_graph_destroy(apk_ctx* ctx, apk_graph* graph);
  * embed_row_f32_dtoken kernels (token id read on the device).
  * table: [vocab][apk_row_bytes(fmt,n_in)] bytes, 16-byte aligned; ids: u32[t];
  * out: [t][n_in] of out_dtype.  An id >= vocab leaves its row untouched and
- * raises APK_FAULT_TOKEN_RANGE.  All ten formats of apk_dq_fmt are taken (Q8_0 and Q4_K,
- * the formats of the benchmark configurations, by dedicated kernels); n_in must be a
- * multiple of 8 and a row must fit 64 KiB (apk_can_embed tells). */
+ * raises APK_FAULT_TOKEN_RANGE.  All ten formats of apk_dq_fmt are taken, decoded straight from
+ * global memory (F16 / BF16 staged through LDS); n_in must be a multiple of 8, and an F16 / BF16
+ * row must fit 64 KiB (apk_can_embed tells). */
 int apk_embed_rows(apk_ctx* ctx, int fmt, const void* table, size_t vocab, size_t n_in, const uint32_t* ids,
                    size_t t, void* out, int out_dtype);
 /* The same followed by `*v *= scale` in f32 when scale != 1 (before the narrowing of an
