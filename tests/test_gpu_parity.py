@@ -136,6 +136,35 @@ def test_embed_all_ten_formats_bit_exact(be, ora, fmt_name, out_f16):
     assert np.array_equal(got.view(np.uint16 if out_f16 else np.uint32), want_s.view(np.uint16 if out_f16 else np.uint32))
 
 
+@pytest.mark.parametrize("fmt_name,n_in", [("Q8_0", 20480), ("Q6K", 12288), ("Q5K", 16384), ("Q2K", 9216), ("Q3K", 8448),
+                                           ("Q5_0", 9984), ("F32", 4104), ("Q4K", 16384), ("BF16", 32752)])
+@pytest.mark.parametrize("out_f16", [False, True])
+def test_embed_long_rows_take_several_workgroups(be, ora, fmt_name, n_in, out_f16):
+    """Rows longer than one workgroup covers (chunks of a row), up to the staging limit of the LDS-staged formats."""
+    import allpaka_amd as apk
+
+    fmt, vocab = ora.FMT[fmt_name], 5
+    g = np.random.default_rng(n_in)
+    rb = ora.expected_bytes(fmt, n_in)
+    raw = g.integers(0, 256, size=vocab * rb, dtype=np.uint8)
+    if fmt_name in _SCALE_OFFS:
+        bb, offs = _SCALE_OFFS[fmt_name]
+        blocks = raw.reshape(-1, bb)
+        for o in offs:
+            blocks[:, o + 1] &= 0x3B  # finite, small f16 scale fields
+    elif fmt_name == "F32":
+        raw = synth().normal_f32(g, vocab * n_in).view(np.uint8).copy()
+    else:
+        raw.view(np.uint16)[:] &= np.uint16(0xBFFF)
+    ids = np.array([4, 0, 2, 4], np.uint32)
+    want = ora.embed_rows(raw, fmt, vocab, n_in, ids, out_f16=out_f16)
+    qm = apk.QuantMat(be, dev(raw), fmt, vocab, n_in)
+    out = torch.zeros((ids.size, n_in), dtype=torch.float16 if out_f16 else torch.float32, device="cuda")
+    qm.rows_into(dev(ids), out)
+    v = np.uint16 if out_f16 else np.uint32
+    assert np.array_equal(host(out).view(v), want.view(v))
+
+
 def test_embed_subnormal_scales_and_reference_vectors(be, ora):
     import allpaka_amd as apk
 
