@@ -321,7 +321,17 @@ def other_shapes(args, L, h, apklib, synth, torch, gen, dev, randn, pool, p, tim
         us = timed(lambda i: check(L.apk_embed_rows(h, apklib.FMT_Q4K, p(table), vocab, H, p(ids[i % 8]), rows,
                                                     p(outs[i % len(outs)]), F16)), 200 if rows < T else reps)
         record("embed_rows Q4_K->f16", f"qwen3-32b T={rows}", us, rows * (rb + 4 + H * 2), note=None if rows == T else "launch-bound")
-    del table, outs
+    del table
+    # the same gather from the other common embedding formats of GGUF files (random bytes; the f16 scale
+    # fields are whatever the bytes give -- the kernels do not care)
+    for name, fmt in (("Q6_K", apklib.FMT_Q6K), ("Q8_0", apklib.FMT_Q8_0), ("Q5_K", apklib.FMT_Q5K)):
+        rbx = L.apk_row_bytes(fmt, H)
+        tb = torch.randint(0, 256, (vocab * rbx,), generator=gen, device=dev, dtype=torch.uint8)
+        torch.cuda.synchronize()
+        us = timed(lambda i: check(L.apk_embed_rows(h, fmt, p(tb), vocab, H, p(ids[i % 8]), T, p(outs[i % len(outs)]), F16)), reps)
+        record(f"embed_rows {name}->f16", f"qwen3-32b T={T}", us, T * (rbx + 4 + H * 2))
+        del tb
+    del outs
 
     # Qwen3-0.6B shapes, f32 activations (configs 0 and 1)
     m0 = synth.MODELS["qwen3-0.6b"]
