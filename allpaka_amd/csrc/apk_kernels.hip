@@ -164,6 +164,23 @@ DEV uint32_t total_order_key(float f) {  // f32::total_cmp as an unsigned key
     b ^= (int32_t)(((uint32_t)(b >> 31)) >> 1);
     return (uint32_t)b ^ 0x80000000u;
 }
+DEV uint32_t dpp_u32(uint32_t v, int s) {
+    return s == 0   ? (uint32_t)__builtin_amdgcn_mov_dpp((int)v, DPP_XOR1, 0xf, 0xf, true)
+           : s == 1 ? (uint32_t)__builtin_amdgcn_mov_dpp((int)v, DPP_XOR2, 0xf, 0xf, true)
+           : s == 2 ? (uint32_t)__builtin_amdgcn_mov_dpp((int)v, DPP_HALF_MIRROR, 0xf, 0xf, true)
+                    : (uint32_t)__builtin_amdgcn_mov_dpp((int)v, DPP_MIRROR, 0xf, 0xf, true);
+}
+DEV uint32_t wave_max_u32(uint32_t v) {  // every lane gets the maximum (a wave-uniform value)
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+        const uint32_t o = dpp_u32(v, s);
+        v = o > v ? o : v;
+    }
+    const uint32_t a = (uint32_t)__builtin_amdgcn_readlane((int)v, 0), b = (uint32_t)__builtin_amdgcn_readlane((int)v, 16),
+                   c = (uint32_t)__builtin_amdgcn_readlane((int)v, 32), d = (uint32_t)__builtin_amdgcn_readlane((int)v, 48);
+    const uint32_t ab = a > b ? a : b, cd = c > d ? c : d;
+    return ab > cd ? ab : cd;
+}
 DEV uint64_t max_u64(uint64_t a, uint64_t b) { return a > b ? a : b; }
 DEV uint64_t wave_max_u64(uint64_t v) {  // every lane gets the maximum
     v = max_u64(v, dpp_u64<DPP_XOR1>(v));
@@ -1385,25 +1402,40 @@ DEV void route_topk_body(const float* logits, const float* bias, int rows, int n
     uint32_t my_id = 0;
     float my_score = 0.0f, total = 0.0f;
     for (int r = 0; r < k; r++) {
-        uint64_t best = 0;  // (key << 32) | ~index; 0 = nothing left on this lane
+        // the best key still in play: per lane, then across the wave (32-bit DPP maximum) ...
+        uint32_t lbest = 0;
 #pragma unroll
-        for (int j = 0; j < EPL; j++) {
-            if (!(taken & (1u << j))) {
-                uint64_t cand = ((uint64_t)key[j] << 32) | (uint64_t)(0xffffffffu - (uint32_t)(lane + 64 * j));
-                best = cand > best ? cand : best;
+        for (int j = 0; j < EPL; j++)
+            if (!(taken & (1u << j))) lbest = key[j] > lbest ? key[j] : lbest;
+        const uint32_t best = wave_max_u32(lbest);
+        // ... and its lowest index: expert = lane + 64*j, so the first slot j with a match holds it,
+        // at the lowest matching lane (k <= n_expert: some valid slot is always left, and only valid,
+        // untaken slots can match)
+        int slot = -1, owner = 0;
+        if constexpr (EPL <= 4) {
+#pragma unroll
+            for (int j = 0; j < EPL; j++) {
+                const uint64_t mask = __ballot(!(taken & (1u << j)) && key[j] == best);
+                if (slot < 0 && mask != 0) {  // uniform
+                    slot = j;
+                    owner = __builtin_ctzll(mask);
+                }
             }
-        }
-        best = wave_max_u64(best);
-        const uint32_t e = 0xffffffffu - (uint32_t)(best & 0xffffffffu);
-        const int owner = (int)(e & 63u), slot = (int)(e >> 6);
-        float s = 0.0f;
-        if (lane == owner) {
-            taken |= 1u << slot;
+        } else {  // many slots per lane: each lane's lowest matching index, then a wave minimum
+            uint32_t cand = 0;  // ~index, so that the maximum is the lowest index; 0 = no match
 #pragma unroll
-            for (int j = 0; j < EPL; j++) s = slot == j ? score[j] : s;  // selects, not an indexed (scratch) read
+            for (int j = EPL - 1; j >= 0; j--)
+                if (!(taken & (1u << j)) && key[j] == best) cand = ~(uint32_t)(lane + 64 * j);
+            const uint32_t win = ~wave_max_u32(cand);
+            owner = (int)(win & 63u);
+            slot = (int)(win >> 6);
         }
-        // owner is the same in every lane (it comes out of the wave maximum): a scalar lane select
-        s = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, s), __builtin_amdgcn_readfirstlane(owner)));
+        const uint32_t e = (uint32_t)owner + 64u * (uint32_t)slot;
+        float s = 0.0f;
+#pragma unroll
+        for (int j = 0; j < EPL; j++) s = slot == j ? score[j] : s;  // selects, not an indexed (scratch) read
+        if (lane == owner) taken |= 1u << slot;
+        s = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, s), owner));
         total += s;  // best-first sequential f32 sum, as the reference's iterator sum
         if (lane == r) {
             my_id = e;
