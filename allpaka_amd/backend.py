@@ -310,6 +310,8 @@ class Backend:
         check(self.L.apk_moe_permute(self.h, _ptr(ids), _ptr(w), rows, k, n_expert, _ptr(table), _ptr(n_used), _ptr(tok),
                                      _ptr(tok_off), _ptr(hit_row), _ptr(hit_w)))
         self._leave()
+        if self._recording:  # nothing has run: the whole table, of which a replay fills the leading rows
+            return table, tok, tok_off, hit_row, hit_w
         return table[: int(n_used.item())], tok, tok_off, hit_row, hit_w
 
     def gather_rows(self, src, tok):

@@ -65,7 +65,7 @@ std::vector<std::string> all_kernel_names() {
     std::vector<std::string> v = {"apk_swiglu_f32", "apk_swiglu_f16", "apk_rope_table", "apk_embed_q4k_f32",
                                   "apk_embed_q4k_f16", "apk_embed_q8_0_f32", "apk_embed_q8_0_f16", "apk_route_topk",
                                   "apk_moe_permute", "apk_gather_rows", "apk_scatter_rows", "apk_argmax_rows", "apk_add_rmsnorm_ragged_f32", "apk_copy",
-                                  "apk_qknorm_rope_generic_f32", "apk_qknorm_rope_generic_f16", "apk_route_topk_wide", "apk_add_assign_f32", "apk_add_assign_f16", "apk_softmax_rows"};
+                                  "apk_qknorm_rope_generic_f32", "apk_qknorm_rope_generic_f16", "apk_route_topk_wide", "apk_add_assign_f32", "apk_add_assign_f16", "apk_softmax_rows", "apk_moe_count", "apk_moe_rank"};
     for (const char* t : {"f32", "f16"}) {
         for (const char* f : {"q5k", "q6k", "q2k", "q3k", "q5_0", "f16", "f32", "bf16"}) v.push_back(std::string("apk_embed_") + f + "_" + t);
         for (int c : kAddnormTiles) v.push_back(std::string("apk_add_rmsnorm_") + t + "_c" + std::to_string(c));
@@ -99,6 +99,10 @@ struct apk_ctx {
     size_t capture_nodes = 0;      // launches recorded so far
     bool capture_argmax = false;   // the recording holds the argmax scratch address
     size_t graphs_with_argmax = 0; // live graphs that do: the scratch must not move under them
+    uint32_t* permute_counts = nullptr;  // counts[part][expert] of the two-launch grouping
+    size_t permute_counts_cap = 0;       // in u32
+    bool capture_permute = false;
+    size_t graphs_with_permute = 0;
     std::mutex mu;
     std::map<uintptr_t, Mapping> attached;
     std::atomic<uint64_t> calls{0}, dispatches{0}, encode_ns{0}, wait_ns{0};
@@ -109,6 +113,7 @@ struct apk_graph {
     hipGraphExec_t exec = nullptr;
     size_t nodes = 0;
     bool uses_argmax = false;
+    bool uses_permute = false;
 };
 
 namespace {
@@ -252,6 +257,7 @@ int apk_shutdown(apk_ctx* c) {
     if (c->ids_stage_host) (void)hipHostFree(c->ids_stage_host);
     if (c->fault_dev) (void)hipFree(c->fault_dev);
     if (c->argmax_scratch) (void)hipFree(c->argmax_scratch);
+    if (c->permute_counts) (void)hipFree(c->permute_counts);
     if (c->ev0) (void)hipEventDestroy(c->ev0);
     if (c->ev1) (void)hipEventDestroy(c->ev1);
     if (c->stream) (void)hipStreamDestroy(c->stream);
@@ -409,6 +415,7 @@ int apk_capture_begin(apk_ctx* c) {
     c->capturing = true;
     c->capture_nodes = 0;
     c->capture_argmax = false;
+    c->capture_permute = false;
     return APK_OK;
 }
 
@@ -440,6 +447,8 @@ int apk_capture_end(apk_ctx* c, apk_graph** out) {
     gr->nodes = c->capture_nodes;
     gr->uses_argmax = c->capture_argmax;
     if (gr->uses_argmax) c->graphs_with_argmax++;
+    gr->uses_permute = c->capture_permute;
+    if (gr->uses_permute) c->graphs_with_permute++;
     *out = gr;
     return APK_OK;
 }
@@ -479,6 +488,7 @@ int apk_graph_destroy(apk_ctx* c, apk_graph* g) {
     if (int rc = set_device(c)) return rc;
     HIP_TRY(hipStreamSynchronize(c->stream));  // a replay may still be running
     if (g->uses_argmax && c->graphs_with_argmax) c->graphs_with_argmax--;
+    if (g->uses_permute && c->graphs_with_permute) c->graphs_with_permute--;
     if (g->exec) (void)hipGraphExecDestroy(g->exec);
     if (g->graph) (void)hipGraphDestroy(g->graph);
     delete g;
@@ -881,8 +891,34 @@ int apk_moe_permute(apk_ctx* c, const uint32_t* ids, const float* w, size_t rows
     if (rows * k >= 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_moe_permute: rows*k too large");
     if (int rc = set_device(c)) return rc;
     int rows_i = (int)rows, k_i = (int)k, ne_i = (int)n_expert;
-    void* args[] = {&ids, &w, &rows_i, &k_i, &ne_i, &table, &n_used, &tok, &tok_off, &hit_row, &hit_w, &c->fault_dev};
-    return launch(c, "apk_moe_permute", (unsigned)n_expert, 512, 0, args);
+    if (rows <= 2048) {
+        // one launch: every workgroup (one per expert) walks all picks -- fastest for decode and
+        // medium prefill batches
+        void* args[] = {&ids, &w, &rows_i, &k_i, &ne_i, &table, &n_used, &tok, &tok_off, &hit_row, &hit_w, &c->fault_dev};
+        return launch(c, "apk_moe_permute", (unsigned)n_expert, 512, 0, args);
+    }
+    // large batches: histogram per part of 1024 tokens, then one workgroup per (expert, part)
+    const size_t parts = (rows + 1023) / 1024;
+    if (n_expert * parts > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_moe_permute: too large");
+    const size_t need = parts * n_expert;
+    if (need > c->permute_counts_cap) {
+        if (c->capturing || c->graphs_with_permute)
+            return fail(APK_DECLINE_CAPTURE, "apk_moe_permute: the scratch would have to grow %s",
+                        c->capturing ? "inside a recording (run once unrecorded first)"
+                                     : "while a recorded graph holds its address (destroy the graph first)");
+        HIP_TRY(hipStreamSynchronize(c->stream));  // a previous launch may still use the old scratch
+        if (c->permute_counts) (void)hipFree(c->permute_counts);
+        c->permute_counts = nullptr;
+        c->permute_counts_cap = 0;
+        HIP_TRY(hipMalloc((void**)&c->permute_counts, need * 4));
+        c->permute_counts_cap = need;
+    }
+    if (c->capturing) c->capture_permute = true;
+    int parts_i = (int)parts;
+    void* cargs[] = {&ids, &rows_i, &k_i, &ne_i, &c->permute_counts, &c->fault_dev};
+    if (int rc = launch(c, "apk_moe_count", (unsigned)parts, 512, 0, cargs)) return rc;
+    void* rargs[] = {&ids, &w, &rows_i, &k_i, &ne_i, &parts_i, &c->permute_counts, &table, &n_used, &tok, &tok_off, &hit_row, &hit_w};
+    return launch(c, "apk_moe_rank", (unsigned)(n_expert * parts), 512, 0, rargs);
 }
 
 int apk_gather_rows(apk_ctx* c, const void* src, const uint32_t* tok, size_t src_rows, size_t total_rows, size_t cols,

@@ -1595,6 +1595,146 @@ extern "C" __global__ __launch_bounds__(APK_PERMUTE_THREADS) void apk_moe_permut
     }
 }
 
+// The same grouping for large batches, as two launches.  In the single launch above every
+// workgroup walks all rows*k picks, which is fastest up to a couple of thousand tokens and
+// grows linearly beyond.  Here the tokens are cut into parts of APK_PART_TOKENS:
+//   apk_moe_count  one workgroup per part histograms the part's picks (LDS integer atomics:
+//                  order-independent) into counts[part][expert];
+//   apk_moe_rank   one workgroup per (expert, part): row0 of the expert and the rows of the
+//                  expert in earlier parts come from counts (sums, no atomics), then the part's
+//                  tokens are ranked in token order with the same ballot scan.
+// Same outputs, bit for bit: the order inside an expert is still ascending token order.
+#define APK_PART_TOKENS 1024
+extern "C" __global__ __launch_bounds__(APK_PERMUTE_THREADS) void apk_moe_count(const uint32_t* ids, int rows, int k,
+                                                                                int n_expert, uint32_t* counts,
+                                                                                uint32_t* fault) {
+    __shared__ uint32_t hist[1024];
+    const int part = blockIdx.x, tid = threadIdx.x;
+    for (int i = tid; i < n_expert; i += blockDim.x) hist[i] = 0;
+    __syncthreads();
+    const int t0 = part * APK_PART_TOKENS, t1 = min(rows, t0 + APK_PART_TOKENS);
+    const uint32_t* p0 = ids + (uint64_t)t0 * k;
+    const int total = (t1 - t0) * k;
+    bool bad = false;
+    for (int base = 0; base < total; base += 4 * (int)blockDim.x) {  // four picks in flight per lane
+        uint32_t v[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) v[j] = p0[min(base + j * (int)blockDim.x + tid, total - 1)];
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            if (base + j * (int)blockDim.x + tid < total) {
+                if (v[j] < (uint32_t)n_expert) atomicAdd(&hist[v[j]], 1u);
+                else bad = true;
+            }
+    }
+    if (bad) atomicOr(fault, APK_FAULT_EXPERT_RANGE);
+    __syncthreads();
+    for (int i = tid; i < n_expert; i += blockDim.x) counts[(uint64_t)part * n_expert + i] = hist[i];
+}
+
+extern "C" __global__ __launch_bounds__(APK_PERMUTE_THREADS) void apk_moe_rank(
+    const uint32_t* ids, const float* w, int rows, int k, int n_expert, int parts, const uint32_t* counts, uint32_t* table,
+    uint32_t* n_used_out, uint32_t* tok, uint32_t* tok_off, uint32_t* hit_row, float* hit_w) {
+    __shared__ uint32_t wave_a[APK_PERMUTE_THREADS / 64], wave_b[APK_PERMUTE_THREADS / 64], wave_tot[APK_PERMUTE_THREADS / 64];
+    __shared__ uint32_t s_row0, s_used;
+    const int e = blockIdx.x / parts, part = blockIdx.x - e * parts;
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, nwv = (int)(blockDim.x >> 6);
+    {  // rows of lower experts (all parts) and how many of them are non-empty
+        uint32_t r0 = 0, used = 0;
+        for (int i = tid; i < e; i += blockDim.x) {
+            uint32_t c = 0;
+            for (int q = 0; q < parts; q++) c += counts[(uint64_t)q * n_expert + i];
+            r0 += c;
+            used += c != 0;
+        }
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            r0 += __shfl_xor(r0, o, 64);
+            used += __shfl_xor(used, o, 64);
+        }
+        if (lane == 0) {
+            wave_a[wv] = r0;
+            wave_b[wv] = used;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            uint32_t a = 0, b = 0;
+            for (int i = 0; i < nwv; i++) {
+                a += wave_a[i];
+                b += wave_b[i];
+            }
+            s_row0 = a;
+            s_used = b;
+        }
+        __syncthreads();
+    }
+    uint32_t before = 0, mine_total = 0;  // this expert's rows in earlier parts / in all parts (uniform)
+    for (int q = 0; q < parts; q++) {
+        const uint32_t c = counts[(uint64_t)q * n_expert + e];
+        before += q < part ? c : 0u;
+        mine_total += c;
+    }
+    const uint32_t mine = counts[(uint64_t)part * n_expert + e];
+    const int t0 = part * APK_PART_TOKENS, t1 = min(rows, t0 + APK_PART_TOKENS);
+    if (e == 0) {
+        for (int t = t0 + tid; t < t1; t += blockDim.x) tok_off[t] = (uint32_t)t * (uint32_t)k;
+        if (part == parts - 1 && tid == 0) tok_off[rows] = (uint32_t)rows * (uint32_t)k;
+    }
+    if (part == 0 && tid == 0) {
+        if (mine_total) {
+            table[3 * s_used] = (uint32_t)e;
+            table[3 * s_used + 1] = s_row0;
+            table[3 * s_used + 2] = mine_total;
+        }
+        if (e == n_expert - 1) *n_used_out = s_used + (mine_total != 0);
+    }
+    if (mine == 0) return;  // uniform for the workgroup
+    uint32_t running = s_row0 + before;
+    for (int base = t0; base < t1; base += blockDim.x) {
+        const int t = base + tid;
+        int j_hit = -1, slot = 0;
+        if (t < t1) {
+            const uint32_t* mine_ids = ids + (uint64_t)t * k;
+            int j = 0;
+            if ((k & 3) == 0) {
+                for (; j + 8 <= k; j += 8) {
+                    const u32x4 a = *(const u32x4*)(mine_ids + j), b = *(const u32x4*)(mine_ids + j + 4);
+                    const uint32_t v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        if (v[i] == (uint32_t)e && j_hit < 0) j_hit = j + i;
+                        slot += v[i] < (uint32_t)e;
+                    }
+                }
+            }
+            for (; j < k; j++) {
+                const uint32_t id = mine_ids[j];
+                if (id == (uint32_t)e && j_hit < 0) j_hit = j;
+                slot += id < (uint32_t)e;
+            }
+        }
+        const bool flag = j_hit >= 0;
+        const uint64_t mask = __ballot(flag);
+        const uint32_t in_wave = (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
+        if (lane == 0) wave_tot[wv] = (uint32_t)__popcll(mask);
+        __syncthreads();
+        uint32_t bef = 0, all = 0;
+        for (int i = 0; i < nwv; i++) {
+            const uint32_t c = wave_tot[i];
+            bef += i < wv ? c : 0;
+            all += c;
+        }
+        if (flag) {
+            const uint32_t r = running + bef + in_wave;
+            tok[r] = (uint32_t)t;
+            hit_row[(uint64_t)t * k + slot] = r;
+            hit_w[(uint64_t)t * k + slot] = w[(uint64_t)t * k + j_hit];
+        }
+        running += all;
+        __syncthreads();
+    }
+}
+
 // Gathered activations in tok order (moe.rs:348-352): dst[r,:] = src[tok[r],:].
 // One workgroup per APK_GATHER_ROWS destination rows, 16-byte tiles; row_vecs = row bytes / 16.
 // The source row numbers of the group are read first (uniform for the workgroup), then the

@@ -126,8 +126,8 @@ int apk_timer_end(apk_ctx* ctx, float* ms_out);
  * As there, a graph bakes in every pointer and size its ops were called with, and
  * nothing may allocate, copy to or from the host, or wait inside a recording:
  * apk_sync, apk_malloc, apk_free, apk_h2d, apk_d2h, apk_attach, apk_detach,
- * apk_take_faults, apk_timer_*, apk_embed_rows_host_ids and an apk_argmax_rows that
- * would have to grow its scratch return APK_DECLINE_CAPTURE and record nothing
+ * apk_take_faults, apk_timer_*, apk_embed_rows_host_ids and an apk_argmax_rows or a
+ * large-batch apk_moe_permute that would have to grow its scratch return APK_DECLINE_CAPTURE and record nothing
  * (run the chain once unrecorded first, as the reference does).  A declined op
  * leaves the recording intact.  One recording per context at a time. */
 typedef struct apk_graph apk_graph;

@@ -755,7 +755,9 @@ def test_route_reference_vectors_ties_sigmoid_bias(be, ora):
 
 
 # ------------------------------------------------------- grouping and gather
-@pytest.mark.parametrize("rows,k,n_expert", [(1024, 8, 128), (1, 8, 128), (5, 2, 4), (600, 8, 16), (64, 1, 256), (777, 3, 7), (2048, 8, 128)])
+@pytest.mark.parametrize("rows,k,n_expert", [(1024, 8, 128), (1, 8, 128), (5, 2, 4), (600, 8, 16), (64, 1, 256), (777, 3, 7), (2048, 8, 128),
+                                             # beyond 2048 tokens: the two-launch form (parts of 1024 tokens)
+                                             (2049, 3, 7), (5000, 8, 128), (4096, 8, 256), (3000, 1, 1000), (7001, 6, 60)])
 def test_moe_permute_and_gather_bit_exact(be, ora, rows, k, n_expert):
     s = synth()
     g = s.rng(4, rows + k)

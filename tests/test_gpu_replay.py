@@ -322,3 +322,42 @@ def test_one_recording_serves_every_token_of_a_decode(be, ora, f16):
     assert be.take_faults() == 8  # APK_FAULT_CACHE_RANGE
     assert np.array_equal(host(kc), want_kc)
     rec.graph.destroy()
+
+
+def test_grouping_scratch_cannot_move_under_a_graph(be, ora):
+    """The two-launch grouping of large batches keeps per-part counts in context scratch: same rule as the
+    argmax scratch."""
+    import allpaka_amd as apk
+    from allpaka_amd import synth as s
+
+    b2 = apk.Backend(0)  # fresh context: no scratch yet
+    try:
+        rows, k, ne = 3000, 4, 32
+        logits = s.normal_f32(s.rng(4, 31), (rows, ne))
+        ids, w = ora.route_rows(logits, k, threads=4)
+        want = ora.moe_group(ids, w, ne)
+        dids, dw = dev(ids), dev(w)
+        b2.capture_begin()
+        with pytest.raises(apk.Declined) as e:
+            b2.moe_permute(dids, dw, ne)
+        assert e.value.reason == CAPTURE
+        b2.capture_abort()
+        got = b2.moe_permute(dids, dw, ne)  # unrecorded: allocates the scratch
+        outs = None
+        with b2.record() as rec:
+            outs = b2.moe_permute(dids, dw, ne)
+        assert rec.graph.nodes == 2
+        for t in outs:
+            t.zero_()
+        rec.graph.launch()
+        b2.sync()
+        for name, a, b in zip(["table", "tok", "tok_off", "hit_row", "hit_w"], outs, want):
+            assert np.array_equal(host(a)[: b.shape[0]].view(np.uint32), b.view(np.uint32)), name
+        big_ids = dev(np.zeros((9000, 4), np.uint32) + np.arange(4, dtype=np.uint32))
+        with pytest.raises(apk.Declined) as e:
+            b2.moe_permute(big_ids, dev(np.ones((9000, 4), np.float32)), ne)  # more parts: the scratch would move
+        assert e.value.reason == CAPTURE
+        rec.graph.destroy()
+        assert b2.moe_permute(big_ids, dev(np.ones((9000, 4), np.float32)), ne)[1].numel() == 36000
+    finally:
+        b2.close()
