@@ -1,0 +1,105 @@
+"""Tensors of more than 2^32 bytes / 2^31 elements: the index arithmetic of the streaming kernels is
+64-bit.  Inputs are generated on the device; slices from the start, the 2^31- and 2^32-byte marks and the
+very end are compared with the oracle."""
+import numpy as np
+import pytest
+
+from util import f16_ulp_diff
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+@pytest.fixture(scope="module")
+def be():
+    import allpaka_amd
+
+    b = allpaka_amd.Backend(0)
+    yield b
+    b.close()
+
+
+def bits(t):
+    return t.detach().cpu().numpy().view(np.uint16)
+
+
+def test_streams_past_four_gigabytes(be, ora):
+    n = (1 << 31) + (1 << 20) + 24  # fp16 elements: 4 GiB + 2 MiB + 48 bytes per tensor
+    gen = torch.Generator(device="cuda").manual_seed(11)
+    gate = torch.empty(n, dtype=torch.float16, device="cuda")
+    up = torch.empty(n, dtype=torch.float16, device="cuda")
+    step = 1 << 28
+    for i in range(0, n, step):  # filled in pieces: no 8 GiB float32 temporary
+        m = min(step, n - i)
+        gate[i:i + m] = torch.randn(m, generator=gen, device="cuda", dtype=torch.float32).half()
+        up[i:i + m] = torch.randn(m, generator=gen, device="cuda", dtype=torch.float32).half()
+    windows = [(0, 4096), ((1 << 30) - 2048, 4096), ((1 << 31) - 2048, 4096), (n - 4096, 4096)]
+    before = [(bits(gate[a:a + m]).copy(), bits(up[a:a + m]).copy()) for a, m in windows]
+    be.swiglu(gate, up)
+    for (a, m), (g0, u0) in zip(windows, before):
+        want = g0.copy()
+        ora.swiglu(want, u0)
+        assert f16_ulp_diff(bits(gate[a:a + m]), want) <= 2, a
+        assert np.array_equal(bits(up[a:a + m]), u0)
+    # residual add in place over the same tensors: exact
+    before = [(bits(gate[a:a + m]).copy(), bits(up[a:a + m]).copy()) for a, m in windows]
+    be.add_assign_slice(gate, up)
+    for (a, m), (g0, u0) in zip(windows, before):
+        want = ora.f32_to_f16_bits(ora.f16_bits_to_f32(g0) + ora.f16_bits_to_f32(u0))
+        assert np.array_equal(bits(gate[a:a + m]), want), a
+    # rows x n beyond 2^32 bytes: residual add + RMSNorm over 131 080 rows of 16 384 (the same memory, reshaped)
+    rows, width = 131080, 16384
+    x = gate[: rows * width].view(rows, width)
+    d = up[: rows * width].view(rows, width)
+    h = torch.empty_like(x)
+    gamma = torch.ones(width, device="cuda")
+    pick = [0, 1, 65535, 65536, 131071, 131072, 131079]
+    before = [(bits(x[r]).copy(), bits(d[r]).copy()) for r in pick]
+    be.add_rmsnorm_rows(x, d, h, gamma, 1e-6)
+    for r, (x0, d0) in zip(pick, before):
+        wx, wh = x0.reshape(1, -1).copy(), np.zeros((1, width), np.uint16)
+        ora.add_rmsnorm_rows(wx, d0.reshape(1, -1), wh, np.ones(width, np.float32), 1e-6)
+        assert np.array_equal(bits(x[r]), wx[0]), r
+        assert f16_ulp_diff(bits(h[r]), wh[0]) <= 2, r
+    assert be.take_faults() == 0
+
+
+def test_head_rows_and_permuted_rows_past_four_gigabytes(be, ora):
+    from allpaka_amd import synth as s
+
+    # QK-norm + RoPE over q of 262 200 rows x 64 heads x 128 (4.3 GB of fp16)
+    rows, n_q, n_kv, hd = 262200, 64, 1, 128
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    q = torch.empty((rows, n_q * hd), dtype=torch.float16, device="cuda")
+    for i in range(0, rows, 32768):
+        m = min(32768, rows - i)
+        q[i:i + m] = torch.randn((m, n_q * hd), generator=gen, device="cuda", dtype=torch.float32).half()
+    k = torch.randn((rows, n_kv * hd), generator=gen, device="cuda", dtype=torch.float32).half()
+    g = s.rng(3, 9)
+    qw, kw = s.normal_f32(g, hd, 1.0, 0.05), s.normal_f32(g, hd, 1.0, 0.05)
+    inv = ora.rope_inv_freq(hd, 1e6)
+    pos = torch.arange(rows, dtype=torch.int32, device="cuda") % 32768
+    table = be.rope_table(pos, torch.from_numpy(inv).cuda())
+    pick = [0, 1, 131071, 131072, 262143, 262144, rows - 1]
+    before = [(bits(q[r]).copy(), bits(k[r]).copy()) for r in pick]
+    be.qknorm_rope_neox(q, k, torch.from_numpy(qw).cuda(), torch.from_numpy(kw).cuda(), table, n_q, n_kv, hd, 1e-6)
+    for r, (q0, k0) in zip(pick, before):
+        wq, wk = q0.reshape(1, -1).copy(), k0.reshape(1, -1).copy()
+        ora.qknorm_rope_rows(wq, wk, n_q, n_kv, hd, qw, kw, table[r:r + 1].cpu().numpy(), 1e-6)
+        assert np.array_equal(bits(q[r]), wq[0]) and np.array_equal(bits(k[r]), wk[0]), r
+    del q, k, table
+    # the permuted rows [T*k, 2048] f32 beyond 4 GiB: T = 65 552 tokens, k = 8 (524 416 rows of 8 KiB)
+    T, kk, cols = 65552, 8, 2048
+    hs = torch.randn((T, cols), generator=gen, device="cuda")
+    # a valid CSR by construction: row of hit j of token t is j*T + t (expert-major, token-ascending)
+    hit_row = (torch.arange(kk, device="cuda", dtype=torch.int64)[None, :] * T + torch.arange(T, device="cuda", dtype=torch.int64)[:, None])
+    hit_row = hit_row.to(torch.int32).contiguous()
+    tok = torch.arange(T, device="cuda", dtype=torch.int32).repeat(kk).contiguous()
+    xs = be.scatter_rows(hs, hit_row.view(-1), kk)
+    for r in (0, T - 1, T, 3 * T + 77, 524287, 524288, T * kk - 1):  # 524 288 rows * 8 KiB = 4 GiB
+        assert torch.equal(xs[r], hs[r % T]), r
+    xg = be.gather_rows(hs, tok)
+    for r in (0, T - 1, T, 3 * T + 77, 524287, 524288, T * kk - 1):
+        assert torch.equal(xg[r], hs[r % T]), r
+    assert be.take_faults() == 0
