@@ -64,7 +64,7 @@ const int kQkHeadDims[] = {64, 128, 256};
 std::vector<std::string> all_kernel_names() {
     std::vector<std::string> v = {"apk_swiglu_f32", "apk_swiglu_f16", "apk_rope_table", "apk_embed_q4k_f32",
                                   "apk_embed_q4k_f16", "apk_embed_q8_0_f32", "apk_embed_q8_0_f16", "apk_route_topk",
-                                  "apk_moe_permute", "apk_gather_rows", "apk_scatter_rows", "apk_argmax_rows", "apk_add_rmsnorm_ragged_f32", "apk_copy",
+                                  "apk_moe_permute", "apk_gather_rows", "apk_scatter_rows", "apk_argmax_rows", "apk_add_rmsnorm_ragged_f32", "apk_add_rmsnorm_ragged_f16", "apk_copy",
                                   "apk_qknorm_rope_generic_f32", "apk_qknorm_rope_generic_f16", "apk_route_topk_wide", "apk_add_assign_f32", "apk_add_assign_f16", "apk_softmax_rows", "apk_moe_count", "apk_moe_rank"};
     for (const char* t : {"f32", "f16"}) {
         for (const char* f : {"q5k", "q6k", "q2k", "q3k", "q5_0", "f16", "f32", "bf16"}) v.push_back(std::string("apk_embed_") + f + "_" + t);
@@ -562,35 +562,36 @@ int apk_add_rmsnorm_rows(apk_ctx* c, void* x, const void* delta, void* h, const 
     const size_t vec = 16 / es;
     if (rows > 0x7fffffffu || n > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: too large");
     if (n == 0) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: n is 0");
-    if (n % vec) {
-        // rows that are not whole 16-byte tiles: f32 has an element-wise path, fp16 declines
-        if (dtype != APK_F32) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: n=%zu is not a multiple of %zu", n, vec);
-        if (h == x && delta) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: h aliases x while delta is given");
-        if (int rc = set_device(c)) return rc;
-        int n_r = (int)n;
-        void* rargs[] = {&x, &delta, &h, &gamma, &n_r, &eps};
-        return launch(c, "apk_add_rmsnorm_ragged_f32", (unsigned)rows, 256, 0, rargs);
-    }
-    if (!aligned16(x) || !aligned16(h) || !aligned16(gamma) || (delta && !aligned16(delta)))
-        return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: tensors must be 16-byte aligned");
-    const size_t nchunks = n / vec;
     // Tiles per lane (NCH) and waves per row (W = ceil(nchunks / (64*NCH))): the first
     // choice that keeps the whole batch resident in one round (rows * W <= 2048 waves,
     // 8 per CU) -- a wave per row for prefill batches, many waves per row for a few
     // decode rows -- else the fewest waves per row the register budget allows.
+    const size_t nchunks = n / vec;
     const int max_nch = dtype == APK_F16 ? 10 : 20;
     int nch = 0;
     size_t waves = 0;
-    for (size_t i = 0; i < sizeof kAddnormTiles / sizeof kAddnormTiles[0]; i++) {
-        const int cand = kAddnormTiles[i];
-        if (cand > max_nch) break;
-        const size_t w = (nchunks + 64 * (size_t)cand - 1) / (64 * (size_t)cand);
-        if (w * 64 > (size_t)kAddnormBound[i]) continue;
-        nch = cand;
-        waves = w;
-        if (rows * w <= 2048) break;
+    if (n % vec == 0) {
+        for (size_t i = 0; i < sizeof kAddnormTiles / sizeof kAddnormTiles[0]; i++) {
+            const int cand = kAddnormTiles[i];
+            if (cand > max_nch) break;
+            const size_t w = (nchunks + 64 * (size_t)cand - 1) / (64 * (size_t)cand);
+            if (w * 64 > (size_t)kAddnormBound[i]) continue;
+            nch = cand;
+            waves = w;
+            if (rows * w <= 2048) break;
+        }
     }
-    if (!nch) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: row of %zu elements is too long", n);
+    if (!nch) {
+        // rows that are not whole 16-byte tiles, or longer than the tiled kernels hold in registers
+        // (20 480 elements): the element-wise two-pass kernel
+        if (h == x && delta) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: h aliases x while delta is given");
+        if (int rc = set_device(c)) return rc;
+        int n_r = (int)n;
+        void* rargs[] = {&x, &delta, &h, &gamma, &n_r, &eps};
+        return launch(c, dtype == APK_F32 ? "apk_add_rmsnorm_ragged_f32" : "apk_add_rmsnorm_ragged_f16", (unsigned)rows, 256, 0, rargs);
+    }
+    if (!aligned16(x) || !aligned16(h) || !aligned16(gamma) || (delta && !aligned16(delta)))
+        return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: tensors must be 16-byte aligned");
     const size_t threads = waves * 64;
     if (int rc = set_device(c)) return rc;
     int n_i = (int)n;

@@ -454,32 +454,48 @@ DEV void add_rmsnorm_body(T* x, const T* delta, T* h, const float* gamma, int n,
     if (delta) add_rmsnorm_impl<T, NCH, true>(x, delta, h, gamma, n, eps, vblock);   // uniform for the launch
     else add_rmsnorm_impl<T, NCH, false>(x, delta, h, gamma, n, eps, vblock);
 }
-// f32 rows whose length is not a whole number of 16-byte tiles (so rows are not 16-byte
-// aligned either): one element per lane per step, two passes; the second pass re-reads
-// the lane's own elements of the updated row.  Correctness path for odd shapes (the
-// reference's 2- and 6-element unit tests), not a fast one.
-extern "C" __global__ __launch_bounds__(256) void apk_add_rmsnorm_ragged_f32(float* x, const float* delta, float* h,
-                                                                            const float* gamma, int n, float eps) {
-    __shared__ double part[4];
+// Rows whose length is not a whole number of 16-byte tiles (so rows are not 16-byte aligned
+// either), or longer than the tiled kernels keep in registers: one element per lane per step,
+// two passes over the row.  The first pass only accumulates the statistics of x + delta; the
+// second recomputes the sum, writes it back and normalises the unrounded value -- for fp16 rows
+// the norm must see the f32 sum, not its fp16 rounding.  Correctness path for odd shapes (the
+// reference's 2- and 6-element unit tests, rows beyond 20 480 elements), not a fast one.
+template <typename T>
+DEV void add_rmsnorm_loop_body(T* x, const T* delta, T* h, const float* gamma, int n, float eps) {
+    typedef typename stat<T>::acc_t acc_t;
+    __shared__ acc_t part[4];
     const uint64_t row = blockIdx.x;
-    float* xr = x + row * (uint64_t)n;
-    float* hr = h + row * (uint64_t)n;
-    double ss = 0;
+    T* xr = x + row * (uint64_t)n;
+    T* hr = h + row * (uint64_t)n;
+    const T* dr = delta ? delta + row * (uint64_t)n : nullptr;
+    acc_t ss = 0;
     for (int i = threadIdx.x; i < n; i += blockDim.x) {
-        float v = xr[i];
-        if (delta) {
-            v = v + delta[row * (uint64_t)n + i];
-            xr[i] = v;
-        }
-        ss = stat<float>::sq(ss, v);
+        float v = (float)xr[i];
+        if (dr) v = v + (float)dr[i];
+        ss = stat<T>::sq(ss, v);
     }
-    ss = stat<float>::wave_sum(ss);
+    ss = stat<T>::wave_sum(ss);
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
     __syncthreads();
     ss = 0;
     for (int w = 0; w < (int)(blockDim.x >> 6); w++) ss += part[w];
-    const double scale = stat<float>::rscale(ss, n, eps);
-    for (int i = threadIdx.x; i < n; i += blockDim.x) hr[i] = stat<float>::apply(xr[i], scale, gamma[i]);
+    const typename stat<T>::scale_t scale = stat<T>::rscale(ss, n, eps);
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        float v = (float)xr[i];
+        if (dr) {
+            v = v + (float)dr[i];
+            xr[i] = (T)v;
+        }
+        hr[i] = (T)stat<T>::apply(v, scale, gamma[i]);
+    }
+}
+extern "C" __global__ __launch_bounds__(256) void apk_add_rmsnorm_ragged_f32(float* x, const float* delta, float* h,
+                                                                            const float* gamma, int n, float eps) {
+    add_rmsnorm_loop_body<float>(x, delta, h, gamma, n, eps);
+}
+extern "C" __global__ __launch_bounds__(256) void apk_add_rmsnorm_ragged_f16(f16_t* x, const f16_t* delta, f16_t* h,
+                                                                            const float* gamma, int n, float eps) {
+    add_rmsnorm_loop_body<f16_t>(x, delta, h, gamma, n, eps);
 }
 
 // The launch bound is the largest workgroup the host uses with that tile count

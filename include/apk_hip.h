@@ -182,8 +182,8 @@ int apk_softmax_rows(apk_ctx* ctx, float* x, size_t rows, size_t n);
  * ops::rmsnorm_into / rmsnorm_rows_into (ops/blas.rs:105-178, ops/norm.rs:193-304;
  * call sites model/decode.rs:584,764, model/prefill.rs:155,308-314).
  * x, delta, h: [rows][n] of dtype (h may alias x when delta is NULL);
- * gamma: f32[n].  fp16 rows must be a multiple of 8 elements; f32 rows of any length are
- * taken (a multiple of 4 takes the fast 16-byte-tile path). */
+ * gamma: f32[n].  Rows of any length are taken: whole 16-byte tiles up to 20 480 elements by
+ * the tiled kernels, anything else by an element-wise two-pass kernel. */
 int apk_add_rmsnorm_rows(apk_ctx* ctx, void* x, const void* delta, void* h, const float* gamma, size_t n,
                          size_t rows, float eps, int dtype);
 

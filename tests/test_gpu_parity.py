@@ -263,13 +263,24 @@ def test_rmsnorm_reference_vectors_and_asserts(be, ora):
         be.rmsnorm(torch.zeros(4, device="cuda"), torch.zeros(8, device="cuda"), 0.0)
     import allpaka_amd as apk
 
-    with pytest.raises(apk.Declined):  # fp16 rows that are not whole 16-byte tiles: declined, not faulted
-        be.rmsnorm(torch.zeros(6, device="cuda", dtype=torch.float16), torch.zeros(6, device="cuda"), 0.0)
-    # f32 rows of any length take the element-wise path: ops/mod.rs:130-135 ([1,1] * [2,3]) and odd lengths
+    with pytest.raises(apk.Declined):  # a norm written over its own input while a residual is added: declined
+        t6 = torch.zeros(6, device="cuda")
+        be.add_rmsnorm_rows(t6, t6.clone(), t6, torch.ones(6, device="cuda"), 0.0)
+    # rows of any length take the element-wise path: ops/mod.rs:130-135 ([1,1] * [2,3]), odd lengths, and
+    # rows longer than the tiled kernels hold (beyond 20 480 elements), for both activation types
     x = torch.tensor([1.0, 1.0], device="cuda")
     be.rmsnorm(x, torch.tensor([2.0, 3.0], device="cuda"), 0.0)
     assert abs(host(x)[0] - 2.0) < 1e-5 and abs(host(x)[1] - 3.0) < 1e-5
-    for rows, n in [(1, 6), (5, 1031), (3, 7)]:
+    for rows, n in [(2, 6), (3, 1031), (2, 32768), (1, 40001)]:
+        g = synth().rng(1, n + 1)
+        xs, ds = synth().to_f16_bits(synth().normal_f32(g, (rows, n))), synth().to_f16_bits(synth().normal_f32(g, (rows, n)))
+        gm = synth().normal_f32(g, n, 1.0, 0.05)
+        wx, wh = xs.copy(), np.zeros_like(xs)
+        ora.add_rmsnorm_rows(wx, ds, wh, gm, 1e-6)
+        tx, th = dev(xs), torch.zeros_like(dev(xs))
+        be.add_rmsnorm_rows(tx, dev(ds), th, dev(gm), 1e-6)
+        assert np.array_equal(host(tx), wx) and f16_ulp_diff(host(th), wh) <= TOL_F16_ULP, (rows, n)
+    for rows, n in [(1, 6), (5, 1031), (3, 7), (2, 40004)]:
         g = synth().rng(1, n)
         xs, ds = synth().normal_f32(g, (rows, n)), synth().normal_f32(g, (rows, n))
         gm = synth().normal_f32(g, n, 1.0, 0.05)
