@@ -399,7 +399,30 @@ def other_shapes(args, L, h, apklib, synth, torch, gen, dev, randn, pool, p, tim
     us = timed(lambda i: check(L.apk_moe_combine_add_rmsnorm(h, p(cb[i % len(cb)]["x"]), p(cb[i % len(cb)]["flat"]), p(tok_off), p(hit_row),
                                                              p(hit_w), TM * K, p(cb[i % len(cb)]["h"]), p(gm), HM, TM, EPS, F32)), reps)
     record("moe_combine + add + rmsnorm (one launch)", tagm, us, TM * K * HM * 4 + 3 * TM * HM * 4 + HM * 4 + TM * K * 8)
-    del cb
+    # the five launches of one MoE layer in a row (router, grouping, token-side permute, SwiGLU on the grouped rows,
+    # combine + residual + next norm), op by op and recorded once and replayed
+    se2 = pool(2 * TM * K * FM * 4, lambda: dict(gate=randn((TM * K, FM), f32), up=randn((TM * K, FM), f32)))
+    torch.cuda.synchronize()
+    moe_bytes = (TM * NE * 4 + TM * K * 8) + (TM * K * 8 + TM * K * 12 + TM * 4) + (TM * HM * 4 + TM * K * HM * 4 + TM * K * 4) \
+        + 3 * TM * K * FM * 4 + (TM * K * HM * 4 + 3 * TM * HM * 4 + HM * 4 + TM * K * 8)
+
+    def moe_layer(i):
+        check(L.apk_route_topk(h, p(logits[i % 8]), None, TM, NE, K, 1, 1.0, 0, p(ids_m), p(w_m)))
+        check(L.apk_moe_permute(h, p(ids_m), p(w_m), TM, K, NE, p(tbl), p(n_used), p(tok), p(tok_off), p(hit_row), p(hit_w)))
+        check(L.apk_scatter_rows(h, p(ga[i % len(ga)]["hs"]), p(hit_row), TM, K, TM * K, HM, p(ga[i % len(ga)]["xe"]), F32))
+        check(L.apk_swiglu(h, p(se2[i % len(se2)]["gate"]), p(se2[i % len(se2)]["up"]), TM * K * FM, F32))
+        check(L.apk_moe_combine_add_rmsnorm(h, p(cb[i % len(cb)]["x"]), p(cb[i % len(cb)]["flat"]), p(tok_off), p(hit_row), p(hit_w),
+                                            TM * K, p(cb[i % len(cb)]["h"]), p(gm), HM, TM, EPS, F32))
+
+    record("MoE layer chain (router, grouping, permute, swiglu, combine+norm), op by op", tagm, timed(moe_layer, 24), moe_bytes, launches=5)
+    gmoe = C.c_void_p()
+    check(L.apk_capture_begin(h))
+    for i in range(24):
+        moe_layer(i)
+    check(L.apk_capture_end(h, C.byref(gmoe)))
+    record("MoE layer chain, recorded once and replayed", tagm, timed(lambda i: check(L.apk_graph_launch(h, gmoe)), 6) / 24, moe_bytes, launches=5)
+    check(L.apk_graph_destroy(h, gmoe))
+    del cb, se2
     # greedy pick over the vocabulary (after the output head): 1 and 64 rows of 151936 logits
     V = synth.MODELS["qwen3-32b"]["vocab"]
     lg = [randn((64, V), f32) for _ in range(17)]  # 17 x 38.9 MB
