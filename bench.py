@@ -471,7 +471,32 @@ def cpu_baseline(np, T, H, NQ, NKV, HD, FF, EPS):
         layer()
         times.append(time.perf_counter() - t0)
     med = sorted(times)[len(times) // 2]
-    return {"value": round(med * 1e6, 1), "unit": "us/layer", "cores": cores, "kind": "port",
+
+    def med_us(fn, reps=5):
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        return round(sorted(ts)[len(ts) // 2] * 1e6, 1)
+
+    # the same ops one by one, and the other ops of the path at their benchmark shapes (a few repetitions each)
+    from allpaka_amd import synth
+    per_op = {
+        "add_assign + rmsnorm_rows_into (pool-parallel)": med_us(lambda: (ora.add_assign_par(x.reshape(-1), d.reshape(-1), cores),
+                                                                          ora.rmsnorm_rows_into(hbuf.reshape(-1), x.reshape(-1), gamma, EPS, threads=cores))),
+        "qknorm_rope rows (serial)": med_us(lambda: ora.qknorm_rope_rows(q, k, NQ, NKV, HD, qw, kw, ropes, EPS), 3),
+        "swiglu (serial)": med_us(lambda: (gate.__setitem__(slice(None), up), ora.swiglu(gate.reshape(-1), up.reshape(-1))), 3),
+    }
+    gq = synth.rng(2, 1)
+    table = synth.q4_k_table(gq, 4096, H)  # a slice of the vocabulary is enough for the CPU gather: rows are independent
+    ids = gq.integers(0, 4096, size=T, dtype=np.uint32)
+    per_op["embed_rows Q4_K (serial row_into loop)"] = med_us(lambda: ora.embed_rows(table, ora.FMT["Q4K"], 4096, H, ids), 3)
+    logits = gq.standard_normal((1024, 128), dtype=np.float32)
+    per_op["route_gated, 1024 tokens x 128 experts, k=8 (parallel over tokens)"] = med_us(lambda: ora.route_rows(logits, 8, ora.SOFTMAX, True, 1.0, threads=cores))
+    rid, rw = ora.route_rows(logits, 8, ora.SOFTMAX, True, 1.0, threads=cores)
+    per_op["grouping + CSR, 1024 tokens (serial)"] = med_us(lambda: ora.moe_group(rid, rw, 128))
+    return {"value": round(med * 1e6, 1), "unit": "us/layer", "cores": cores, "kind": "port", "per_op_us": per_op,
             "sample": f"median of {len(times)} repetitions of the whole T={T} layer chain in f32 (the reference's CPU activations are f32); "
                       "C restatement of the reference CPU path, not the reference binary; residual add and row norms "
                       "pool-parallel, QK-norm+RoPE and SwiGLU serial, as the reference runs them"}
