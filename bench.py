@@ -235,6 +235,11 @@ def main():
             h, p(qk[i % len(qk)]["q"]), p(qk[i % len(qk)]["k"]), p(kvp[i % len(qk)]["v"]), p(qw), p(kw), p(rope), p(pos),
             p(kvp[i % len(qk)]["kc"]), p(kvp[i % len(qk)]["vc"]), T, T, NQ, NKV, HD, HD, EPS, F16)), reps)
         record("qknorm_rope_neox + K/V cache store (one launch)", tag, us, bytes_qkrope + T * NKV * HD * b + 2 * T * NKV * HD * 2 + T * 4)
+        # what fusing the residual add into the norm buys: the same result as two launches of this library's own ops
+        us = timed(lambda i: (apklib.check(L.apk_add_assign(h, p(an[i % len(an)]["x"]), p(an[i % len(an)]["d"]), T * H, F16)),
+                              apklib.check(L.apk_add_rmsnorm_rows(h, p(an[i % len(an)]["x"]), None, p(an[i % len(an)]["h"]), p(gamma1), H, T, EPS, F16))), reps)
+        record("UNFUSED residual add, then RMSNorm (two launches)", tag, us, 3 * T * H * b + 2 * T * H * b + 4 * H, launches=2,
+               note="for comparison with add_rmsnorm")
         del an, qk, sw, kvp
         # the same headline shape with f32 activations, the reference's own activation type (f64 statistics,
         # the reference's operation order): twice the bytes per launch
