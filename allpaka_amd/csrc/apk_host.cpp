@@ -69,6 +69,7 @@ std::vector<std::string> all_kernel_names() {
     for (const char* t : {"f32", "f16"}) {
         for (const char* f : {"q5k", "q6k", "q2k", "q3k", "q5_0", "f16", "f32", "bf16"}) v.push_back(std::string("apk_embed_") + f + "_" + t);
         for (int c : kAddnormTiles) v.push_back(std::string("apk_add_rmsnorm_") + t + "_c" + std::to_string(c));
+        for (int l : {4, 8, 16, 32}) v.push_back(std::string("apk_add_rmsnorm_small_") + t + "_l" + std::to_string(l));
         for (int c : {1, 2, 4}) v.push_back(std::string("apk_combine_add_rmsnorm_") + t + "_c" + std::to_string(c));
         for (int hd : kQkHeadDims) v.push_back(std::string("apk_layer_prologue_") + t + "_hd" + std::to_string(hd));
         for (int hd : kQkHeadDims)
@@ -592,6 +593,20 @@ int apk_add_rmsnorm_rows(apk_ctx* c, void* x, const void* delta, void* h, const 
     }
     if (!aligned16(x) || !aligned16(h) || !aligned16(gamma) || (delta && !aligned16(delta)))
         return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: tensors must be 16-byte aligned");
+    if (nchunks <= 32 && rows >= 16) {
+        // short rows in bulk (one head each, say): several rows per wave
+        const int lpr = nchunks <= 4 ? 4 : nchunks <= 8 ? 8 : nchunks <= 16 ? 16 : 32;
+        if (h == x && delta) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: h aliases x while delta is given");
+        const uint64_t rows_per_block = 4 * (64 / lpr);
+        const uint64_t grid = (rows + rows_per_block - 1) / rows_per_block;
+        if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: too large");
+        if (int rc = set_device(c)) return rc;
+        int n_s = (int)n;
+        uint32_t rows32 = (uint32_t)rows;
+        void* sargs[] = {&x, &delta, &h, &gamma, &n_s, &rows32, &eps};
+        return launch(c, std::string("apk_add_rmsnorm_small_") + (dtype == APK_F32 ? "f32" : "f16") + "_l" + std::to_string(lpr),
+                      (unsigned)grid, 256, 0, sargs);
+    }
     const size_t threads = waves * 64;
     if (int rc = set_device(c)) return rc;
     int n_i = (int)n;

@@ -454,6 +454,51 @@ DEV void add_rmsnorm_body(T* x, const T* delta, T* h, const float* gamma, int n,
     if (delta) add_rmsnorm_impl<T, NCH, true>(x, delta, h, gamma, n, eps, vblock);   // uniform for the launch
     else add_rmsnorm_impl<T, NCH, false>(x, delta, h, gamma, n, eps, vblock);
 }
+// Short rows (at most 32 tiles: 256 fp16 / 128 f32 elements, e.g. one head): LPR lanes per row,
+// 64/LPR rows per wave, one tile per lane, the statistics reduced inside the LPR-lane group --
+// a wave per row would leave most lanes idle.
+template <typename T, int LPR>
+DEV void add_rmsnorm_small_body(T* x, const T* delta, T* h, const float* gamma, int n, uint32_t rows, float eps) {
+    constexpr int VEC = io<T>::VEC;
+    typedef typename stat<T>::acc_t acc_t;
+    const int nchunks = n / VEC;
+    const uint32_t lane = threadIdx.x & 63u, l = lane % LPR;
+    const uint64_t row = ((uint64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * (64 / LPR) + lane / LPR;
+    const bool live = row < rows && (int)l < nchunks;
+    const uint64_t off = min(row, (uint64_t)rows - 1) * (uint64_t)n + (uint64_t)min((int)l, nchunks - 1) * VEC;  // clamped: read, not used
+    float g[VEC], v[VEC];
+#pragma unroll
+    for (int q = 0; q < VEC; q += 4) io<float>::load(gamma + min((int)l, nchunks - 1) * VEC + q, g + q);
+    io<T>::load_nt(x + off, v);
+    if (delta) {
+        float d[VEC];
+        io<T>::load_nt(delta + off, d);
+#pragma unroll
+        for (int i = 0; i < VEC; i++) v[i] = v[i] + d[i];
+        if (live) io<T>::store(x + off, v);
+    }
+    acc_t ss = 0;
+    if (live) {
+#pragma unroll
+        for (int i = 0; i < VEC; i++) ss = stat<T>::sq(ss, v[i]);
+    }
+    ss = group_sum<LPR>(ss);
+    const typename stat<T>::scale_t scale = stat<T>::rscale(ss, n, eps);
+    if (live) {
+        float o[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; i++) o[i] = stat<T>::apply(v[i], scale, g[i]);
+        io<T>::store_nt(h + off, o);
+    }
+}
+#define APK_ADDNORM_SMALL(T, TN, LPR)                                                                              \
+    extern "C" __global__ __launch_bounds__(256) void apk_add_rmsnorm_small_##TN##_l##LPR(                         \
+        T* x, const T* delta, T* h, const float* gamma, int n, uint32_t rows, float eps) {                         \
+        add_rmsnorm_small_body<T, LPR>(x, delta, h, gamma, n, rows, eps);                                          \
+    }
+APK_ADDNORM_SMALL(float, f32, 4) APK_ADDNORM_SMALL(float, f32, 8) APK_ADDNORM_SMALL(float, f32, 16) APK_ADDNORM_SMALL(float, f32, 32)
+APK_ADDNORM_SMALL(f16_t, f16, 4) APK_ADDNORM_SMALL(f16_t, f16, 8) APK_ADDNORM_SMALL(f16_t, f16, 16) APK_ADDNORM_SMALL(f16_t, f16, 32)
+
 // Rows whose length is not a whole number of 16-byte tiles (so rows are not 16-byte aligned
 // either), or longer than the tiled kernels keep in registers: one element per lane per step,
 // two passes over the row.  The first pass only accumulates the statistics of x + delta; the
