@@ -577,6 +577,7 @@ int apk_add_rmsnorm_rows(apk_ctx* c, void* x, const void* delta, void* h, const 
             if (cand > max_nch) break;
             const size_t w = (nchunks + 64 * (size_t)cand - 1) / (64 * (size_t)cand);
             if (w * 64 > (size_t)kAddnormBound[i]) continue;
+            if (nch && w >= waves) continue;  // more tiles per lane only where that saves waves (no idle tiles)
             nch = cand;
             waves = w;
             if (rows * w <= 2048) break;
@@ -607,13 +608,18 @@ int apk_add_rmsnorm_rows(apk_ctx* c, void* x, const void* delta, void* h, const 
         return launch(c, std::string("apk_add_rmsnorm_small_") + (dtype == APK_F32 ? "f32" : "f16") + "_l" + std::to_string(lpr),
                       (unsigned)grid, 256, 0, sargs);
     }
-    const size_t threads = waves * 64;
+    // a wave per row: four rows (waves) to a workgroup -- thousands of single-wave workgroups would be bound by
+    // the rate at which the chip starts workgroups
+    const uint32_t rpb = (waves == 1 && rows >= 8) ? 4 : 1;
+    const size_t threads = rpb > 1 ? 256 : waves * 64;
+    const size_t grid = rpb > 1 ? (rows + rpb - 1) / rpb : rows;
     if (int rc = set_device(c)) return rc;
     int n_i = (int)n;
-    void* args[] = {&x, &delta, &h, &gamma, &n_i, &eps};
+    uint32_t rows32 = (uint32_t)rows;
+    void* args[] = {&x, &delta, &h, &gamma, &n_i, &eps, (void*)&rpb, &rows32};
     return launch_keyed(c, OP_ADDNORM, (uint32_t)dtype << 8 | (uint32_t)nch,
                         [&] { return std::string("apk_add_rmsnorm_") + (dtype == APK_F32 ? "f32" : "f16") + "_c" + std::to_string(nch); },
-                        (unsigned)rows, (unsigned)threads, 0, args);
+                        (unsigned)grid, (unsigned)threads, 0, args);
 }
 
 struct KvStore {  // the fused K/V cache store of apk_qknorm_rope_kv_store (all NULL/0: plain op)

@@ -370,12 +370,20 @@ template <> struct headstat<f16_t> {
 };
 
 template <typename T, int NCH, bool HAS_DELTA>
-DEV void add_rmsnorm_impl(T* x, const T* delta, T* h, const float* gamma, int n, float eps, uint32_t vblock) {
+DEV void add_rmsnorm_impl(T* x, const T* delta, T* h, const float* gamma, int n, float eps, uint32_t vblock,
+                          uint32_t rows_per_block, uint32_t rows) {
     constexpr int VEC = io<T>::VEC;
     typedef typename stat<T>::acc_t acc_t;
     __shared__ acc_t part[16];
     const int nchunks = n / VEC;
-    const uint64_t row = vblock;
+    // Two shapes of workgroup: all its waves share one row (rows_per_block == 1: few long rows), or
+    // every wave has a row of its own (a wave covers the row with NCH tiles per lane; the workgroup
+    // only bundles 4 such waves, because the chip starts workgroups at a limited rate -- about 2 ns
+    // each -- and thousands of single-wave workgroups would be bound by that).
+    const bool own_row = rows_per_block > 1;  // uniform
+    const uint32_t tid = own_row ? (threadIdx.x & 63u) : threadIdx.x, stride = own_row ? 64u : blockDim.x;
+    const uint64_t row = own_row ? (uint64_t)vblock * rows_per_block + (threadIdx.x >> 6) : vblock;
+    if (own_row && row >= rows) return;  // whole wave
     T* xr = x + row * (uint64_t)n;
     T* hr = h + row * (uint64_t)n;
     const T* dr = HAS_DELTA ? delta + row * (uint64_t)n : nullptr;
@@ -392,14 +400,14 @@ DEV void add_rmsnorm_impl(T* x, const T* delta, T* h, const float* gamma, int n,
     if constexpr (PRE_GAMMA) {
 #pragma unroll
         for (int j = 0; j < NCH; j++) {
-            const int c = min((int)(threadIdx.x + j * blockDim.x), nchunks - 1);
+            const int c = min((int)(tid + j * stride), nchunks - 1);
 #pragma unroll
             for (int q = 0; q < VEC; q += 4) io<float>::load(gamma + c * VEC + q, gpre[j] + q);
         }
     }
 #pragma unroll
     for (int j = 0; j < NCH; j++) {
-        const int c = min((int)(threadIdx.x + j * blockDim.x), nchunks - 1);
+        const int c = min((int)(tid + j * stride), nchunks - 1);
         xraw[j] = io<T>::ldraw_nt(xr + c * VEC);
         if constexpr (HAS_DELTA) draw[j] = io<T>::ldraw_nt(dr + c * VEC);
     }
@@ -408,7 +416,7 @@ DEV void add_rmsnorm_impl(T* x, const T* delta, T* h, const float* gamma, int n,
     acc_t ss = 0;
 #pragma unroll
     for (int j = 0; j < NCH; j++) {
-        const int c = threadIdx.x + j * blockDim.x;
+        const int c = tid + j * stride;
         io<T>::widen(xraw[j], v[j]);
         if constexpr (HAS_DELTA) {
             float d[VEC];
@@ -423,7 +431,7 @@ DEV void add_rmsnorm_impl(T* x, const T* delta, T* h, const float* gamma, int n,
         ss += c < nchunks ? s8 : (acc_t)0;
     }
     ss = stat<T>::wave_sum(ss);
-    const int nwaves = (blockDim.x + 63) >> 6;
+    const int nwaves = own_row ? 1 : (int)((blockDim.x + 63) >> 6);
     if (nwaves > 1) {
         if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
         __syncthreads();
@@ -433,7 +441,7 @@ DEV void add_rmsnorm_impl(T* x, const T* delta, T* h, const float* gamma, int n,
     const typename stat<T>::scale_t scale = stat<T>::rscale(ss, n, eps);
 #pragma unroll
     for (int j = 0; j < NCH; j++) {
-        const int c = threadIdx.x + j * blockDim.x;
+        const int c = tid + j * stride;
         if (c < nchunks) {
             float g[VEC], o[VEC];
             if constexpr (PRE_GAMMA) {
@@ -450,9 +458,10 @@ DEV void add_rmsnorm_impl(T* x, const T* delta, T* h, const float* gamma, int n,
     }
 }
 template <typename T, int NCH>
-DEV void add_rmsnorm_body(T* x, const T* delta, T* h, const float* gamma, int n, float eps, uint32_t vblock) {
-    if (delta) add_rmsnorm_impl<T, NCH, true>(x, delta, h, gamma, n, eps, vblock);   // uniform for the launch
-    else add_rmsnorm_impl<T, NCH, false>(x, delta, h, gamma, n, eps, vblock);
+DEV void add_rmsnorm_body(T* x, const T* delta, T* h, const float* gamma, int n, float eps, uint32_t vblock,
+                          uint32_t rows_per_block = 1, uint32_t rows = 0) {
+    if (delta) add_rmsnorm_impl<T, NCH, true>(x, delta, h, gamma, n, eps, vblock, rows_per_block, rows);   // uniform for the launch
+    else add_rmsnorm_impl<T, NCH, false>(x, delta, h, gamma, n, eps, vblock, rows_per_block, rows);
 }
 // Short rows (at most 32 tiles: 256 fp16 / 128 f32 elements, e.g. one head): LPR lanes per row,
 // 64/LPR rows per wave, one tile per lane, the statistics reduced inside the LPR-lane group --
@@ -547,8 +556,8 @@ extern "C" __global__ __launch_bounds__(256) void apk_add_rmsnorm_ragged_f16(f16
 // (it also caps the registers the compiler may take: 512 / (bound/64/4) per lane).
 #define APK_ADDNORM(T, TN, NCH, MAXT)                                                                        \
     extern "C" __global__ __launch_bounds__(MAXT) void apk_add_rmsnorm_##TN##_c##NCH(                        \
-        T* x, const T* delta, T* h, const float* gamma, int n, float eps) {                                  \
-        add_rmsnorm_body<T, NCH>(x, delta, h, gamma, n, eps, blockIdx.x);                                    \
+        T* x, const T* delta, T* h, const float* gamma, int n, float eps, uint32_t rows_per_block, uint32_t rows) { \
+        add_rmsnorm_body<T, NCH>(x, delta, h, gamma, n, eps, blockIdx.x, rows_per_block, rows);              \
     }
 #define APK_ADDNORM_ALL(T, TN)                                                                                   \
     APK_ADDNORM(T, TN, 1, 1024) APK_ADDNORM(T, TN, 2, 1024) APK_ADDNORM(T, TN, 3, 512) APK_ADDNORM(T, TN, 4, 512) \
