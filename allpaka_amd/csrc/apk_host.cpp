@@ -58,7 +58,7 @@ struct Mapping {
 // missing symbol fails there and not at the first launch.
 const int kAddnormTiles[] = {1, 2, 3, 4, 5, 6, 8, 10, 12, 16, 20};  // 16-byte tiles per lane
 const int kAddnormBound[] = {1024, 1024, 512, 512, 256, 256, 256, 256, 256, 256, 256};  // launch bound of each
-const int kQkIters[] = {1, 2, 4, 8};
+const int kQkIters[] = {1, 2};
 const int kQkHeadDims[] = {64, 128, 256};
 
 std::vector<std::string> all_kernel_names() {
@@ -667,19 +667,16 @@ static int qknorm_rope_common(apk_ctx* c, void* q, void* k, const float* qw, con
         return launch(c, dtype == APK_F32 ? "apk_qknorm_rope_generic_f32" : "apk_qknorm_rope_generic_f16", (unsigned)grid, 256, 0, gargs);
     }
     // A wave owns (row, q or k, group of HPW*ITER heads), HPW = heads per wave pass; k waves
-    // take one pass.  The largest ITER for q that still leaves >= 1536 waves (6 per CU)
-    // amortises the row's [sin, cos] tile and the norm weight over the most heads; small
-    // batches take ITER = 1.
+    // take one pass.  Measured over 1024..8192 rows: fp16 is fastest with two passes per q wave
+    // (16 heads, 4 KB), f32 with one (4 heads, 2 KB); more passes per wave gain nothing where
+    // the batch happens to be a whole number of resident rounds and lose up to 15 % elsewhere.
+    // Small batches (under 6 waves per CU) take one pass: more waves.
     const size_t epl = 16 / es, lph = head_dim / 2 / epl, hpw = 64 / lph;
     const size_t gk = (n_kv + hpw - 1) / hpw;
     int iter = 1;
-    for (int cand : {8, 4, 2}) {
-        if ((size_t)cand > (n_q + hpw - 1) / hpw) continue;
-        const size_t gq = (n_q + hpw * cand - 1) / (hpw * cand);
-        if (rows * (gq + gk) >= 1536) { iter = cand; break; }
-    }
+    if (dtype == APK_F16 && n_q > hpw && rows * ((n_q + 2 * hpw - 1) / (2 * hpw) + gk) >= 1536) iter = 2;
     const uint64_t waves = (uint64_t)rows * ((n_q + hpw * iter - 1) / (hpw * iter) + gk);
-    const unsigned block = iter >= 4 ? 64 : 256;
+    const unsigned block = 256;
     const uint64_t grid = (waves * 64 + block - 1) / block;
     if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope: too large");
     if (validate_only) return APK_OK;

@@ -378,8 +378,7 @@ DEV void add_rmsnorm_impl(T* x, const T* delta, T* h, const float* gamma, int n,
     const int nchunks = n / VEC;
     // Two shapes of workgroup: all its waves share one row (rows_per_block == 1: few long rows), or
     // every wave has a row of its own (a wave covers the row with NCH tiles per lane; the workgroup
-    // only bundles 4 such waves, because the chip starts workgroups at a limited rate -- about 2 ns
-    // each -- and thousands of single-wave workgroups would be bound by that).
+    // only bundles 4 such waves, which the host asks for where rows come in their thousands).
     const bool own_row = rows_per_block > 1;  // uniform
     const uint32_t tid = own_row ? (threadIdx.x & 63u) : threadIdx.x, stride = own_row ? 64u : blockDim.x;
     const uint64_t row = own_row ? (uint64_t)vblock * rows_per_block + (threadIdx.x >> 6) : vblock;
@@ -766,8 +765,10 @@ extern "C" __global__ __launch_bounds__(256) void apk_argmax_rows(const float* l
 // heads), HPW = 64/LPH heads per pass: one tensor per wave means one norm
 // weight per wave and no per-element selects; the row's [sin, cos] tile and
 // the weight are loaded once and reused over ITER passes (q: ITERQ passes,
-// k: 1 pass -- under GQA k has few heads).  The host picks ITERQ so that a
-// large batch is about one resident round of waves.
+// k: 1 pass -- under GQA k has few heads).  Waves are kept short (ITERQ 1 or 2, about
+// 4 KB of heads each): a wave that carries a row's 64 q heads in 8 passes lives as long as
+// the whole launch, and a batch a few rows beyond one resident round of such waves
+// (2061 rows instead of 2048) then takes 15 % longer; short waves fill in evenly.
 // Arithmetic: the reference's, for both activation types (see `headstat`): f64 statistics,
 // (x as f64 * scale) as f32 * w, then the four products and two sums of the rotation,
 // not contracted.  fp16 results are that f32 result rounded once.
@@ -891,8 +892,7 @@ DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const fl
         }
     }
 }
-// At most 128 VGPRs (4 waves per SIMD): the q waves of a 2048-row batch are 8 per CU and the k
-// waves another 8, so at 16 resident waves per CU the whole launch is one round with no tail.
+// At most 128 VGPRs (at least 4 waves per SIMD).
 #define APK_QK_OCC __attribute__((amdgpu_waves_per_eu(4)))
 #define APK_QKROPE(T, TN, HD, ITER)                                                                          \
     extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void apk_qknorm_rope_##TN##_hd##HD##_i##ITER(   \
@@ -900,9 +900,8 @@ DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const fl
         qknorm_rope_body<T, HD, ITER>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, blockIdx.x);                  \
     }
 #define APK_QKROPE_ALL(T, TN)                                                                                          \
-    APK_QKROPE(T, TN, 64, 1) APK_QKROPE(T, TN, 64, 2) APK_QKROPE(T, TN, 64, 4) APK_QKROPE(T, TN, 64, 8)                \
-    APK_QKROPE(T, TN, 128, 1) APK_QKROPE(T, TN, 128, 2) APK_QKROPE(T, TN, 128, 4) APK_QKROPE(T, TN, 128, 8)            \
-    APK_QKROPE(T, TN, 256, 1) APK_QKROPE(T, TN, 256, 2) APK_QKROPE(T, TN, 256, 4) APK_QKROPE(T, TN, 256, 8)
+    APK_QKROPE(T, TN, 64, 1) APK_QKROPE(T, TN, 64, 2) APK_QKROPE(T, TN, 128, 1) APK_QKROPE(T, TN, 128, 2)              \
+    APK_QKROPE(T, TN, 256, 1) APK_QKROPE(T, TN, 256, 2)
 APK_QKROPE_ALL(float, f32)
 APK_QKROPE_ALL(f16_t, f16)
 
@@ -916,9 +915,8 @@ APK_QKROPE_ALL(f16_t, f16)
                                             k_cache, v_cache, capacity, fault);                                   \
     }
 #define APK_QKROPE_KV_ALL(T, TN)                                                                                       \
-    APK_QKROPE_KV(T, TN, 64, 1) APK_QKROPE_KV(T, TN, 64, 2) APK_QKROPE_KV(T, TN, 64, 4) APK_QKROPE_KV(T, TN, 64, 8)    \
-    APK_QKROPE_KV(T, TN, 128, 1) APK_QKROPE_KV(T, TN, 128, 2) APK_QKROPE_KV(T, TN, 128, 4) APK_QKROPE_KV(T, TN, 128, 8) \
-    APK_QKROPE_KV(T, TN, 256, 1) APK_QKROPE_KV(T, TN, 256, 2) APK_QKROPE_KV(T, TN, 256, 4) APK_QKROPE_KV(T, TN, 256, 8)
+    APK_QKROPE_KV(T, TN, 64, 1) APK_QKROPE_KV(T, TN, 64, 2) APK_QKROPE_KV(T, TN, 128, 1) APK_QKROPE_KV(T, TN, 128, 2)  \
+    APK_QKROPE_KV(T, TN, 256, 1) APK_QKROPE_KV(T, TN, 256, 2)
 APK_QKROPE_KV_ALL(float, f32)
 APK_QKROPE_KV_ALL(f16_t, f16)
 
