@@ -64,7 +64,7 @@ const int kQkHeadDims[] = {64, 128, 256};
 std::vector<std::string> all_kernel_names() {
     std::vector<std::string> v = {"apk_swiglu_f32", "apk_swiglu_f16", "apk_rope_table", "apk_embed_q4k_f32",
                                   "apk_embed_q4k_f16", "apk_embed_q8_0_f32", "apk_embed_q8_0_f16", "apk_route_topk",
-                                  "apk_moe_permute", "apk_gather_rows", "apk_scatter_rows", "apk_argmax_rows", "apk_add_rmsnorm_ragged_f32", "apk_add_rmsnorm_ragged_f16", "apk_copy",
+                                  "apk_moe_permute", "apk_gather_rows", "apk_scatter_rows_t1", "apk_scatter_rows_t2", "apk_argmax_rows", "apk_add_rmsnorm_ragged_f32", "apk_add_rmsnorm_ragged_f16", "apk_copy",
                                   "apk_qknorm_rope_generic_f32", "apk_qknorm_rope_generic_f16", "apk_route_topk_wide", "apk_add_assign_f32", "apk_add_assign_f16", "apk_softmax_rows", "apk_moe_count", "apk_moe_rank"};
     for (const char* t : {"f32", "f16"}) {
         for (const char* f : {"q5k", "q6k", "q2k", "q3k", "q5_0", "f16", "f32", "bf16"}) v.push_back(std::string("apk_embed_") + f + "_" + t);
@@ -986,11 +986,18 @@ int apk_scatter_rows(apk_ctx* c, const void* src, const uint32_t* hit_row, size_
         return fail(APK_DECLINE_SHAPE, "apk_scatter_rows: rows must be whole 16-byte tiles");
     if (rows > 0x7fffffffu || total_rows > 0xffffffffu || k > 0x7fffffffu || cols * es / 16 > 0x7fffffffu)
         return fail(APK_DECLINE_SHAPE, "apk_scatter_rows: too large");
+    // one workgroup per (token, slice, hit); one 16-byte tile per lane from 64 MB of output on, two below
+    // (fewer, slightly longer waves are ahead while the launch is short)
+    const int row_vecs = (int)(cols * es / 16);
+    const int tpt = (uint64_t)rows * k * cols * es >= (64u << 20) ? 1 : 2;
+    const uint64_t slices = ((uint64_t)row_vecs + 256 * tpt - 1) / (256 * tpt);
+    const uint64_t items = (uint64_t)rows * slices;
+    const uint64_t grid = (items + 7) / 8 * 8 * k;
+    if (items > 0xffffffffu || grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_scatter_rows: too large");
     if (int rc = set_device(c)) return rc;
-    int k_i = (int)k, row_vecs = (int)(cols * es / 16);
-    uint32_t total32 = (uint32_t)total_rows;
-    void* args[] = {&src, &hit_row, &k_i, &total32, &row_vecs, &dst, &c->fault_dev};
-    return launch(c, "apk_scatter_rows", (unsigned)rows, 256, 0, args);
+    uint32_t k32 = (uint32_t)k, total32 = (uint32_t)total_rows, items32 = (uint32_t)items, slices32 = (uint32_t)slices;
+    void* args[] = {&src, &hit_row, &k32, &total32, (void*)&row_vecs, &dst, &c->fault_dev, &items32, &slices32};
+    return launch(c, tpt == 1 ? "apk_scatter_rows_t1" : "apk_scatter_rows_t2", (unsigned)grid, 256, 0, args);
 }
 
 int apk_moe_combine_add_rmsnorm(apk_ctx* c, void* x, const void* flat, const uint32_t* tok_off, const uint32_t* hit_row,

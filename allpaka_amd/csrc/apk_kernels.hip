@@ -1848,29 +1848,47 @@ extern "C" __global__ __launch_bounds__(256) void apk_gather_rows(const u32x4* s
 // The same permutation driven from the token side: dst[hit_row[t*k + j], :] = src[t, :]
 // for the k hits of token t (the CSR lists of apk_moe_permute).  Each source row is read
 // from HBM once and written k times; the gather form above re-reads it from every XCD's
-// own L2 (8 XCDs, 8 fills of the same row through the fabric).  One workgroup per token.
-extern "C" __global__ __launch_bounds__(256) void apk_scatter_rows(const u32x4* src, const uint32_t* hit_row, int k,
-                                                                  uint32_t total_rows, int row_vecs, u32x4* dst,
-                                                                  uint32_t* fault) {
-    const uint64_t t = blockIdx.x;
-    const u32x4* sp = src + t * row_vecs;
-    const uint32_t* hits = hit_row + t * k;
-    for (int c = threadIdx.x; c < row_vecs; c += 2 * blockDim.x) {
-        const int c2 = c + blockDim.x;
-        const bool two = c2 < row_vecs;
-        const u32x4 a = __builtin_nontemporal_load(sp + c);
-        const u32x4 b = __builtin_nontemporal_load(sp + (two ? c2 : c));
-        for (int j = 0; j < k; j++) {
-            const uint32_t r = hits[j];
-            if (r >= total_rows) {
-                if (c == 0) atomicOr(fault, APK_FAULT_ROW_RANGE);
-                continue;
-            }
-            u32x4* dp = dst + (uint64_t)r * row_vecs;
-            __builtin_nontemporal_store(a, dp + c);
-            if (two) __builtin_nontemporal_store(b, dp + c2);
-        }
+// own L2 (8 XCDs, 8 fills of the same row through the fabric).
+// One workgroup per (token, slice of 256*TPT tiles, hit): TPT loads and TPT stores per lane and
+// the wave is gone -- a write-heavy launch runs faster the shorter its waves are (a workgroup
+// that kept a token's tiles and stored them k times took 62 us where this takes 50 us, for
+// 302 MB; a plain copy of as many bytes 48 us).  The k workgroups that share a source slice are
+// consecutive on one XCD (workgroup b is started on XCD b % 8), so k - 1 of the k loads hit
+// that XCD's L2; without that order the launch takes 76 us.
+template <int TPT>
+DEV void scatter_rows_body(const u32x4* src, const uint32_t* hit_row, uint32_t k, uint32_t total_rows, int row_vecs,
+                           u32x4* dst, uint32_t* fault, uint32_t items, uint32_t slices) {
+    const uint32_t b = blockIdx.x, xcd = b & 7u, m = b >> 3;
+    const uint32_t item = xcd + 8u * (m / k), j = m % k;
+    if (item >= items) return;  // uniform
+    const uint32_t t = item / slices, s = item - t * slices;
+    const uint32_t r = hit_row[(uint64_t)t * k + j];
+    const u32x4* sp = src + (uint64_t)t * row_vecs;
+    u32x4 a[TPT];
+    int c[TPT];
+#pragma unroll
+    for (int i = 0; i < TPT; i++) {
+        c[i] = (int)((s * TPT + i) * 256u + threadIdx.x);
+        a[i] = sp[min(c[i], row_vecs - 1)];  // not nontemporal: the next k - 1 workgroups want it in L2
     }
+    if (r >= total_rows) {  // uniform
+        if (threadIdx.x == 0 && s == 0) atomicOr(fault, APK_FAULT_ROW_RANGE);
+        return;
+    }
+    u32x4* dp = dst + (uint64_t)r * row_vecs;
+#pragma unroll
+    for (int i = 0; i < TPT; i++)
+        if (c[i] < row_vecs) __builtin_nontemporal_store(a[i], dp + c[i]);
+}
+extern "C" __global__ __launch_bounds__(256) void apk_scatter_rows_t1(const u32x4* src, const uint32_t* hit_row, uint32_t k,
+                                                                     uint32_t total_rows, int row_vecs, u32x4* dst,
+                                                                     uint32_t* fault, uint32_t items, uint32_t slices) {
+    scatter_rows_body<1>(src, hit_row, k, total_rows, row_vecs, dst, fault, items, slices);
+}
+extern "C" __global__ __launch_bounds__(256) void apk_scatter_rows_t2(const u32x4* src, const uint32_t* hit_row, uint32_t k,
+                                                                     uint32_t total_rows, int row_vecs, u32x4* dst,
+                                                                     uint32_t* fault, uint32_t items, uint32_t slices) {
+    scatter_rows_body<2>(src, hit_row, k, total_rows, row_vecs, dst, fault, items, slices);
 }
 
 // Reference stream for bandwidth calibration: dst = src, one 16-byte tile per lane.

@@ -857,6 +857,24 @@ def test_permute_declines_and_faults(be):
     assert be.take_faults() & 4 and np.all(host(out)[[0, 1, 3]] == 1.0)
 
 
+@pytest.mark.parametrize("rows,k,cols,f16", [(600, 8, 3600, False), (600, 8, 3600, True), (3, 2, 8200, False), (4099, 1, 520, True),
+                                             (9, 64, 4, False)])
+def test_scatter_rows_is_the_permutation(be, rows, k, cols, f16):
+    """dst[hit_row[t*k + j]] = src[t] for any permutation of the rows, bit for bit: both slice widths
+    (outputs under and over 64 MiB), rows that end inside a slice, slice counts that do not fill the last
+    group of eight workgroups."""
+    gen = torch.Generator(device="cuda").manual_seed(rows * 31 + cols)
+    src = torch.randn((rows, cols), generator=gen, device="cuda")
+    if f16:
+        src = src.half()
+    hit_row = torch.randperm(rows * k, generator=gen, device="cuda").to(torch.int32)
+    out = be.scatter_rows(src, hit_row, k)
+    want = torch.empty_like(out)
+    want[hit_row.long()] = src.repeat_interleave(k, dim=0)
+    assert be.take_faults() == 0
+    assert torch.equal(out, want)
+
+
 # ----------------------------------------------- full-size property checks
 def test_full_size_prefill_properties(be, ora):
     """Qwen3-32B shapes at T=2048 (fp16): the oracle checks a row subset; the rest is
