@@ -65,7 +65,7 @@ std::vector<std::string> all_kernel_names() {
     std::vector<std::string> v = {"apk_swiglu_f32", "apk_swiglu_f16", "apk_rope_table", "apk_embed_q4k_f32",
                                   "apk_embed_q4k_f16", "apk_embed_q8_0_f32", "apk_embed_q8_0_f16", "apk_route_topk",
                                   "apk_moe_permute", "apk_gather_rows", "apk_scatter_rows_t1", "apk_scatter_rows_t2", "apk_argmax_rows", "apk_add_rmsnorm_ragged_f32", "apk_add_rmsnorm_ragged_f16", "apk_copy",
-                                  "apk_qknorm_rope_generic_f32", "apk_qknorm_rope_generic_f16", "apk_route_topk_wide", "apk_add_assign_f32", "apk_add_assign_f16", "apk_softmax_rows", "apk_moe_count", "apk_moe_rank"};
+                                  "apk_qknorm_rope_generic_f32", "apk_qknorm_rope_generic_f16", "apk_route_topk_wide", "apk_route_topk_e64", "apk_route_topk_e128", "apk_add_assign_f32", "apk_add_assign_f16", "apk_softmax_rows", "apk_moe_count", "apk_moe_rank"};
     for (const char* t : {"f32", "f16"}) {
         for (const char* f : {"q5k", "q6k", "q2k", "q3k", "q5_0", "f16", "f32", "bf16"}) v.push_back(std::string("apk_embed_") + f + "_" + t);
         for (int c : kAddnormTiles) v.push_back(std::string("apk_add_rmsnorm_") + t + "_c" + std::to_string(c));
@@ -910,7 +910,8 @@ int apk_route_topk(apk_ctx* c, const float* logits, const float* bias, size_t ro
     const unsigned block = 256, per_block = block / 64;
     const uint64_t grid = (rows + per_block - 1) / per_block;
     void* args[] = {&logits, &bias, &rows_i, &ne_i, &k_i, &norm, &scale, &sigmoid, &ids, &w};
-    return launch(c, n_expert <= 256 ? "apk_route_topk" : "apk_route_topk_wide", (unsigned)grid, block, 0, args);
+    const char* which = n_expert <= 64 ? "apk_route_topk_e64" : n_expert <= 128 ? "apk_route_topk_e128" : n_expert <= 256 ? "apk_route_topk" : "apk_route_topk_wide";
+    return launch(c, which, (unsigned)grid, block, 0, args);
 }
 
 int apk_moe_permute(apk_ctx* c, const uint32_t* ids, const float* w, size_t rows, size_t k, size_t n_expert,

@@ -1522,6 +1522,17 @@ extern "C" __global__ __launch_bounds__(256) void apk_route_topk(const float* lo
                                                                 int sigmoid, uint32_t* ids, float* wout) {
     route_topk_body<4>(logits, bias, rows, n_expert, k, norm, scale, sigmoid, ids, wout);
 }
+// narrow routers: one or two experts per lane (a round of the selection costs per slot held)
+extern "C" __global__ __launch_bounds__(256) void apk_route_topk_e64(const float* logits, const float* bias, int rows,
+                                                                    int n_expert, int k, int norm, float scale,
+                                                                    int sigmoid, uint32_t* ids, float* wout) {
+    route_topk_body<1>(logits, bias, rows, n_expert, k, norm, scale, sigmoid, ids, wout);
+}
+extern "C" __global__ __launch_bounds__(256) void apk_route_topk_e128(const float* logits, const float* bias, int rows,
+                                                                     int n_expert, int k, int norm, float scale,
+                                                                     int sigmoid, uint32_t* ids, float* wout) {
+    route_topk_body<2>(logits, bias, rows, n_expert, k, norm, scale, sigmoid, ids, wout);
+}
 // routers wider than 256 experts (the reference's heap path, moe.rs:536-545): up to 1024
 extern "C" __global__ __launch_bounds__(256) void apk_route_topk_wide(const float* logits, const float* bias, int rows,
                                                                      int n_expert, int k, int norm, float scale,

@@ -699,7 +699,8 @@ def _ref_logits(n):
 
 
 @pytest.mark.parametrize("rows,n_expert,k", [(1024, 128, 8), (1, 128, 8), (7, 64, 4), (33, 256, 8), (5, 60, 6), (3, 4, 4), (9, 200, 1),
-                                            (40, 257, 8), (17, 384, 6), (5, 1024, 8), (3, 1000, 64)])
+                                            (40, 257, 8), (17, 384, 6), (5, 1024, 8), (3, 1000, 64), (33, 65, 8), (12, 100, 64), (6, 129, 8),
+                                            (9, 64, 64)])
 @pytest.mark.parametrize("norm,scale", [(True, 1.0), (False, 1.5)])
 def test_route_topk(be, ora, rows, n_expert, k, norm, scale):
     s = synth()
