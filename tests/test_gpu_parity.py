@@ -224,7 +224,9 @@ def test_embed_errors_and_declines(be, ora):
 @pytest.mark.parametrize("n,rows", [(1024, 1), (1024, 512), (5120, 1), (5120, 6), (5120, 64), (2048, 33), (128, 5),
                                     (8, 3), (4096 + 64, 3), (8192, 2), (16384, 2),
                                     # short rows in bulk: several rows per wave
-                                    (128, 100), (8, 33), (256, 77), (64, 1000), (24, 16), (200, 19), (104, 4097)])
+                                    (128, 100), (8, 33), (256, 77), (64, 1000), (24, 16), (200, 19), (104, 4097),
+                                    # batches beyond one resident round of waves: two tiles per lane, several waves per row
+                                    (5120, 4100), (4096, 2100), (16384, 1030), (1032, 4100), (8192, 520), (2560, 8200)])
 @pytest.mark.parametrize("f16", [False, True])
 @pytest.mark.parametrize("with_delta", [True, False])
 def test_add_rmsnorm_rows(be, ora, n, rows, f16, with_delta):
