@@ -415,6 +415,15 @@ class QuantMat:
         check(self.b.L.apk_embed_rows_host_ids(self.b.h, self.ty, _ptr(self.data), self.n_out, self.n_in, ids, 1, _ptr(dst), _dt(dst)))
         self.b.sync()
 
+    def dequant_rows(self, row0, count, dtype=torch.float16):
+        """Rows [row0, row0 + count) dequantized without an id list: QuantMat::row_into over a range, or the
+        reference's dequant_rows_f16 ahead of a dense GEMM (gpu/cuda/runtime/gemm.rs:213-260)."""
+        out = torch.empty((count, self.n_in), dtype=dtype, device=self.b.device)
+        self.b._enter()
+        check(self.b.L.apk_dequant_rows(self.b.h, self.ty, _ptr(self.data), self.n_out, self.n_in, row0, count, _ptr(out), _dt(out)))
+        self.b._leave()
+        return out
+
     def rows_into(self, ids, dst, embed_scale=1.0):
         """The embedding loop of forward_batch (prefill.rs:92-109) as one launch; ids on the device;
         embed_scale: the multiplier of models that scale their token embeddings."""

@@ -787,12 +787,13 @@ int apk_rope_table(apk_ctx* c, const uint32_t* positions, const float* inv_freq,
     return launch(c, "apk_rope_table", (unsigned)grid, 256, 0, args);
 }
 
+// ids_dev == nullptr with have_ids == false: the rows row0, row0 + 1, ... (apk_dequant_rows)
 static int embed_common(apk_ctx* c, int fmt, const void* table, size_t vocab, size_t n_in, const uint32_t* ids_dev,
-                        size_t t, void* out, int out_dtype, float scale = 1.0f) {
+                        size_t t, void* out, int out_dtype, float scale = 1.0f, bool have_ids = true, uint32_t row0 = 0) {
     if (!apk_can_embed(fmt, n_in)) return fail(APK_DECLINE_UNSUPPORTED, "apk_embed_rows: fmt %d / n_in %zu", fmt, n_in);
     if (!elem_size(out_dtype)) return fail(APK_DECLINE_UNSUPPORTED, "apk_embed_rows: out_dtype %d", out_dtype);
     if (t == 0) return APK_OK;
-    if (!table || !ids_dev || !out) return fail(APK_DECLINE_NULL, "apk_embed_rows: NULL tensor");
+    if (!table || (have_ids && !ids_dev) || !out) return fail(APK_DECLINE_NULL, "apk_embed_rows: NULL tensor");
     if (!aligned16(table) || !aligned16(out)) return fail(APK_DECLINE_SHAPE, "apk_embed_rows: table/out must be 16-byte aligned");
     if (vocab == 0 || vocab > 0xffffffffu || n_in > 0x7fffffffu || t > 0x7fffffffu)
         return fail(APK_DECLINE_SHAPE, "apk_embed_rows: sizes out of range");
@@ -803,7 +804,7 @@ static int embed_common(apk_ctx* c, int fmt, const void* table, size_t vocab, si
         // one workgroup per row, 8 lanes per 256-element super-block
         size_t threads = (n_in / 256 * 8 + 63) / 64 * 64;
         if (threads > 256) threads = 256;
-        void* args[] = {&table, &vocab32, &n_i, &ids_dev, &out, &c->fault_dev, &scale};
+        void* args[] = {&table, &vocab32, &n_i, &ids_dev, &out, &c->fault_dev, &scale, &row0};
         return launch_keyed(c, OP_EMBED, (uint32_t)fmt << 8 | (uint32_t)out_dtype,
                             [&] { return std::string(out_dtype == APK_F32 ? "apk_embed_q4k_f32" : "apk_embed_q4k_f16"); }, (unsigned)t,
                             (unsigned)threads, 0, args);
@@ -818,7 +819,7 @@ static int embed_common(apk_ctx* c, int fmt, const void* table, size_t vocab, si
         const uint64_t grid = (uint64_t)t * chunks;
         if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_embed_rows: too large");
         uint32_t chunks32 = (uint32_t)chunks;
-        void* args[] = {&table, &vocab32, &n_i, &ids_dev, &chunks32, &out, &c->fault_dev, &scale};
+        void* args[] = {&table, &vocab32, &n_i, &ids_dev, &chunks32, &out, &c->fault_dev, &scale, &row0};
         return launch_keyed(c, OP_EMBED, (uint32_t)fmt << 8 | (uint32_t)out_dtype,
                             [&] { return std::string("apk_embed_") + kFmtName[fmt] + (out_dtype == APK_F32 ? "_f32" : "_f16"); },
                             (unsigned)grid, (unsigned)threads, 0, args);
@@ -833,7 +834,7 @@ static int embed_common(apk_ctx* c, int fmt, const void* table, size_t vocab, si
         const uint64_t grid = (uint64_t)t * chunks;
         if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_embed_rows: too large");
         uint32_t chunks32 = (uint32_t)chunks;
-        void* args[] = {&table, &vocab32, &n_i, &ids_dev, &chunks32, &out, &c->fault_dev, &scale};
+        void* args[] = {&table, &vocab32, &n_i, &ids_dev, &chunks32, &out, &c->fault_dev, &scale, &row0};
         return launch_keyed(c, OP_EMBED, (uint32_t)fmt << 8 | (uint32_t)out_dtype,
                             [&] { return std::string("apk_embed_") + kFmtName[fmt] + (out_dtype == APK_F32 ? "_f32" : "_f16"); },
                             (unsigned)grid, (unsigned)threads, 0, args);
@@ -844,7 +845,7 @@ static int embed_common(apk_ctx* c, int fmt, const void* table, size_t vocab, si
     size_t threads = (n_in / (16 / elem_size(out_dtype)) + 63) / 64 * 64;  // one output tile per lane
     if (threads > 256) threads = 256;
     uint64_t table_bytes = (uint64_t)vocab * row_bytes;
-    void* args[] = {&table, &table_bytes, &vocab32, &n_i, &ids_dev, &out, &c->fault_dev, &scale};
+    void* args[] = {&table, &table_bytes, &vocab32, &n_i, &ids_dev, &out, &c->fault_dev, &scale, &row0};
     return launch_keyed(c, OP_EMBED, (uint32_t)fmt << 8 | (uint32_t)out_dtype,
                         [&] { return std::string("apk_embed_") + kFmtName[fmt] + (out_dtype == APK_F32 ? "_f32" : "_f16"); }, (unsigned)t,
                         (unsigned)threads, (unsigned)shmem, args);
@@ -862,6 +863,15 @@ int apk_embed_rows_scaled(apk_ctx* c, int fmt, const void* table, size_t vocab, 
     if (!c) return fail(APK_DECLINE_NULL, "apk_embed_rows_scaled: ctx is NULL");
     CallScope s(c);
     return embed_common(c, fmt, table, vocab, n_in, ids, t, out, out_dtype, scale);
+}
+
+int apk_dequant_rows(apk_ctx* c, int fmt, const void* table, size_t n_rows, size_t n_in, size_t row0, size_t count,
+                     void* out, int out_dtype) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_dequant_rows: ctx is NULL");
+    CallScope s(c);
+    if (row0 > n_rows || count > n_rows - row0)
+        return fail(APK_DECLINE_RANGE, "apk_dequant_rows: rows [%zu, +%zu) of %zu", row0, count, n_rows);
+    return embed_common(c, fmt, table, n_rows, n_in, nullptr, count, out, out_dtype, 1.0f, false, (uint32_t)row0);
 }
 
 int apk_embed_rows_host_ids(apk_ctx* c, int fmt, const void* table, size_t vocab, size_t n_in,

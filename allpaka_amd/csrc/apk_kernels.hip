@@ -1050,10 +1050,10 @@ template <int N> DEV void embed_scale(float* v, float scale) {
 
 template <typename TO>
 DEV void embed_q4k_body(const uint8_t* table, uint32_t vocab, int n_in, const uint32_t* ids, TO* out, uint32_t* fault,
-                        float scale) {
+                        float scale, uint32_t row0) {
     const int nsb = n_in / 256;
     const uint64_t t = blockIdx.x;
-    const uint32_t id = ids[t];
+    const uint32_t id = ids ? ids[t] : row0 + (uint32_t)t;  // no id list: the rows row0, row0 + 1, ...
     if (id >= vocab) {
         if (threadIdx.x == 0) atomicOr(fault, APK_FAULT_TOKEN_RANGE);
         return;
@@ -1111,13 +1111,13 @@ DEV void embed_q4k_body(const uint8_t* table, uint32_t vocab, int n_in, const ui
 }
 extern "C" __global__ __launch_bounds__(256) void apk_embed_q4k_f32(const uint8_t* table, uint32_t vocab, int n_in,
                                                                    const uint32_t* ids, float* out, uint32_t* fault,
-                                                                   float scale) {
-    embed_q4k_body<float>(table, vocab, n_in, ids, out, fault, scale);
+                                                                   float scale, uint32_t row0) {
+    embed_q4k_body<float>(table, vocab, n_in, ids, out, fault, scale, row0);
 }
 extern "C" __global__ __launch_bounds__(256) void apk_embed_q4k_f16(const uint8_t* table, uint32_t vocab, int n_in,
                                                                    const uint32_t* ids, f16_t* out, uint32_t* fault,
-                                                                   float scale) {
-    embed_q4k_body<f16_t>(table, vocab, n_in, ids, out, fault, scale);
+                                                                   float scale, uint32_t row0) {
+    embed_q4k_body<f16_t>(table, vocab, n_in, ids, out, fault, scale, row0);
 }
 
 // ---- formats decoded straight from global memory -------------------------------------
@@ -1253,11 +1253,11 @@ template <> struct dqd<8> {  // F32
 // number and the token id are uniform for the workgroup (scalar loads, no per-lane division).
 template <int FMT, typename TO>
 DEV void embed_direct_body(const uint8_t* table, uint32_t vocab, int n_in, const uint32_t* ids, uint32_t chunks, TO* out,
-                           uint32_t* fault, float scale) {
+                           uint32_t* fault, float scale, uint32_t row0) {
     constexpr int OPT = io<TO>::VEC;  // outputs per tile
     const uint32_t tiles_per_row = (uint32_t)n_in / OPT;
     const uint32_t t = blockIdx.x / chunks, chunk = blockIdx.x - t * chunks;
-    const uint32_t id = ids[t];
+    const uint32_t id = ids ? ids[t] : row0 + (uint32_t)t;  // no id list: the rows row0, row0 + 1, ...
     if (id >= vocab) {  // uniform
         if (threadIdx.x == 0 && chunk == 0) atomicOr(fault, APK_FAULT_TOKEN_RANGE);
         return;
@@ -1287,10 +1287,10 @@ DEV void embed_direct_body(const uint8_t* table, uint32_t vocab, int n_in, const
 // (the compiler merges the identical loads), and for every k the 8 lanes write one whole line.
 template <int FMT, typename TO>
 DEV void embed_direct_sb_body(const uint8_t* __restrict__ table, uint32_t vocab, int n_in, const uint32_t* __restrict__ ids,
-                              uint32_t chunks, TO* __restrict__ out, uint32_t* fault, float scale) {
+                              uint32_t chunks, TO* __restrict__ out, uint32_t* fault, float scale, uint32_t row0) {
     constexpr int OPT = io<TO>::VEC, K = 256 / OPT / 8;
     const uint32_t t = blockIdx.x / chunks, chunk = blockIdx.x - t * chunks;
-    const uint32_t id = ids[t];
+    const uint32_t id = ids ? ids[t] : row0 + (uint32_t)t;  // no id list: the rows row0, row0 + 1, ...
     if (id >= vocab) {  // uniform
         if (threadIdx.x == 0 && chunk == 0) atomicOr(fault, APK_FAULT_TOKEN_RANGE);
         return;
@@ -1314,26 +1314,26 @@ DEV void embed_direct_sb_body(const uint8_t* __restrict__ table, uint32_t vocab,
 #define APK_EMBED_DIRECT_SB(NAME, FMT)                                                                                   \
     extern "C" __global__ __launch_bounds__(256) void apk_embed_##NAME##_f32(                                            \
         const uint8_t* table, uint32_t vocab, int n_in, const uint32_t* ids, uint32_t chunks, float* out, uint32_t* fault, \
-        float scale) {                                                                                                   \
-        embed_direct_sb_body<FMT, float>(table, vocab, n_in, ids, chunks, out, fault, scale);                            \
+        float scale, uint32_t row0) {                                                                                    \
+        embed_direct_sb_body<FMT, float>(table, vocab, n_in, ids, chunks, out, fault, scale, row0);                      \
     }                                                                                                                    \
     extern "C" __global__ __launch_bounds__(256) void apk_embed_##NAME##_f16(                                            \
         const uint8_t* table, uint32_t vocab, int n_in, const uint32_t* ids, uint32_t chunks, f16_t* out, uint32_t* fault, \
-        float scale) {                                                                                                   \
-        embed_direct_sb_body<FMT, f16_t>(table, vocab, n_in, ids, chunks, out, fault, scale);                            \
+        float scale, uint32_t row0) {                                                                                    \
+        embed_direct_sb_body<FMT, f16_t>(table, vocab, n_in, ids, chunks, out, fault, scale, row0);                      \
     }
 APK_EMBED_DIRECT_SB(q6k, 2) APK_EMBED_DIRECT_SB(q5k, 1) APK_EMBED_DIRECT_SB(q2k, 4) APK_EMBED_DIRECT_SB(q3k, 5)
 
 #define APK_EMBED_DIRECT(NAME, FMT)                                                                                      \
     extern "C" __global__ __launch_bounds__(256) void apk_embed_##NAME##_f32(                                            \
         const uint8_t* table, uint32_t vocab, int n_in, const uint32_t* ids, uint32_t chunks, float* out, uint32_t* fault, \
-        float scale) {                                                                                                   \
-        embed_direct_body<FMT, float>(table, vocab, n_in, ids, chunks, out, fault, scale);                               \
+        float scale, uint32_t row0) {                                                                                    \
+        embed_direct_body<FMT, float>(table, vocab, n_in, ids, chunks, out, fault, scale, row0);                         \
     }                                                                                                                    \
     extern "C" __global__ __launch_bounds__(256) void apk_embed_##NAME##_f16(                                            \
         const uint8_t* table, uint32_t vocab, int n_in, const uint32_t* ids, uint32_t chunks, f16_t* out, uint32_t* fault, \
-        float scale) {                                                                                                   \
-        embed_direct_body<FMT, f16_t>(table, vocab, n_in, ids, chunks, out, fault, scale);                               \
+        float scale, uint32_t row0) {                                                                                    \
+        embed_direct_body<FMT, f16_t>(table, vocab, n_in, ids, chunks, out, fault, scale, row0);                         \
     }
 APK_EMBED_DIRECT(q8_0, 3) APK_EMBED_DIRECT(q5_0, 6) APK_EMBED_DIRECT(f32, 8)
 
@@ -1358,11 +1358,11 @@ template <> struct dq<9> {  // BF16, allpaka-dtype lib.rs:188-190
 // writing consecutive tiles.
 template <int FMT, typename TO>
 DEV void embed_staged_body(const uint8_t* table, uint64_t table_bytes, uint32_t vocab, int n_in, const uint32_t* ids,
-                           TO* out, uint32_t* fault, float scale) {
+                           TO* out, uint32_t* fault, float scale, uint32_t row0) {
     extern __shared__ __attribute__((aligned(16))) uint8_t stage[];
     constexpr int OPT = io<TO>::VEC, BE = dq<FMT>::BE, BB = dq<FMT>::BB;
     const uint64_t t = blockIdx.x;
-    const uint32_t id = ids[t];
+    const uint32_t id = ids ? ids[t] : row0 + (uint32_t)t;  // no id list: the rows row0, row0 + 1, ...
     if (id >= vocab) {
         if (threadIdx.x == 0) atomicOr(fault, APK_FAULT_TOKEN_RANGE);
         return;
@@ -1399,16 +1399,16 @@ DEV void embed_staged_body(const uint8_t* table, uint64_t table_bytes, uint32_t 
         io<TO>::store_nt(out + t * (uint64_t)n_in + e0, o);
     }
 }
-#define APK_EMBED_GEN(NAME, FMT)                                                                                          \
-    extern "C" __global__ __launch_bounds__(256) void apk_embed_##NAME##_f32(                                             \
-        const uint8_t* table, uint64_t table_bytes, uint32_t vocab, int n_in, const uint32_t* ids, float* out,            \
-        uint32_t* fault, float scale) {                                                                                   \
-        embed_staged_body<FMT, float>(table, table_bytes, vocab, n_in, ids, out, fault, scale);                           \
-    }                                                                                                                     \
-    extern "C" __global__ __launch_bounds__(256) void apk_embed_##NAME##_f16(                                             \
-        const uint8_t* table, uint64_t table_bytes, uint32_t vocab, int n_in, const uint32_t* ids, f16_t* out,            \
-        uint32_t* fault, float scale) {                                                                                   \
-        embed_staged_body<FMT, f16_t>(table, table_bytes, vocab, n_in, ids, out, fault, scale);                           \
+#define APK_EMBED_GEN(NAME, FMT)                                                                                         \
+    extern "C" __global__ __launch_bounds__(256) void apk_embed_##NAME##_f32(                                            \
+        const uint8_t* table, uint64_t table_bytes, uint32_t vocab, int n_in, const uint32_t* ids, float* out,           \
+        uint32_t* fault, float scale, uint32_t row0) {                                                                   \
+        embed_staged_body<FMT, float>(table, table_bytes, vocab, n_in, ids, out, fault, scale, row0);                    \
+    }                                                                                                                    \
+    extern "C" __global__ __launch_bounds__(256) void apk_embed_##NAME##_f16(                                            \
+        const uint8_t* table, uint64_t table_bytes, uint32_t vocab, int n_in, const uint32_t* ids, f16_t* out,           \
+        uint32_t* fault, float scale, uint32_t row0) {                                                                   \
+        embed_staged_body<FMT, f16_t>(table, table_bytes, vocab, n_in, ids, out, fault, scale, row0);                    \
     }
 APK_EMBED_GEN(f16, 7) APK_EMBED_GEN(bf16, 9)  // (measured faster staged than decoded in place)
 

@@ -40,6 +40,7 @@ SYMBOLS = {
     "apk_graph_destroy": (_i, [_vp, _vp]),
     "apk_embed_rows": (_i, [_vp, _i, _vp, _sz, _sz, _vp, _sz, _vp, _i]),
     "apk_embed_rows_scaled": (_i, [_vp, _i, _vp, _sz, _sz, _vp, _sz, _f, _vp, _i]),
+    "apk_dequant_rows": (_i, [_vp, _i, _vp, _sz, _sz, _sz, _sz, _vp, _i]),
     "apk_embed_rows_host_ids": (_i, [_vp, _i, _vp, _sz, _sz, _vp, _sz, _vp, _i]),
     "apk_add_assign": (_i, [_vp, _vp, _vp, _sz, _i]),
     "apk_softmax_rows": (_i, [_vp, _vp, _sz, _sz]),

@@ -335,6 +335,14 @@ def other_shapes(args, L, h, apklib, synth, torch, gen, dev, randn, pool, p, tim
         torch.cuda.synchronize()
         us = timed(lambda i: check(L.apk_embed_rows(h, fmt, p(tb), vocab, H, p(ids[i % 8]), T, p(outs[i % len(outs)]), F16)), reps)
         record(f"embed_rows {name}->f16", f"qwen3-32b T={T}", us, T * (rbx + 4 + H * 2))
+        if name == "Q6_K":
+            # a range of rows with no id list: a [8192 x 5120] slice of the same bytes widened to fp16, the step the
+            # reference runs ahead of a dense GEMM on a quantized weight (the table rotates through 8192-row windows)
+            wrows = 8192
+            wouts = pool(wrows * H * 2, lambda: torch.empty((wrows, H), dtype=torch.float16, device=dev))
+            us = timed(lambda i: check(L.apk_dequant_rows(h, fmt, p(tb), vocab, H, (i % 16) * wrows, wrows, p(wouts[i % len(wouts)]), F16)), reps)
+            record("dequant_rows Q6_K->f16 (row range, no id list)", f"[{wrows} x {H}] weight", us, wrows * (rbx + H * 2))
+            del wouts
         del tb
     del outs
 

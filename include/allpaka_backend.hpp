@@ -217,6 +217,15 @@ class QuantMat {
         check(apk_embed_rows_host_ids(Gpu::get().ctx(), ty_, dev_->ptr(), n_out_, n_in_, &id, 1, dout.ptr(), APK_F32));
         dout.read_back(dst.data());
     }
+    // rows [row0, row0 + count) as f32, one launch, no id list (the same rows as row_into in a loop)
+    std::vector<float> dequant_rows(size_t row0, size_t count) const {
+        std::vector<float> out(count * n_in_);
+        if (count == 0) return out;
+        Dev<float> dout(out.size());
+        check(apk_dequant_rows(Gpu::get().ctx(), ty_, dev_->ptr(), n_out_, n_in_, row0, count, dout.ptr(), APK_F32));
+        dout.read_back(out.data());
+        return out;
+    }
 
   private:
     int ty_;

@@ -166,6 +166,14 @@ int apk_embed_rows_scaled(apk_ctx* ctx, int fmt, const void* table, size_t vocab
  * (APK_DECLINE_RANGE), as the reference's callers reject token >= vocab first. */
 int apk_embed_rows_host_ids(apk_ctx* ctx, int fmt, const void* table, size_t vocab, size_t n_in,
                             const uint32_t* ids_host, size_t t, void* out, int out_dtype);
+/* The rows [row0, row0 + count) of a quantized matrix of n_rows rows, dequantized in place of a
+ * gather: out[i, :] = dequant(row row0 + i), no id list.  Replaces QuantMat::row_into over a
+ * range (quantmat/mod.rs:75-89, dequant.rs:26-92) and the reference's dequant_rows_f16 kernel,
+ * which widens a weight matrix to fp16 ahead of a dense GEMM (gpu/cuda/kernels.rs:2795-2870,
+ * launched from gpu/cuda/runtime/gemm.rs:213-260).  Same formats, alignment and bit-exact results
+ * as apk_embed_rows; a range outside the matrix is declined (APK_DECLINE_RANGE). */
+int apk_dequant_rows(apk_ctx* ctx, int fmt, const void* table, size_t n_rows, size_t n_in, size_t row0, size_t count,
+                     void* out, int out_dtype);
 
 /* Residual add on its own: a[i] += b[i].  Replaces ops::add_assign_slice / add_assign_par
  * (ops/blas.rs:105-213) where no norm follows (where one does, apk_add_rmsnorm_rows does

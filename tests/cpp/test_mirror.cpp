@@ -158,6 +158,13 @@ static void q8_0_is_scale_times_value() {  // crates/allpaka-gguf/src/dequant.rs
     CHECK(throws<Error>([&] { m.row(1); }));
     CHECK(throws<Error>([&] { QuantMat bad(block, GgmlType::Q8_0, 1, 48); }));
     CHECK(throws<Error>([&] { std::vector<float> d(32); m.row_into(0, d); }));
+    // the same bytes as two rows of 32: a range of rows in one launch equals the rows one by one
+    QuantMat m2(block, GgmlType::Q8_0, 2, 32);
+    auto both = m2.dequant_rows(0, 2);
+    CHECK(both.size() == 64 && both == out);
+    auto second = m2.dequant_rows(1, 1);
+    CHECK(second.size() == 32 && second == m2.row(1));
+    CHECK(throws<Declined>([&] { m2.dequant_rows(1, 2); }));
 }
 static void route_picks_the_top_k_and_renormalises() {  // crates/allpaka-model/tests/gpu_eligible_forward.rs:88-97
     std::vector<float> logp = {std::log(0.1f), std::log(0.5f), std::log(0.15f), std::log(0.25f)};

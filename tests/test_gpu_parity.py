@@ -126,6 +126,13 @@ def test_embed_all_ten_formats_bit_exact(be, ora, fmt_name, out_f16):
     got = host(out)
     assert np.array_equal(got.view(np.uint16 if out_f16 else np.uint32), want.view(np.uint16 if out_f16 else np.uint32))
     assert np.array_equal(host(qm.row(3, dtype=out.dtype)), want[0])  # token 3 of 6, as the reference's test
+    # a range of rows without an id list (the dequant of a weight matrix ahead of a dense GEMM): the same rows
+    want_r = ora.embed_rows(raw, fmt, vocab, hidden, np.arange(1, 6, dtype=np.uint32), out_f16=out_f16)
+    got_r = host(qm.dequant_rows(1, 5, dtype=out.dtype))
+    assert np.array_equal(got_r.view(np.uint16 if out_f16 else np.uint32), want_r.view(np.uint16 if out_f16 else np.uint32))
+    assert qm.dequant_rows(6, 0, dtype=out.dtype).shape == (0, hidden)
+    with pytest.raises(apk.Declined):
+        qm.dequant_rows(2, 5)  # rows 2..6 of 6
     # models that scale their token embeddings: one f32 multiply after the dequant (prefill.rs:107-109;
     # Gemma's factor is sqrt(hidden), here of a 3584-wide model)
     scale = float(np.sqrt(np.float32(3584.0)))
