@@ -251,4 +251,153 @@ inline std::vector<std::pair<size_t, float>> route_gated(const std::vector<float
     return out;
 }
 
+// The batched router of Ffn::moe_batch (moe.rs:204-227): route_gated_into_slice for every row of
+// logits [rows][n_expert]; ids and w are [rows][k], best first.
+struct Routed {
+    size_t rows = 0, k = 0;
+    std::vector<uint32_t> ids;
+    std::vector<float> w;
+};
+inline Routed route_rows(const std::vector<float>& logits, size_t n_expert, size_t k, Gating gating, bool norm, float scale,
+                         const std::vector<float>* bias) {
+    if (n_expert == 0 || logits.size() % n_expert) throw Panic("logits is not rows x n_expert");
+    if (bias && bias->size() != n_expert) throw Panic("bias length is not n_expert");
+    Routed r;
+    r.rows = logits.size() / n_expert;
+    r.k = k < n_expert ? k : n_expert;
+    r.ids.resize(r.rows * r.k);
+    r.w.resize(r.rows * r.k);
+    if (r.rows == 0 || r.k == 0) return r;
+    Dev<float> dl(logits.data(), logits.size()), dw(r.w.size()), db(bias ? bias->data() : nullptr, n_expert);
+    Dev<uint32_t> di(r.ids.size());
+    check(apk_route_topk(Gpu::get().ctx(), dl.ptr(), bias ? db.ptr() : nullptr, r.rows, n_expert, r.k, norm ? 1 : 0, scale,
+                         gating == Gating::Sigmoid ? 1 : 0, di.ptr(), dw.ptr()));
+    di.read_back(r.ids.data());
+    dw.read_back(r.w.data());
+    return r;
+}
+
+// groups / used / table / tok of Ffn::moe_batch and the per-token hit lists of its combine
+// (moe.rs:229-271, :298-309), i.e. GroupedFfnReq.{groups, tok, total_rows} and
+// GroupedCombine.{tok_off, hit_row, hit_w} (gpu/types.rs:429-467).
+struct Grouped {
+    std::vector<std::array<uint32_t, 3>> groups;  // [expert, row0, rows] of the experts that were hit, ascending
+    std::vector<uint32_t> tok;                    // source token of each flat row
+    std::vector<uint32_t> tok_off, hit_row;       // CSR: token t's hits are [tok_off[t], tok_off[t+1])
+    std::vector<float> hit_w;
+    size_t total_rows = 0;
+};
+inline Grouped moe_group(const Routed& r, size_t n_expert) {
+    Grouped g;
+    const size_t total = r.rows * r.k;
+    g.total_rows = total;
+    g.tok_off.assign(r.rows + 1, 0);
+    if (total == 0) return g;
+    Dev<uint32_t> di(r.ids.data(), total), dtable(n_expert * 3), dn(1), dtok(total), doff(r.rows + 1), dhit(total);
+    Dev<float> dw(r.w.data(), total), dhw(total);
+    check(apk_moe_permute(Gpu::get().ctx(), di.ptr(), dw.ptr(), r.rows, r.k, n_expert, dtable.ptr(), dn.ptr(), dtok.ptr(),
+                          doff.ptr(), dhit.ptr(), dhw.ptr()));
+    uint32_t faults = 0;
+    check(apk_take_faults(Gpu::get().ctx(), &faults));
+    if (faults) throw Panic("expert id out of range");  // groups[e] would index out of bounds
+    uint32_t n_used = 0;
+    dn.read_back(&n_used);
+    std::vector<uint32_t> table(n_expert * 3);
+    dtable.read_back(table.data());
+    for (uint32_t i = 0; i < n_used; i++) g.groups.push_back({table[3 * i], table[3 * i + 1], table[3 * i + 2]});
+    g.tok.resize(total);
+    g.hit_row.resize(total);
+    g.hit_w.resize(total);
+    dtok.read_back(g.tok.data());
+    doff.read_back(g.tok_off.data());
+    dhit.read_back(g.hit_row.data());
+    dhw.read_back(g.hit_w.data());
+    return g;
+}
+
+// The gathered expert activations xe[r] = x[tok[r]] (moe.rs:348-352), produced from the token side.
+inline std::vector<float> gather_rows(const std::vector<float>& x, size_t hidden, const Grouped& g, size_t k) {
+    if (hidden == 0 || x.size() % hidden) throw Panic("x is not rows x hidden");
+    const size_t rows = x.size() / hidden;
+    if (rows * k != g.total_rows) throw Panic("grouping does not belong to these rows");
+    std::vector<float> xe(g.total_rows * hidden);
+    if (xe.empty()) return xe;
+    Dev<float> dx(x.data(), x.size()), dxe(xe.size());
+    Dev<uint32_t> dhit(g.hit_row.data(), g.hit_row.size());
+    check(apk_scatter_rows(Gpu::get().ctx(), dx.ptr(), dhit.ptr(), rows, k, g.total_rows, hidden, dxe.ptr(), APK_F32));
+    dxe.read_back(xe.data());
+    return xe;
+}
+
+// The combine of Ffn::moe_batch (moe.rs:298-333: per token, add_scaled_slice over its hits in order),
+// the residual add (decode.rs:775) and, when next_norm is given, the next layer's rmsnorm_rows_into
+// (prefill.rs:308-314) in one pass: x += sum; h = rmsnorm(x) * next_norm.
+inline void moe_combine_add_rmsnorm(std::vector<float>& x, const std::vector<float>& flat, size_t hidden, const Grouped& g,
+                                    std::vector<float>* h, const std::vector<float>* next_norm, float eps) {
+    if (hidden == 0 || x.size() % hidden || flat.size() != g.total_rows * hidden) throw Panic("shape mismatch");
+    const size_t rows = x.size() / hidden;
+    if (g.tok_off.size() != rows + 1) throw Panic("grouping does not belong to these rows");
+    if (h && (!next_norm || next_norm->size() != hidden || h->size() < x.size())) throw Panic("next norm shape mismatch");
+    if (rows == 0) return;
+    Dev<float> dx(x.data(), x.size()), dflat(flat.data(), flat.size()), dhw(g.hit_w.data(), g.hit_w.size()), dh(h ? x.size() : 1),
+        dgamma(h ? next_norm->data() : nullptr, h ? hidden : 1);
+    Dev<uint32_t> doff(g.tok_off.data(), g.tok_off.size()), dhit(g.hit_row.data(), g.hit_row.size());
+    check(apk_moe_combine_add_rmsnorm(Gpu::get().ctx(), dx.ptr(), dflat.ptr(), doff.ptr(), dhit.ptr(), dhw.ptr(), g.total_rows,
+                                      h ? dh.ptr() : nullptr, h ? dgamma.ptr() : nullptr, hidden, rows, eps, APK_F32));
+    dx.read_back(x.data());
+    if (h) dh.read_back(h->data());
+}
+
+// The greedy pick of forward_greedy (decode.rs:628-630): max_by(total_cmp), i.e. the LAST maximum.
+inline uint32_t argmax(const std::vector<float>& logits) {
+    if (logits.empty()) return 0;  // unwrap_or(0)
+    Dev<float> dl(logits.data(), logits.size());
+    Dev<uint32_t> dout(1);
+    check(apk_argmax_rows(Gpu::get().ctx(), dl.ptr(), 1, logits.size(), dout.ptr()));
+    uint32_t out = 0;
+    dout.read_back(&out);
+    return out;
+}
+
+// One layer's K and V planes of the cache, [capacity][kv_dim] f16 each (kv.rs:682-697), on the device.
+class KvLayer {
+  public:
+    KvLayer(size_t capacity, size_t kv_dim) : capacity_(capacity), kv_dim_(kv_dim), k_(capacity * kv_dim), v_(capacity * kv_dim) {}
+    // The attention prologue of a chunk (attention.rs:131-200): per-head rmsnorm + NeoX rotation of q and k
+    // in place, then KvCache::store_at(layer, pos[r], k_row, v_row) for every row -- one launch.
+    void qknorm_rope_store(std::vector<float>& q, std::vector<float>& k, const std::vector<float>& v, const std::vector<float>* q_norm,
+                           const std::vector<float>* k_norm, const std::vector<std::array<float, 2>>& rope,
+                           const std::vector<uint32_t>& pos, size_t n_q, size_t n_kv, size_t head_dim, float eps) {
+        const size_t rows = pos.size();
+        if (n_kv * head_dim != kv_dim_ || k.size() != rows * kv_dim_ || v.size() != k.size() || q.size() != rows * n_q * head_dim)
+            throw Panic("k / v rows are not kv_dim wide");  // assert_eq!(k.len(), self.kv_dim)
+        if (rope.size() != rows * head_dim / 2) throw Panic("rope table does not cover the rows");
+        for (uint32_t p : pos)
+            if (p >= capacity_) throw Panic("position " + std::to_string(p) + " past capacity " + std::to_string(capacity_));
+        if (rows == 0) return;
+        Dev<float> dq(q.data(), q.size()), dk(k.data(), k.size()), dv(v.data(), v.size()), drope(&rope[0][0], rope.size() * 2),
+            dqw(q_norm ? q_norm->data() : nullptr, head_dim), dkw(k_norm ? k_norm->data() : nullptr, head_dim);
+        Dev<uint32_t> dpos(pos.data(), rows);
+        check(apk_qknorm_rope_kv_store(Gpu::get().ctx(), dq.ptr(), dk.ptr(), dv.ptr(), q_norm ? dqw.ptr() : nullptr,
+                                       k_norm ? dkw.ptr() : nullptr, drope.ptr(), dpos.ptr(), k_.ptr(), v_.ptr(), capacity_, rows, n_q,
+                                       n_kv, head_dim, head_dim, eps, APK_F32));
+        dq.read_back(q.data());
+        dk.read_back(k.data());
+    }
+    // the stored f16 bits of one position
+    std::vector<uint16_t> k_row(size_t pos) const { return row(k_, pos); }
+    std::vector<uint16_t> v_row(size_t pos) const { return row(v_, pos); }
+
+  private:
+    std::vector<uint16_t> row(const Dev<uint16_t>& plane, size_t pos) const {
+        if (pos >= capacity_) throw Panic("position past capacity");
+        std::vector<uint16_t> out(kv_dim_);
+        check(apk_d2h(Gpu::get().ctx(), out.data(), plane.ptr() + pos * kv_dim_, kv_dim_ * 2));
+        check(apk_sync(Gpu::get().ctx()));
+        return out;
+    }
+    size_t capacity_, kv_dim_;
+    Dev<uint16_t> k_, v_;
+};
+
 }  // namespace allpaka_backend

@@ -3,6 +3,7 @@
 // Each test names the reference test it follows (crates/allpaka-backend/src/ops/mod.rs unless noted).
 #include <cmath>
 #include <cstdio>
+#include <cstring>
 #include <functional>
 
 #include "allpaka_backend.hpp"
@@ -181,6 +182,152 @@ static void route_picks_the_top_k_and_renormalises() {  // crates/allpaka-model/
     CHECK(route_gated({1.0f, 2.0f}, 0, Gating::Softmax, true, 1.0f, nullptr).empty());
 }
 
+// ---- the MoE grouping, combine, greedy pick and cache store, against the reference's CPU algorithm restated here
+static Routed picks(size_t rows, size_t k, std::vector<uint32_t> ids, std::vector<float> w) {
+    Routed r;
+    r.rows = rows; r.k = k; r.ids = std::move(ids); r.w = std::move(w);
+    return r;
+}
+static Grouped group_on_the_cpu(const Routed& r, size_t n_expert) {  // moe.rs:229-271 then :298-309, line by line
+    std::vector<std::vector<std::pair<size_t, float>>> groups(n_expert);
+    for (size_t i = 0; i < r.rows; i++)
+        for (size_t j = 0; j < r.k; j++) groups[r.ids[i * r.k + j]].push_back({i, r.w[i * r.k + j]});
+    Grouped g;
+    uint32_t row0 = 0;
+    std::vector<size_t> used;
+    for (size_t e = 0; e < n_expert; e++)
+        if (!groups[e].empty()) used.push_back(e);
+    for (size_t e : used) {
+        g.groups.push_back({(uint32_t)e, row0, (uint32_t)groups[e].size()});
+        for (auto& p : groups[e]) g.tok.push_back((uint32_t)p.first);
+        row0 += (uint32_t)groups[e].size();
+    }
+    g.total_rows = row0;
+    std::vector<size_t> counts(r.rows, 0);
+    g.hit_row.assign(r.rows * r.k, 0);
+    g.hit_w.assign(r.rows * r.k, 0.0f);
+    for (size_t gi = 0; gi < used.size(); gi++)
+        for (size_t idx = 0; idx < groups[used[gi]].size(); idx++) {
+            const size_t i = groups[used[gi]][idx].first;
+            g.hit_row[i * r.k + counts[i]] = g.groups[gi][1] + (uint32_t)idx;
+            g.hit_w[i * r.k + counts[i]] = groups[used[gi]][idx].second;
+            counts[i]++;
+        }
+    g.tok_off.assign(r.rows + 1, 0);
+    for (size_t i = 0; i < r.rows; i++) g.tok_off[i + 1] = g.tok_off[i] + (uint32_t)counts[i];
+    return g;
+}
+static bool same_grouping(const Grouped& a, const Grouped& b) {
+    return a.groups == b.groups && a.tok == b.tok && a.tok_off == b.tok_off && a.hit_row == b.hit_row && a.hit_w == b.hit_w &&
+           a.total_rows == b.total_rows;
+}
+static void moe_group_orders_rows_by_expert_then_token() {  // moe.rs:229-271
+    // 4 tokens, 2 picks each, 4 experts; expert 1 is never picked and gets no group
+    Routed r = picks(4, 2, {2, 0, 0, 3, 2, 3, 0, 2}, {0.6f, 0.4f, 0.7f, 0.3f, 0.5f, 0.5f, 0.9f, 0.1f});
+    Grouped g = moe_group(r, 4);
+    CHECK((g.groups == std::vector<std::array<uint32_t, 3>>{{0, 0, 3}, {2, 3, 3}, {3, 6, 2}}));
+    CHECK((g.tok == std::vector<uint32_t>{0, 1, 3, 0, 2, 3, 1, 2}));
+    CHECK((g.tok_off == std::vector<uint32_t>{0, 2, 4, 6, 8}));
+    CHECK((g.hit_row == std::vector<uint32_t>{0, 3, 1, 6, 4, 7, 2, 5}));
+    CHECK((g.hit_w == std::vector<float>{0.4f, 0.6f, 0.7f, 0.3f, 0.5f, 0.5f, 0.9f, 0.1f}));
+    CHECK(g.total_rows == 8);
+    CHECK(same_grouping(g, group_on_the_cpu(r, 4)));
+    // a larger batch with an uneven spread, picks straight from the device router
+    const size_t rows = 300, n_expert = 24, k = 5;
+    std::vector<float> logits(rows * n_expert);
+    for (size_t i = 0; i < logits.size(); i++) logits[i] = std::sin(0.37f * (float)i) * 3.0f + ((i % n_expert) == 7 ? -40.0f : 0.0f);
+    Routed rr = route_rows(logits, n_expert, k, Gating::Softmax, true, 1.0f, nullptr);
+    CHECK(rr.rows == rows && rr.k == k);
+    Grouped gg = moe_group(rr, n_expert);
+    CHECK(same_grouping(gg, group_on_the_cpu(rr, n_expert)));
+    for (auto& grp : gg.groups) CHECK(grp[0] != 7);  // nobody picks expert 7
+    CHECK(throws<Panic>([] { moe_group(picks(1, 1, {9}, {1.0f}), 4); }));  // groups[9] of 4
+    CHECK(moe_group(picks(0, 2, {}, {}), 4).total_rows == 0);
+}
+static void gather_then_combine_is_the_weighted_sum_of_the_hits() {  // moe.rs:298-333, :348-352
+    const size_t rows = 50, n_expert = 8, k = 3, hidden = 256;
+    std::vector<float> logits(rows * n_expert), x(rows * hidden), gamma(hidden);
+    for (size_t i = 0; i < logits.size(); i++) logits[i] = std::cos(0.91f * (float)i);
+    for (size_t i = 0; i < x.size(); i++) x[i] = std::sin(0.013f * (float)i) - 0.2f;
+    for (size_t i = 0; i < hidden; i++) gamma[i] = 1.0f + 0.002f * (float)i;
+    Routed r = route_rows(logits, n_expert, k, Gating::Softmax, true, 1.0f, nullptr);
+    Grouped g = moe_group(r, n_expert);
+    std::vector<float> xe = gather_rows(x, hidden, g, k);
+    CHECK(xe.size() == g.total_rows * hidden);
+    for (size_t row = 0; row < g.total_rows; row++)
+        for (size_t i = 0; i < hidden; i += 17) CHECK(xe[row * hidden + i] == x[g.tok[row] * hidden + i]);
+    // stand-in for the experts' down rows: twice the gathered row
+    std::vector<float> flat(xe);
+    for (float& v : flat) v *= 2.0f;
+    std::vector<float> want(x), h(x.size(), 0.0f), got(x);
+    for (size_t t = 0; t < rows; t++)
+        for (size_t i = 0; i < hidden; i++) {
+            float out = 0.0f;
+            for (uint32_t j = g.tok_off[t]; j < g.tok_off[t + 1]; j++) out = std::fmaf(flat[g.hit_row[j] * hidden + i], g.hit_w[j], out);
+            want[t * hidden + i] += out;
+        }
+    moe_combine_add_rmsnorm(got, flat, hidden, g, &h, &gamma, 1e-6f);
+    for (size_t i = 0; i < got.size(); i++) CHECK(got[i] == want[i]);  // the same fused multiply-adds in the same order
+    for (size_t t = 0; t < rows; t += 7) {
+        double ss = 0.0;
+        for (size_t i = 0; i < hidden; i++) ss += (double)want[t * hidden + i] * want[t * hidden + i];
+        const double scale = 1.0 / std::sqrt(ss / hidden + 1e-6);
+        for (size_t i = 0; i < hidden; i++) CHECK(close(h[t * hidden + i], (float)(want[t * hidden + i] * scale) * gamma[i]));
+    }
+    std::vector<float> plain(x);
+    moe_combine_add_rmsnorm(plain, flat, hidden, g, nullptr, nullptr, 0.0f);  // the last layer: no next norm
+    CHECK(plain == want);
+    CHECK(throws<Panic>([&] { std::vector<float> shorter(flat.begin(), flat.end() - 1), xx(x); moe_combine_add_rmsnorm(xx, shorter, hidden, g, nullptr, nullptr, 0.0f); }));
+}
+static void argmax_is_the_last_maximum() {  // decode.rs:628-630: max_by(total_cmp)
+    CHECK(argmax({0.5f, 3.0f, -1.0f, 2.0f}) == 1);
+    CHECK(argmax({1.0f, 7.0f, 7.0f, 0.0f, 7.0f, 6.0f}) == 4);   // max_by keeps the last of equal maxima
+    CHECK(argmax({0.0f, -0.0f}) == 0 && argmax({-0.0f, 0.0f}) == 1);  // total_cmp: -0.0 < +0.0
+    CHECK(argmax({}) == 0);
+    std::vector<float> wide(151936);
+    for (size_t i = 0; i < wide.size(); i++) wide[i] = std::sin(0.001f * (float)i);
+    size_t best = 0;
+    for (size_t i = 0; i < wide.size(); i++)
+        if (wide[i] >= wide[best]) best = i;
+    CHECK(argmax(wide) == best);
+}
+static uint16_t half_bits(float f) {  // f16::from_f32, round to nearest even (values here are normal halves or zero)
+    uint32_t u;
+    std::memcpy(&u, &f, 4);
+    const uint32_t sign = (u >> 16) & 0x8000u;
+    const int32_t exp = (int32_t)((u >> 23) & 0xff) - 127 + 15;
+    uint32_t man = u & 0x7fffffu;
+    if (exp <= 0) return (uint16_t)sign;  // flushed in this helper: the test keeps values well above 6e-5
+    uint32_t h = ((uint32_t)exp << 10) | (man >> 13);
+    const uint32_t rem = man & 0x1fffu;
+    if (rem > 0x1000u || (rem == 0x1000u && (h & 1u))) h++;
+    return (uint16_t)(sign | h);
+}
+static void chunk_prologue_stores_the_rotated_k_and_v_rows() {  // attention.rs:131-200, kv.rs:682-697
+    const size_t rows = 5, n_q = 4, n_kv = 2, hd = 128, capacity = 16;
+    std::vector<float> q(rows * n_q * hd), k(rows * n_kv * hd), v(k.size()), qw(hd), kw(hd), inv(hd / 2);
+    for (size_t i = 0; i < q.size(); i++) q[i] = 0.5f + std::sin(0.05f * (float)i);
+    for (size_t i = 0; i < k.size(); i++) { k[i] = 0.5f + std::cos(0.03f * (float)i); v[i] = 1.0f + 0.25f * std::sin(0.11f * (float)i); }
+    for (size_t i = 0; i < hd; i++) { qw[i] = 1.0f + 0.001f * (float)i; kw[i] = 1.0f - 0.001f * (float)i; }
+    for (size_t i = 0; i < hd / 2; i++) inv[i] = std::pow(1e6f, -2.0f * (float)i / (float)hd);
+    std::vector<uint32_t> pos = {3, 4, 5, 6, 9};
+    auto rope = ops::rope_sin_cos_rows(pos, inv);
+    std::vector<float> q2(q), k2(k);
+    ops::qknorm_rope_rows(q2, k2, &qw, &kw, rope, rows, n_q, n_kv, hd, 1e-6f);
+    KvLayer cache(capacity, n_kv * hd);
+    cache.qknorm_rope_store(q, k, v, &qw, &kw, rope, pos, n_q, n_kv, hd, 1e-6f);
+    CHECK(q == q2 && k == k2);  // the same arithmetic as the op without the store
+    for (size_t r = 0; r < rows; r++) {
+        auto kr = cache.k_row(pos[r]), vr = cache.v_row(pos[r]);
+        for (size_t i = 0; i < n_kv * hd; i++) {
+            CHECK(kr[i] == half_bits(k[r * n_kv * hd + i]));
+            CHECK(vr[i] == half_bits(v[r * n_kv * hd + i]));
+        }
+    }
+    CHECK(throws<Panic>([&] { std::vector<uint32_t> far = {1, 2, 3, 4, 16}; cache.qknorm_rope_store(q, k, v, &qw, &kw, rope, far, n_q, n_kv, hd, 1e-6f); }));
+    CHECK(throws<Panic>([&] { std::vector<float> shortv(v.begin(), v.end() - 1); cache.qknorm_rope_store(q, k, shortv, &qw, &kw, rope, pos, n_q, n_kv, hd, 1e-6f); }));
+}
+
 int main() {
     struct { const char* name; void (*fn)(); } tests[] = {
         {"rmsnorm_normalises_to_unit_rms_before_the_weight", rmsnorm_normalises_to_unit_rms_before_the_weight},
@@ -197,6 +344,10 @@ int main() {
         {"device_rope_rows_match_the_host_table", device_rope_rows_match_the_host_table},
         {"q8_0_is_scale_times_value", q8_0_is_scale_times_value},
         {"route_picks_the_top_k_and_renormalises", route_picks_the_top_k_and_renormalises},
+        {"moe_group_orders_rows_by_expert_then_token", moe_group_orders_rows_by_expert_then_token},
+        {"gather_then_combine_is_the_weighted_sum_of_the_hits", gather_then_combine_is_the_weighted_sum_of_the_hits},
+        {"argmax_is_the_last_maximum", argmax_is_the_last_maximum},
+        {"chunk_prologue_stores_the_rotated_k_and_v_rows", chunk_prologue_stores_the_rotated_k_and_v_rows},
     };
     try {
         Gpu::get();
