@@ -82,6 +82,24 @@ def test_add_rmsnorm_random(be, ora, case):
     check_float(host(th), wh, f16, (rows, n, f16))
 
 
+@pytest.mark.parametrize("case", range(12))
+def test_add_rmsnorm_random_batches(be, ora, case):
+    """Row counts in the thousands: the launch shapes the host picks by batch size (a wave per row while the
+    batch is resident at once, two tiles per lane beyond, four rows per workgroup from 8192 rows on)."""
+    g = np.random.default_rng(1500 + case)
+    f16 = bool(case & 1)
+    n = int(g.integers(8, 770)) * 8
+    rows = int(g.integers(1000, min(9000, 12_000_000 // n) + 1))
+    x, d = act(g, (rows, n), f16), act(g, (rows, n), f16)
+    gamma = S().normal_f32(g, n, 1.0, 0.05)
+    wx, wh = x.copy(), np.zeros_like(x)
+    ora.add_rmsnorm_rows(wx, d, wh, gamma, 1e-6)
+    tx, th = dev(x), torch.zeros_like(dev(x))
+    be.add_rmsnorm_rows(tx, dev(d), th, dev(gamma), 1e-6)
+    assert np.array_equal(host(tx), wx), (rows, n, f16)
+    check_float(host(th), wh, f16, (rows, n, f16))
+
+
 @pytest.mark.parametrize("case", range(CASES))
 def test_qknorm_rope_random(be, ora, case):
     g = np.random.default_rng(2000 + case)
@@ -115,6 +133,31 @@ def test_qknorm_rope_random(be, ora, case):
         check_float(host(tq), wq, f16, what)
     if n_kv:
         check_float(host(tk), wk, f16, what)
+
+
+@pytest.mark.parametrize("case", range(12))
+def test_qknorm_rope_random_batches(be, ora, case):
+    """Prefill-sized batches of the tiled kernels: enough waves for two passes per q wave in fp16, row
+    counts that are no multiple of anything."""
+    g = np.random.default_rng(2500 + case)
+    f16 = bool(case & 1)
+    hd = int(g.choice([64, 128, 256]))
+    n_q, n_kv = int(g.integers(1, 41)), int(g.integers(0, 9))
+    rows = int(g.integers(200, min(3000, 10_000_000 // ((n_q + n_kv) * hd)) + 1))
+    q, k = act(g, (rows, n_q * hd), f16), act(g, (rows, n_kv * hd), f16)
+    qw, kw = S().normal_f32(g, hd, 1.0, 0.05), S().normal_f32(g, hd, 1.0, 0.05)
+    positions = [int(v) for v in g.integers(0, 32768, size=rows)]
+    ropes = ora.rope_table(positions, ora.rope_inv_freq(hd, 1e6))
+    wq, wk = q.copy(), k.copy()
+    ora.qknorm_rope_rows(wq, wk, n_q, n_kv, hd, qw, kw, ropes, 1e-6)
+    tq, tk = dev(q), dev(k)
+    be.qknorm_rope_neox(tq, tk, dev(qw), dev(kw), dev(ropes), n_q, n_kv, hd, 1e-6)
+    what = (rows, n_q, n_kv, hd, f16)
+    check_float(host(tq), wq, f16, what)
+    if n_kv:
+        check_float(host(tk), wk, f16, what)
+    if f16:  # the definition, bit for bit
+        assert np.array_equal(host(tq), wq), what
 
 
 @pytest.mark.parametrize("case", range(CASES))
