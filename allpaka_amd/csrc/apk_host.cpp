@@ -184,6 +184,223 @@ int set_device(apk_ctx* c) {
     return APK_OK;
 }
 
+// ---- launch plans: which kernel, how many workgroups of how many lanes, for a shape.  Pure functions of
+// the sizes (no context, no GPU): the entries below launch exactly what these return, and the exported
+// apk_plan_* let a host check them anywhere.
+void plan_reset(apk_plan* p) { memset(p, 0, sizeof *p); }
+void plan_name(apk_plan* p, const std::string& k) { snprintf(p->kernel, sizeof p->kernel, "%s", k.c_str()); }
+
+enum { QK_TILED = 0, QK_GENERIC = 1 };
+// style: 0 = NeoX pairs (i, i + rot_dim/2), 1 = adjacent pairs (2i, 2i+1); with_kv: the K/V cache store fused in
+int plan_qknorm_rope(size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim, int style, int dtype, bool with_kv,
+                     apk_plan* p) {
+    plan_reset(p);
+    const int es = elem_size(dtype);
+    if (!es) return fail(APK_DECLINE_UNSUPPORTED, "apk_qknorm_rope: dtype %d", dtype);
+    if (head_dim == 0 || head_dim > 65536 || rot_dim % 2 || rot_dim > head_dim)
+        return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope: head_dim %zu, rot_dim %zu", head_dim, rot_dim);
+    const bool tiled = style == 0 && rot_dim == head_dim && (head_dim == 64 || head_dim == 128 || head_dim == 256);
+    if (with_kv && !tiled)
+        return fail(APK_DECLINE_UNSUPPORTED, "apk_qknorm_rope_kv_store: NeoX over a whole head of 64/128/256 only (head_dim %zu, rot_dim %zu)",
+                    head_dim, rot_dim);
+    if (rows == 0 || n_q + n_kv == 0) return APK_OK;
+    if (with_kv && n_kv == 0) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_kv_store: no k heads");
+    if (rows > 0x7fffffffu || n_q > 65535 || n_kv > 65535) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope: too large");
+    const char* t = dtype == APK_F32 ? "f32" : "f16";
+    if (!tiled) {
+        // a wave per head, element-wise: any head_dim, partial rotary, either pairing
+        const uint64_t grid = ((uint64_t)rows * (n_q + n_kv) + 3) / 4;
+        if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope: too large");
+        p->variant = QK_GENERIC;
+        plan_name(p, std::string("apk_qknorm_rope_generic_") + t);
+        p->grid = (unsigned)grid;
+        p->block = 256;
+        p->lanes_per_row = 64;
+        p->rows_per_block = 4;
+        return APK_OK;
+    }
+    // A wave owns (row, q or k, group of HPW*ITER heads), HPW = heads per wave pass; k waves
+    // take one pass.  Measured over 1024..8192 rows: fp16 is fastest with two passes per q wave
+    // (16 heads, 4 KB), f32 with one (4 heads, 2 KB); more passes per wave gain nothing where
+    // the batch happens to be a whole number of resident rounds and lose up to 15 % elsewhere.
+    // Small batches (under 6 waves per CU) take one pass: more waves.
+    const size_t epl = 16 / es, lph = head_dim / 2 / epl, hpw = 64 / lph;
+    const size_t gk = (n_kv + hpw - 1) / hpw;
+    unsigned iter = 1;
+    if (dtype == APK_F16 && n_q > hpw && rows * ((n_q + 2 * hpw - 1) / (2 * hpw) + gk) >= 1536) iter = 2;
+    const uint64_t waves = (uint64_t)rows * ((n_q + hpw * iter - 1) / (hpw * iter) + gk);
+    const unsigned block = 256;
+    const uint64_t grid = (waves * 64 + block - 1) / block;
+    if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope: too large");
+    p->variant = QK_TILED;
+    plan_name(p, std::string(with_kv ? "apk_qknorm_rope_kv_" : "apk_qknorm_rope_") + t + "_hd" + std::to_string(head_dim) + "_i" +
+                     std::to_string(iter));
+    p->grid = (unsigned)grid;
+    p->block = block;
+    p->tiles_per_lane = iter;
+    p->lanes_per_row = (unsigned)lph;
+    p->waves_per_row = (unsigned)((n_q + hpw * iter - 1) / (hpw * iter) + gk);
+    p->items = (unsigned)(waves > 0xffffffffu ? 0xffffffffu : waves);
+    return APK_OK;
+}
+
+enum { EMBED_Q4K = 0, EMBED_SUPERBLOCK = 1, EMBED_DIRECT = 2, EMBED_STAGED = 3 };
+int plan_embed(int fmt, size_t n_in, size_t t, int out_dtype, apk_plan* p) {
+    plan_reset(p);
+    if (!apk_can_embed(fmt, n_in)) return fail(APK_DECLINE_UNSUPPORTED, "apk_embed_rows: fmt %d / n_in %zu", fmt, n_in);
+    const int oes = elem_size(out_dtype);
+    if (!oes) return fail(APK_DECLINE_UNSUPPORTED, "apk_embed_rows: out_dtype %d", out_dtype);
+    if (t == 0) return APK_OK;
+    if (n_in > 0x7fffffffu || t > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_embed_rows: sizes out of range");
+    static const char* const kFmtName[10] = {"q4k", "q5k", "q6k", "q8_0", "q2k", "q3k", "q5_0", "f16", "f32", "bf16"};
+    plan_name(p, std::string("apk_embed_") + kFmtName[fmt] + (out_dtype == APK_F32 ? "_f32" : "_f16"));
+    uint64_t grid = t;
+    size_t threads = 0;
+    if (fmt == APK_FMT_Q4K) {
+        // one workgroup per row, 8 lanes per 256-element super-block
+        p->variant = EMBED_Q4K;
+        threads = (n_in / 256 * 8 + 63) / 64 * 64;
+        p->slices_per_row = 1;
+    } else if (fmt == APK_FMT_Q6K || fmt == APK_FMT_Q5K || fmt == APK_FMT_Q2K || fmt == APK_FMT_Q3K) {
+        // decoded straight from global memory, 8 lanes per 256-element super-block (the Q4_K lane layout)
+        p->variant = EMBED_SUPERBLOCK;
+        const size_t lanes = n_in / 256 * 8;
+        threads = (lanes + 63) / 64 * 64;
+        if (threads > 256) threads = 256;
+        p->slices_per_row = (unsigned)((lanes + threads - 1) / threads);
+        p->tiles_per_lane = (unsigned)(256 / (16 / oes) / 8);
+    } else if (fmt == APK_FMT_Q8_0 || fmt == APK_FMT_Q5_0 || fmt == APK_FMT_F32) {
+        // decoded straight from global memory: a lane owns 4 of the row's 16-byte output tiles; a row takes
+        // one workgroup of up to 256 lanes, or several chunks of 1024 tiles
+        p->variant = EMBED_DIRECT;
+        const size_t tiles_per_row = n_in / (16 / oes);
+        threads = ((tiles_per_row + 3) / 4 + 63) / 64 * 64;
+        if (threads > 256) threads = 256;
+        p->slices_per_row = (unsigned)((tiles_per_row + threads * 4 - 1) / (threads * 4));
+        p->tiles_per_lane = 4;
+    } else {
+        // F16 / BF16: one workgroup per row, the row staged in LDS, one output tile per lane and pass
+        p->variant = EMBED_STAGED;
+        threads = (n_in / (16 / oes) + 63) / 64 * 64;
+        p->shmem = (unsigned)(apk_row_bytes(fmt, n_in) + 32);
+        p->slices_per_row = 1;
+    }
+    if (threads > 256) threads = 256;
+    grid *= p->slices_per_row;
+    if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_embed_rows: too large");
+    p->grid = (unsigned)grid;
+    p->block = (unsigned)threads;
+    return APK_OK;
+}
+
+enum { ADDNORM_RAGGED = 0, ADDNORM_SMALL = 1, ADDNORM_TILED = 2 };
+int plan_add_rmsnorm(size_t n, size_t rows, int dtype, apk_plan* p) {
+    plan_reset(p);
+    const int es = elem_size(dtype);
+    if (!es) return fail(APK_DECLINE_UNSUPPORTED, "apk_add_rmsnorm_rows: dtype %d", dtype);
+    if (rows == 0) return APK_OK;
+    const size_t vec = 16 / es;
+    if (rows > 0x7fffffffu || n > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: too large");
+    if (n == 0) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: n is 0");
+    // Tiles per lane (NCH) and waves per row (W = ceil(nchunks / (64*NCH))), by batch size:
+    //  * few rows (rows * W <= 2048 waves, 8 per CU): the smallest NCH, i.e. the most waves per row;
+    //  * a batch that is resident all at once with a wave per row (or the fewest waves the register
+    //    budget allows): that shape -- every load of the launch is in flight at once, no barrier;
+    //  * a larger batch runs in several rounds of waves, and long waves then leave a long tail:
+    //    two tiles per lane and W waves per row, which stays within a few per cent of a plain copy
+    //    of the same bytes (6000 rows of 4096 fp16: 32.5 us against 36.7 us with a wave per row).
+    // Resident waves: 16 per CU up to 10 tiles per lane (<= 128 VGPRs), 12 at 12 tiles (144 VGPRs),
+    // 8 at 16 and 20 tiles (187 / 233 VGPRs).
+    const size_t nchunks = n / vec;
+    const int max_nch = dtype == APK_F16 ? 10 : 20;
+    int nch = 0;
+    size_t waves = 0;
+    if (n % vec == 0) {
+        for (size_t i = 0; i < sizeof kAddnormTiles / sizeof kAddnormTiles[0]; i++) {
+            const int cand = kAddnormTiles[i];
+            if (cand > max_nch) break;
+            const size_t w = (nchunks + 64 * (size_t)cand - 1) / (64 * (size_t)cand);
+            if (w * 64 > (size_t)kAddnormBound[i]) continue;
+            if (nch && w >= waves) continue;  // more tiles per lane only where that saves waves (no idle tiles)
+            nch = cand;
+            waves = w;
+            if (rows * w <= 2048) break;
+        }
+        const size_t resident = nch >= 16 ? 2048 : nch >= 12 ? 3072 : 4096;
+        if (nch > 2 && rows * waves > resident) {
+            const size_t w2 = (nchunks + 127) / 128;
+            if (w2 * 64 <= 1024) {
+                nch = 2;
+                waves = w2;
+            }
+        }
+    }
+    const char* t = dtype == APK_F32 ? "f32" : "f16";
+    if (!nch) {
+        // rows that are not whole 16-byte tiles, or longer than the tiled kernels hold in registers
+        // (20 480 elements): the element-wise two-pass kernel, a workgroup per row
+        p->variant = ADDNORM_RAGGED;
+        plan_name(p, std::string("apk_add_rmsnorm_ragged_") + t);
+        p->grid = (unsigned)rows;
+        p->block = 256;
+        p->waves_per_row = 4;
+        return APK_OK;
+    }
+    if (nchunks <= 32 && rows >= 16) {
+        // short rows in bulk (one head each, say): several rows per wave
+        const unsigned lpr = nchunks <= 4 ? 4 : nchunks <= 8 ? 8 : nchunks <= 16 ? 16 : 32;
+        const uint64_t rows_per_block = 4 * (64 / lpr);
+        const uint64_t grid = (rows + rows_per_block - 1) / rows_per_block;
+        if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: too large");
+        p->variant = ADDNORM_SMALL;
+        plan_name(p, std::string("apk_add_rmsnorm_small_") + t + "_l" + std::to_string(lpr));
+        p->grid = (unsigned)grid;
+        p->block = 256;
+        p->lanes_per_row = lpr;
+        p->rows_per_block = (unsigned)rows_per_block;
+        p->tiles_per_lane = 1;
+        return APK_OK;
+    }
+    // a wave per row: single-wave workgroups spread most evenly over the CUs (2441 rows of 4096 fp16: 14.4 us,
+    // against 17.0 us as 611 workgroups of four waves); from about 8192 rows on the spread no longer matters
+    // and four rows (waves) to a workgroup measure 1-3 % faster
+    const unsigned rpb = (waves == 1 && rows >= 8192) ? 4 : 1;
+    p->variant = ADDNORM_TILED;
+    plan_name(p, std::string("apk_add_rmsnorm_") + t + "_c" + std::to_string(nch));
+    p->grid = (unsigned)(rpb > 1 ? (rows + rpb - 1) / rpb : rows);
+    p->block = (unsigned)(rpb > 1 ? 256 : waves * 64);
+    p->tiles_per_lane = (unsigned)nch;
+    p->waves_per_row = (unsigned)waves;
+    p->rows_per_block = rpb;
+    p->lanes_per_row = (unsigned)waves * 64;
+    return APK_OK;
+}
+
+int plan_scatter(size_t rows, size_t k, size_t cols, int dtype, apk_plan* p) {
+    plan_reset(p);
+    const int es = elem_size(dtype);
+    if (!es) return fail(APK_DECLINE_UNSUPPORTED, "apk_scatter_rows: dtype %d", dtype);
+    if (rows == 0 || k == 0 || cols == 0) return APK_OK;
+    if ((cols * es) % 16) return fail(APK_DECLINE_SHAPE, "apk_scatter_rows: rows must be whole 16-byte tiles");
+    if (rows > 0x7fffffffu || k > 0x7fffffffu || cols * es / 16 > 0x7fffffffu)
+        return fail(APK_DECLINE_SHAPE, "apk_scatter_rows: too large");
+    // one workgroup per (token, slice, hit); one 16-byte tile per lane from 64 MB of output on, two below
+    // (fewer, slightly longer waves are ahead while the launch is short)
+    const uint64_t row_vecs = cols * es / 16;
+    const unsigned tpt = (uint64_t)rows * k * cols * es >= (64u << 20) ? 1 : 2;
+    const uint64_t slices = (row_vecs + 256 * tpt - 1) / (256 * tpt);
+    const uint64_t items = (uint64_t)rows * slices;
+    const uint64_t grid = (items + 7) / 8 * 8 * k;
+    if (items > 0xffffffffu || grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_scatter_rows: too large");
+    plan_name(p, tpt == 1 ? "apk_scatter_rows_t1" : "apk_scatter_rows_t2");
+    p->grid = (unsigned)grid;
+    p->block = 256;
+    p->tiles_per_lane = tpt;
+    p->slices_per_row = (unsigned)slices;
+    p->items = (unsigned)items;
+    return APK_OK;
+}
+
 }  // namespace
 
 #pragma GCC visibility push(default)
@@ -556,84 +773,30 @@ int apk_add_rmsnorm_rows(apk_ctx* c, void* x, const void* delta, void* h, const 
                          float eps, int dtype) {
     if (!c) return fail(APK_DECLINE_NULL, "apk_add_rmsnorm_rows: ctx is NULL");
     CallScope s(c);
-    const int es = elem_size(dtype);
-    if (!es) return fail(APK_DECLINE_UNSUPPORTED, "apk_add_rmsnorm_rows: dtype %d", dtype);
+    if (!elem_size(dtype)) return fail(APK_DECLINE_UNSUPPORTED, "apk_add_rmsnorm_rows: dtype %d", dtype);
     if (rows == 0) return APK_OK;
     if (!x || !h || !gamma) return fail(APK_DECLINE_NULL, "apk_add_rmsnorm_rows: NULL tensor");
-    const size_t vec = 16 / es;
-    if (rows > 0x7fffffffu || n > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: too large");
-    if (n == 0) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: n is 0");
-    // Tiles per lane (NCH) and waves per row (W = ceil(nchunks / (64*NCH))), by batch size:
-    //  * few rows (rows * W <= 2048 waves, 8 per CU): the smallest NCH, i.e. the most waves per row;
-    //  * a batch that is resident all at once with a wave per row (or the fewest waves the register
-    //    budget allows): that shape -- every load of the launch is in flight at once, no barrier;
-    //  * a larger batch runs in several rounds of waves, and long waves then leave a long tail:
-    //    two tiles per lane and W waves per row, which stays within a few per cent of a plain copy
-    //    of the same bytes (6000 rows of 4096 fp16: 32.5 us against 36.7 us with a wave per row).
-    // Resident waves: 16 per CU up to 10 tiles per lane (<= 128 VGPRs), 12 at 12 tiles (144 VGPRs),
-    // 8 at 16 and 20 tiles (187 / 233 VGPRs).
-    const size_t nchunks = n / vec;
-    const int max_nch = dtype == APK_F16 ? 10 : 20;
-    int nch = 0;
-    size_t waves = 0;
-    if (n % vec == 0) {
-        for (size_t i = 0; i < sizeof kAddnormTiles / sizeof kAddnormTiles[0]; i++) {
-            const int cand = kAddnormTiles[i];
-            if (cand > max_nch) break;
-            const size_t w = (nchunks + 64 * (size_t)cand - 1) / (64 * (size_t)cand);
-            if (w * 64 > (size_t)kAddnormBound[i]) continue;
-            if (nch && w >= waves) continue;  // more tiles per lane only where that saves waves (no idle tiles)
-            nch = cand;
-            waves = w;
-            if (rows * w <= 2048) break;
-        }
-        const size_t resident = nch >= 16 ? 2048 : nch >= 12 ? 3072 : 4096;
-        if (nch > 2 && rows * waves > resident) {
-            const size_t w2 = (nchunks + 127) / 128;
-            if (w2 * 64 <= 1024) {
-                nch = 2;
-                waves = w2;
-            }
-        }
-    }
-    if (!nch) {
-        // rows that are not whole 16-byte tiles, or longer than the tiled kernels hold in registers
-        // (20 480 elements): the element-wise two-pass kernel
-        if (h == x && delta) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: h aliases x while delta is given");
-        if (int rc = set_device(c)) return rc;
-        int n_r = (int)n;
-        void* rargs[] = {&x, &delta, &h, &gamma, &n_r, &eps};
-        return launch(c, dtype == APK_F32 ? "apk_add_rmsnorm_ragged_f32" : "apk_add_rmsnorm_ragged_f16", (unsigned)rows, 256, 0, rargs);
-    }
-    if (!aligned16(x) || !aligned16(h) || !aligned16(gamma) || (delta && !aligned16(delta)))
+    apk_plan p;
+    if (int rc = plan_add_rmsnorm(n, rows, dtype, &p)) return rc;
+    // the element-wise and the several-rows-per-wave kernels read a row twice: the norm must not land on it
+    if (p.variant != ADDNORM_TILED && h == x && delta)
+        return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: h aliases x while delta is given");
+    if (p.variant != ADDNORM_RAGGED && (!aligned16(x) || !aligned16(h) || !aligned16(gamma) || (delta && !aligned16(delta))))
         return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: tensors must be 16-byte aligned");
-    if (nchunks <= 32 && rows >= 16) {
-        // short rows in bulk (one head each, say): several rows per wave
-        const int lpr = nchunks <= 4 ? 4 : nchunks <= 8 ? 8 : nchunks <= 16 ? 16 : 32;
-        if (h == x && delta) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: h aliases x while delta is given");
-        const uint64_t rows_per_block = 4 * (64 / lpr);
-        const uint64_t grid = (rows + rows_per_block - 1) / rows_per_block;
-        if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_add_rmsnorm_rows: too large");
-        if (int rc = set_device(c)) return rc;
-        int n_s = (int)n;
-        uint32_t rows32 = (uint32_t)rows;
-        void* sargs[] = {&x, &delta, &h, &gamma, &n_s, &rows32, &eps};
-        return launch(c, std::string("apk_add_rmsnorm_small_") + (dtype == APK_F32 ? "f32" : "f16") + "_l" + std::to_string(lpr),
-                      (unsigned)grid, 256, 0, sargs);
-    }
-    // a wave per row: single-wave workgroups spread most evenly over the CUs (2441 rows of 4096 fp16: 14.4 us,
-    // against 17.0 us as 611 workgroups of four waves); from about 8192 rows on the spread no longer matters
-    // and four rows (waves) to a workgroup measure 1-3 % faster
-    const uint32_t rpb = (waves == 1 && rows >= 8192) ? 4 : 1;
-    const size_t threads = rpb > 1 ? 256 : waves * 64;
-    const size_t grid = rpb > 1 ? (rows + rpb - 1) / rpb : rows;
     if (int rc = set_device(c)) return rc;
     int n_i = (int)n;
     uint32_t rows32 = (uint32_t)rows;
-    void* args[] = {&x, &delta, &h, &gamma, &n_i, &eps, (void*)&rpb, &rows32};
-    return launch_keyed(c, OP_ADDNORM, (uint32_t)dtype << 8 | (uint32_t)nch,
-                        [&] { return std::string("apk_add_rmsnorm_") + (dtype == APK_F32 ? "f32" : "f16") + "_c" + std::to_string(nch); },
-                        (unsigned)grid, (unsigned)threads, 0, args);
+    if (p.variant == ADDNORM_RAGGED) {
+        void* rargs[] = {&x, &delta, &h, &gamma, &n_i, &eps};
+        return launch(c, p.kernel, p.grid, p.block, 0, rargs);
+    }
+    if (p.variant == ADDNORM_SMALL) {
+        void* sargs[] = {&x, &delta, &h, &gamma, &n_i, &rows32, &eps};
+        return launch(c, p.kernel, p.grid, p.block, 0, sargs);
+    }
+    void* args[] = {&x, &delta, &h, &gamma, &n_i, &eps, &p.rows_per_block, &rows32};
+    return launch_keyed(c, OP_ADDNORM, (uint32_t)dtype << 8 | p.tiles_per_lane, [&] { return std::string(p.kernel); }, p.grid, p.block, 0,
+                        args);
 }
 
 struct KvStore {  // the fused K/V cache store of apk_qknorm_rope_kv_store (all NULL/0: plain op)
@@ -649,65 +812,36 @@ struct KvStore {  // the fused K/V cache store of apk_qknorm_rope_kv_store (all 
 static int qknorm_rope_common(apk_ctx* c, void* q, void* k, const float* qw, const float* kw, const float* rope, size_t rows,
                               size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim, float eps, int dtype,
                               const KvStore* kv, int style = 0, bool validate_only = false) {
-    const int es = elem_size(dtype);
-    if (!es) return fail(APK_DECLINE_UNSUPPORTED, "apk_qknorm_rope: dtype %d", dtype);
-    if (head_dim == 0 || head_dim > 65536 || rot_dim % 2 || rot_dim > head_dim)
-        return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope: head_dim %zu, rot_dim %zu", head_dim, rot_dim);
-    const bool tiled = style == 0 && rot_dim == head_dim && (head_dim == 64 || head_dim == 128 || head_dim == 256);
-    if (kv && !tiled)
-        return fail(APK_DECLINE_UNSUPPORTED, "apk_qknorm_rope_kv_store: NeoX over a whole head of 64/128/256 only (head_dim %zu, rot_dim %zu)",
-                    head_dim, rot_dim);
+    apk_plan p;
+    if (int rc = plan_qknorm_rope(rows, n_q, n_kv, head_dim, rot_dim, style, dtype, kv != nullptr, &p)) return rc;
     if (rows == 0 || n_q + n_kv == 0) return APK_OK;
     if ((n_q && !q) || (n_kv && !k) || (!rope && rot_dim)) return fail(APK_DECLINE_NULL, "apk_qknorm_rope: NULL tensor");
     if ((q && !aligned16(q)) || (k && !aligned16(k)) || !aligned16(rope) || (qw && !aligned16(qw)) || (kw && !aligned16(kw)))
         return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope: tensors must be 16-byte aligned");
     if (kv) {
-        if (n_kv == 0) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_kv_store: no k heads");
         if (!kv->v || !kv->cache_pos || !kv->k_cache || !kv->v_cache) return fail(APK_DECLINE_NULL, "apk_qknorm_rope_kv_store: NULL tensor");
         if (!aligned16(kv->v) || !aligned16(kv->k_cache) || !aligned16(kv->v_cache))
             return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_kv_store: tensors must be 16-byte aligned");
         if (kv->capacity == 0 || kv->capacity > 0xffffffffu) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_kv_store: capacity");
     }
-    if (rows > 0x7fffffffu || n_q > 65535 || n_kv > 65535) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope: too large");
+    if (validate_only) return APK_OK;
+    if (int rc = set_device(c)) return rc;
     int rows_i = (int)rows, nq_i = (int)n_q, nkv_i = (int)n_kv;
-    if (!tiled) {
-        // a wave per head, element-wise: any head_dim, partial rotary, either pairing
-        const uint64_t grid = ((uint64_t)rows * (n_q + n_kv) + 3) / 4;
-        if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope: too large");
-        if (validate_only) return APK_OK;
-        if (int rc = set_device(c)) return rc;
+    if (p.variant == QK_GENERIC) {
         int hd_i = (int)head_dim, half_i = (int)(rot_dim / 2);
         void* gargs[] = {&q, &k, &qw, &kw, &rope, &rows_i, &nq_i, &nkv_i, &hd_i, &half_i, &style, &eps};
-        return launch(c, dtype == APK_F32 ? "apk_qknorm_rope_generic_f32" : "apk_qknorm_rope_generic_f16", (unsigned)grid, 256, 0, gargs);
+        return launch(c, p.kernel, p.grid, p.block, 0, gargs);
     }
-    // A wave owns (row, q or k, group of HPW*ITER heads), HPW = heads per wave pass; k waves
-    // take one pass.  Measured over 1024..8192 rows: fp16 is fastest with two passes per q wave
-    // (16 heads, 4 KB), f32 with one (4 heads, 2 KB); more passes per wave gain nothing where
-    // the batch happens to be a whole number of resident rounds and lose up to 15 % elsewhere.
-    // Small batches (under 6 waves per CU) take one pass: more waves.
-    const size_t epl = 16 / es, lph = head_dim / 2 / epl, hpw = 64 / lph;
-    const size_t gk = (n_kv + hpw - 1) / hpw;
-    int iter = 1;
-    if (dtype == APK_F16 && n_q > hpw && rows * ((n_q + 2 * hpw - 1) / (2 * hpw) + gk) >= 1536) iter = 2;
-    const uint64_t waves = (uint64_t)rows * ((n_q + hpw * iter - 1) / (hpw * iter) + gk);
-    const unsigned block = 256;
-    const uint64_t grid = (waves * 64 + block - 1) / block;
-    if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope: too large");
-    if (validate_only) return APK_OK;
-    auto which = [&] {
-        return std::string(kv ? "apk_qknorm_rope_kv_" : "apk_qknorm_rope_") + (dtype == APK_F32 ? "f32" : "f16") + "_hd" +
-               std::to_string(head_dim) + "_i" + std::to_string(iter);
-    };
-    const uint32_t variant = (uint32_t)dtype << 16 | (uint32_t)head_dim << 4 | (uint32_t)iter;
-    if (int rc = set_device(c)) return rc;
+    auto which = [&] { return std::string(p.kernel); };
+    const uint32_t variant = (uint32_t)dtype << 16 | (uint32_t)head_dim << 4 | p.tiles_per_lane;
     if (kv) {
         uint32_t cap32 = (uint32_t)kv->capacity;
         void* kargs[] = {&q, &k, (void*)&kv->v, &qw, &kw, &rope, (void*)&kv->cache_pos, (void*)&kv->k_cache, (void*)&kv->v_cache,
                          &cap32, &rows_i, &nq_i, &nkv_i, &eps, &c->fault_dev};
-        return launch_keyed(c, OP_QKROPE_KV, variant, which, (unsigned)grid, block, 0, kargs);
+        return launch_keyed(c, OP_QKROPE_KV, variant, which, p.grid, p.block, 0, kargs);
     }
     void* args[] = {&q, &k, &qw, &kw, &rope, &rows_i, &nq_i, &nkv_i, &eps};
-    return launch_keyed(c, OP_QKROPE, variant, which, (unsigned)grid, block, 0, args);
+    return launch_keyed(c, OP_QKROPE, variant, which, p.grid, p.block, 0, args);
 }
 
 int apk_qknorm_rope_neox(apk_ctx* c, void* q, void* k, const float* qw, const float* kw, const float* rope,
@@ -790,65 +924,28 @@ int apk_rope_table(apk_ctx* c, const uint32_t* positions, const float* inv_freq,
 // ids_dev == nullptr with have_ids == false: the rows row0, row0 + 1, ... (apk_dequant_rows)
 static int embed_common(apk_ctx* c, int fmt, const void* table, size_t vocab, size_t n_in, const uint32_t* ids_dev,
                         size_t t, void* out, int out_dtype, float scale = 1.0f, bool have_ids = true, uint32_t row0 = 0) {
-    if (!apk_can_embed(fmt, n_in)) return fail(APK_DECLINE_UNSUPPORTED, "apk_embed_rows: fmt %d / n_in %zu", fmt, n_in);
-    if (!elem_size(out_dtype)) return fail(APK_DECLINE_UNSUPPORTED, "apk_embed_rows: out_dtype %d", out_dtype);
+    apk_plan p;
+    if (int rc = plan_embed(fmt, n_in, t, out_dtype, &p)) return rc;
     if (t == 0) return APK_OK;
     if (!table || (have_ids && !ids_dev) || !out) return fail(APK_DECLINE_NULL, "apk_embed_rows: NULL tensor");
     if (!aligned16(table) || !aligned16(out)) return fail(APK_DECLINE_SHAPE, "apk_embed_rows: table/out must be 16-byte aligned");
-    if (vocab == 0 || vocab > 0xffffffffu || n_in > 0x7fffffffu || t > 0x7fffffffu)
-        return fail(APK_DECLINE_SHAPE, "apk_embed_rows: sizes out of range");
+    if (vocab == 0 || vocab > 0xffffffffu) return fail(APK_DECLINE_SHAPE, "apk_embed_rows: sizes out of range");
     if (int rc = set_device(c)) return rc;
     uint32_t vocab32 = (uint32_t)vocab;
     int n_i = (int)n_in;
-    if (fmt == APK_FMT_Q4K) {
-        // one workgroup per row, 8 lanes per 256-element super-block
-        size_t threads = (n_in / 256 * 8 + 63) / 64 * 64;
-        if (threads > 256) threads = 256;
+    const uint32_t key = (uint32_t)fmt << 8 | (uint32_t)out_dtype;
+    auto which = [&] { return std::string(p.kernel); };
+    if (p.variant == EMBED_Q4K) {
         void* args[] = {&table, &vocab32, &n_i, &ids_dev, &out, &c->fault_dev, &scale, &row0};
-        return launch_keyed(c, OP_EMBED, (uint32_t)fmt << 8 | (uint32_t)out_dtype,
-                            [&] { return std::string(out_dtype == APK_F32 ? "apk_embed_q4k_f32" : "apk_embed_q4k_f16"); }, (unsigned)t,
-                            (unsigned)threads, 0, args);
+        return launch_keyed(c, OP_EMBED, key, which, p.grid, p.block, 0, args);
     }
-    static const char* const kFmtName[10] = {"q4k", "q5k", "q6k", "q8_0", "q2k", "q3k", "q5_0", "f16", "f32", "bf16"};
-    if (fmt == APK_FMT_Q6K || fmt == APK_FMT_Q5K || fmt == APK_FMT_Q2K || fmt == APK_FMT_Q3K) {
-        // decoded straight from global memory, 8 lanes per 256-element super-block (the Q4_K lane layout)
-        const size_t lanes = n_in / 256 * 8;
-        size_t threads = (lanes + 63) / 64 * 64;
-        if (threads > 256) threads = 256;
-        const size_t chunks = (lanes + threads - 1) / threads;
-        const uint64_t grid = (uint64_t)t * chunks;
-        if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_embed_rows: too large");
-        uint32_t chunks32 = (uint32_t)chunks;
-        void* args[] = {&table, &vocab32, &n_i, &ids_dev, &chunks32, &out, &c->fault_dev, &scale, &row0};
-        return launch_keyed(c, OP_EMBED, (uint32_t)fmt << 8 | (uint32_t)out_dtype,
-                            [&] { return std::string("apk_embed_") + kFmtName[fmt] + (out_dtype == APK_F32 ? "_f32" : "_f16"); },
-                            (unsigned)grid, (unsigned)threads, 0, args);
+    if (p.variant == EMBED_STAGED) {
+        uint64_t table_bytes = (uint64_t)vocab * apk_row_bytes(fmt, n_in);
+        void* args[] = {&table, &table_bytes, &vocab32, &n_i, &ids_dev, &out, &c->fault_dev, &scale, &row0};
+        return launch_keyed(c, OP_EMBED, key, which, p.grid, p.block, p.shmem, args);
     }
-    if (fmt == APK_FMT_Q8_0 || fmt == APK_FMT_Q5_0 || fmt == APK_FMT_F32) {
-        // decoded straight from global memory: a lane owns 4 of the row's 16-byte output tiles; a row takes
-        // one workgroup of up to 256 lanes, or several chunks of 1024 tiles
-        const size_t tiles_per_row = n_in / (16 / elem_size(out_dtype));
-        size_t threads = ((tiles_per_row + 3) / 4 + 63) / 64 * 64;
-        if (threads > 256) threads = 256;
-        const size_t chunks = (tiles_per_row + threads * 4 - 1) / (threads * 4);
-        const uint64_t grid = (uint64_t)t * chunks;
-        if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_embed_rows: too large");
-        uint32_t chunks32 = (uint32_t)chunks;
-        void* args[] = {&table, &vocab32, &n_i, &ids_dev, &chunks32, &out, &c->fault_dev, &scale, &row0};
-        return launch_keyed(c, OP_EMBED, (uint32_t)fmt << 8 | (uint32_t)out_dtype,
-                            [&] { return std::string("apk_embed_") + kFmtName[fmt] + (out_dtype == APK_F32 ? "_f32" : "_f16"); },
-                            (unsigned)grid, (unsigned)threads, 0, args);
-    }
-    // the remaining formats: one workgroup per row, the row staged in LDS
-    const size_t row_bytes = apk_row_bytes(fmt, n_in);
-    const size_t shmem = row_bytes + 32;
-    size_t threads = (n_in / (16 / elem_size(out_dtype)) + 63) / 64 * 64;  // one output tile per lane
-    if (threads > 256) threads = 256;
-    uint64_t table_bytes = (uint64_t)vocab * row_bytes;
-    void* args[] = {&table, &table_bytes, &vocab32, &n_i, &ids_dev, &out, &c->fault_dev, &scale, &row0};
-    return launch_keyed(c, OP_EMBED, (uint32_t)fmt << 8 | (uint32_t)out_dtype,
-                        [&] { return std::string("apk_embed_") + kFmtName[fmt] + (out_dtype == APK_F32 ? "_f32" : "_f16"); }, (unsigned)t,
-                        (unsigned)threads, (unsigned)shmem, args);
+    void* args[] = {&table, &vocab32, &n_i, &ids_dev, &p.slices_per_row, &out, &c->fault_dev, &scale, &row0};
+    return launch_keyed(c, OP_EMBED, key, which, p.grid, p.block, 0, args);
 }
 
 int apk_embed_rows(apk_ctx* c, int fmt, const void* table, size_t vocab, size_t n_in, const uint32_t* ids, size_t t,
@@ -993,22 +1090,15 @@ int apk_scatter_rows(apk_ctx* c, const void* src, const uint32_t* hit_row, size_
     if (!es) return fail(APK_DECLINE_UNSUPPORTED, "apk_scatter_rows: dtype %d", dtype);
     if (rows == 0 || k == 0 || cols == 0) return APK_OK;
     if (!src || !hit_row || !dst) return fail(APK_DECLINE_NULL, "apk_scatter_rows: NULL tensor");
-    if ((cols * es) % 16 || !aligned16(src) || !aligned16(dst))
-        return fail(APK_DECLINE_SHAPE, "apk_scatter_rows: rows must be whole 16-byte tiles");
-    if (rows > 0x7fffffffu || total_rows > 0xffffffffu || k > 0x7fffffffu || cols * es / 16 > 0x7fffffffu)
-        return fail(APK_DECLINE_SHAPE, "apk_scatter_rows: too large");
-    // one workgroup per (token, slice, hit); one 16-byte tile per lane from 64 MB of output on, two below
-    // (fewer, slightly longer waves are ahead while the launch is short)
-    const int row_vecs = (int)(cols * es / 16);
-    const int tpt = (uint64_t)rows * k * cols * es >= (64u << 20) ? 1 : 2;
-    const uint64_t slices = ((uint64_t)row_vecs + 256 * tpt - 1) / (256 * tpt);
-    const uint64_t items = (uint64_t)rows * slices;
-    const uint64_t grid = (items + 7) / 8 * 8 * k;
-    if (items > 0xffffffffu || grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_scatter_rows: too large");
+    if (!aligned16(src) || !aligned16(dst)) return fail(APK_DECLINE_SHAPE, "apk_scatter_rows: rows must be whole 16-byte tiles");
+    if (total_rows > 0xffffffffu) return fail(APK_DECLINE_SHAPE, "apk_scatter_rows: too large");
+    apk_plan p;
+    if (int rc = plan_scatter(rows, k, cols, dtype, &p)) return rc;
     if (int rc = set_device(c)) return rc;
-    uint32_t k32 = (uint32_t)k, total32 = (uint32_t)total_rows, items32 = (uint32_t)items, slices32 = (uint32_t)slices;
-    void* args[] = {&src, &hit_row, &k32, &total32, (void*)&row_vecs, &dst, &c->fault_dev, &items32, &slices32};
-    return launch(c, tpt == 1 ? "apk_scatter_rows_t1" : "apk_scatter_rows_t2", (unsigned)grid, 256, 0, args);
+    int row_vecs = (int)(cols * es / 16);
+    uint32_t k32 = (uint32_t)k, total32 = (uint32_t)total_rows;
+    void* args[] = {&src, &hit_row, &k32, &total32, &row_vecs, &dst, &c->fault_dev, &p.items, &p.slices_per_row};
+    return launch(c, p.kernel, p.grid, p.block, 0, args);
 }
 
 int apk_moe_combine_add_rmsnorm(apk_ctx* c, void* x, const void* flat, const uint32_t* tok_off, const uint32_t* hit_row,
@@ -1078,6 +1168,39 @@ int apk_argmax_rows(apk_ctx* c, const float* logits, size_t rows, size_t n, uint
     void* args[] = {&logits, &n64, &parts_i, &c->argmax_scratch, &out};
     if (c->capturing) c->capture_argmax = true;
     return launch_keyed(c, OP_ARGMAX, 0, [] { return std::string("apk_argmax_rows"); }, (unsigned)(rows * parts), 256, 0, args);
+}
+
+/* ------------------------------------------------------------- launch plans */
+
+int apk_plan_add_rmsnorm_rows(size_t n, size_t rows, int dtype, apk_plan* plan) {
+    if (!plan) return fail(APK_DECLINE_NULL, "apk_plan_add_rmsnorm_rows: plan is NULL");
+    return plan_add_rmsnorm(n, rows, dtype, plan);
+}
+
+int apk_plan_qknorm_rope(size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim, int adjacent_pairs, int dtype,
+                         int with_kv_store, apk_plan* plan) {
+    if (!plan) return fail(APK_DECLINE_NULL, "apk_plan_qknorm_rope: plan is NULL");
+    return plan_qknorm_rope(rows, n_q, n_kv, head_dim, rot_dim, adjacent_pairs ? 1 : 0, dtype, with_kv_store != 0, plan);
+}
+
+int apk_plan_scatter_rows(size_t rows, size_t k, size_t cols, int dtype, apk_plan* plan) {
+    if (!plan) return fail(APK_DECLINE_NULL, "apk_plan_scatter_rows: plan is NULL");
+    return plan_scatter(rows, k, cols, dtype, plan);
+}
+
+int apk_plan_embed_rows(int fmt, size_t n_in, size_t t, int out_dtype, apk_plan* plan) {
+    if (!plan) return fail(APK_DECLINE_NULL, "apk_plan_embed_rows: plan is NULL");
+    return plan_embed(fmt, n_in, t, out_dtype, plan);
+}
+
+size_t apk_kernel_count(void) { return all_kernel_names().size(); }
+
+int apk_kernel_name(size_t i, char* name, size_t cap) {
+    const std::vector<std::string> v = all_kernel_names();
+    if (!name || cap == 0) return fail(APK_DECLINE_NULL, "apk_kernel_name: name is NULL");
+    if (i >= v.size()) return fail(APK_DECLINE_RANGE, "apk_kernel_name: %zu of %zu", i, v.size());
+    snprintf(name, cap, "%s", v[i].c_str());
+    return APK_OK;
 }
 
 int apk_copy(apk_ctx* c, const void* src, void* dst, size_t bytes) {

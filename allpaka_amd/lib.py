@@ -11,8 +11,18 @@ FMT_Q4K, FMT_Q5K, FMT_Q6K, FMT_Q8_0, FMT_Q2K, FMT_Q3K, FMT_Q5_0, FMT_F16, FMT_F3
 DECLINE_UNSUPPORTED, DECLINE_SHAPE, DECLINE_NULL, DECLINE_RANGE, DECLINE_NO_DEVICE, DECLINE_NOT_ATTACHED, DECLINE_CAPTURE = range(1, 8)
 FAULT_TOKEN_RANGE, FAULT_EXPERT_RANGE, FAULT_ROW_RANGE, FAULT_CACHE_RANGE = 1, 2, 4, 8
 
+
+
+class Plan(C.Structure):
+    """struct apk_plan: the kernel, grid and workgroup size an entry launches for a shape."""
+    _fields_ = [("kernel", C.c_char * 64), ("grid", C.c_uint), ("block", C.c_uint), ("shmem", C.c_uint), ("variant", C.c_uint),
+                ("tiles_per_lane", C.c_uint), ("waves_per_row", C.c_uint), ("rows_per_block", C.c_uint), ("lanes_per_row", C.c_uint),
+                ("slices_per_row", C.c_uint), ("items", C.c_uint)]
+
+
 # every symbol include/apk_hip.h declares: (restype, argtypes)
 _vp, _sz, _i, _f, _u64p, _u32p = C.c_void_p, C.c_size_t, C.c_int, C.c_float, C.POINTER(C.c_uint64), C.POINTER(C.c_uint32)
+_plan = C.POINTER(Plan)
 SYMBOLS = {
     "apk_init": (_i, [_i, C.POINTER(_vp)]),
     "apk_shutdown": (_i, [_vp]),
@@ -58,6 +68,12 @@ SYMBOLS = {
     "apk_moe_combine_add_rmsnorm": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _sz, _sz, _f, _i]),
     "apk_argmax_rows": (_i, [_vp, _vp, _sz, _sz, _vp]),
     "apk_copy": (_i, [_vp, _vp, _vp, _sz]),
+    "apk_plan_add_rmsnorm_rows": (_i, [_sz, _sz, _i, _plan]),
+    "apk_plan_qknorm_rope": (_i, [_sz, _sz, _sz, _sz, _sz, _i, _i, _i, _plan]),
+    "apk_plan_scatter_rows": (_i, [_sz, _sz, _sz, _i, _plan]),
+    "apk_plan_embed_rows": (_i, [_i, _sz, _sz, _i, _plan]),
+    "apk_kernel_count": (_sz, []),
+    "apk_kernel_name": (_i, [_sz, C.c_char_p, _sz]),
 }
 
 

@@ -53,6 +53,22 @@ enum apk_decline {
     APK_DECLINE_CAPTURE = 7       /* not possible while (or: only while) the stream is being recorded  */
 };
 
+/* What an entry would launch for a shape: the kernel of the code object, its grid and workgroup size.
+ * Filled by the apk_plan_* functions below, which need neither a context nor a GPU: the entries launch
+ * exactly what these return, so the host's choice of launch shape can be checked on any machine. */
+typedef struct apk_plan {
+    char kernel[64];          /* kernel name in the code object; "" when there is nothing to launch       */
+    unsigned grid, block;     /* workgroups, lanes per workgroup                                           */
+    unsigned shmem;           /* dynamic LDS bytes                                                         */
+    unsigned variant;         /* entry-specific code path (0 when the entry has one)                       */
+    unsigned tiles_per_lane;  /* 16-byte tiles (or passes) a lane takes                                    */
+    unsigned waves_per_row;   /* waves that share one row (0 where rows are not the unit)                  */
+    unsigned rows_per_block;  /* rows (or row items) a workgroup takes when each wave or lane group owns one */
+    unsigned lanes_per_row;   /* lanes that cover one row or one head                                      */
+    unsigned slices_per_row;  /* workgroup-sized slices a row is cut into                                  */
+    unsigned items;           /* work items of the launch before it is rounded up to whole workgroups      */
+} apk_plan;
+
 /* Unified dequant format codes -- the exact integers of gpu::common::dq_fmt
  * (crates/allpaka-backend/src/gpu/common.rs:47-61). */
 enum apk_dq_fmt {
@@ -317,6 +333,21 @@ int apk_argmax_rows(apk_ctx* ctx, const float* logits, size_t rows, size_t n, ui
 /* dst = src, `bytes` a multiple of 16: the plain stream kernel the bandwidth
  * figures of the other kernels are calibrated against. */
 int apk_copy(apk_ctx* ctx, const void* src, void* dst, size_t bytes);
+
+/* Launch plans (no context, no GPU; see apk_plan): what apk_add_rmsnorm_rows, apk_qknorm_rope_neox /
+ * _norm (adjacent_pairs != 0) / _kv_store (with_kv_store != 0), apk_scatter_rows and apk_embed_rows /
+ * apk_dequant_rows launch for these sizes.  Return APK_OK with plan filled (kernel "" and grid 0 when
+ * the call would be a no-op), or the decline the entry itself would return for the sizes.  They have no
+ * counterpart in the reference: its hosts size their dispatches inline (e.g. gpu/cuda/runtime/gemm.rs:218-233). */
+int apk_plan_add_rmsnorm_rows(size_t n, size_t rows, int dtype, apk_plan* plan);
+int apk_plan_qknorm_rope(size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim, int adjacent_pairs, int dtype,
+                         int with_kv_store, apk_plan* plan);
+int apk_plan_scatter_rows(size_t rows, size_t k, size_t cols, int dtype, apk_plan* plan);
+int apk_plan_embed_rows(int fmt, size_t n_in, size_t t, int out_dtype, apk_plan* plan);
+/* The kernels apk_init resolves from the embedded code object: their number, and the i-th name copied into
+ * name[cap] (every plan names one of them). */
+size_t apk_kernel_count(void);
+int apk_kernel_name(size_t i, char* name, size_t cap);
 
 #ifdef __cplusplus
 }
