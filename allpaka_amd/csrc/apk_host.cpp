@@ -981,6 +981,9 @@ int apk_embed_rows_host_ids(apk_ctx* c, int fmt, const void* table, size_t vocab
     for (size_t i = 0; i < t; i++)
         if (ids_host[i] >= vocab)
             return fail(APK_DECLINE_RANGE, "apk_embed_rows_host_ids: token %u at %zu >= vocab %zu", ids_host[i], i, vocab);
+    // a single token (a decode step with the sampler on the host): the id travels as a kernel argument, with no
+    // staging copy and no wait on the stream
+    if (t == 1) return embed_common(c, fmt, table, vocab, n_in, nullptr, 1, out, out_dtype, 1.0f, false, ids_host[0]);
     if (int rc = set_device(c)) return rc;
     if (t > c->ids_stage_cap) {
         // the previous staging buffer may still be read by an enqueued copy

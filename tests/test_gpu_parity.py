@@ -200,6 +200,42 @@ def test_embed_subnormal_scales_and_reference_vectors(be, ora):
     assert got[0] == 9.0 and got[1] == -1.0 and got[32] == 19.0 and got[33] == -2.0 and np.all(got[64:] == 0.0)
 
 
+def test_embed_with_the_ids_on_the_host(be, ora):
+    """apk_embed_rows_host_ids: the ids are range-checked before anything is enqueued (as the reference's
+    callers reject token >= vocab first); a single token travels as a kernel argument, more through a pinned
+    staging buffer -- the same rows as the device-id entry either way, call after call."""
+    import ctypes as C
+
+    import allpaka_amd.lib as apklib
+
+    s = synth()
+    vocab, hidden = 300, 512
+    for fmt_name in ("Q4K", "Q8_0", "F16"):
+        fmt = ora.FMT[fmt_name]
+        rb = ora.expected_bytes(fmt, hidden)
+        raw = _lcg_bytes(vocab * rb, 0x9E3779B97F4A7C15 + fmt)
+        if fmt_name in _SCALE_OFFS:
+            bb, offs = _SCALE_OFFS[fmt_name]
+            for o in offs:
+                raw.reshape(-1, bb)[:, o], raw.reshape(-1, bb)[:, o + 1] = 0x1F, 0x21
+        else:
+            raw.view(np.uint16)[:] &= np.uint16(0xBFFF)
+        table = dev(raw)
+        for ids in ([7], [299], [5, 0, 299, 5, 17], list(range(40, 90)), [3]):
+            want = ora.embed_rows(raw, fmt, vocab, hidden, np.array(ids, np.uint32), out_f16=True)
+            out = torch.zeros((len(ids), hidden), dtype=torch.float16, device="cuda")
+            harr = (C.c_uint32 * len(ids))(*ids)
+            apklib.check(be.L.apk_embed_rows_host_ids(be.h, fmt, table.data_ptr(), vocab, hidden, harr, len(ids), out.data_ptr(), apklib.F16))
+            be.sync()
+            assert np.array_equal(host(out), want), (fmt_name, ids)
+        for bad in ([300], [1, 2, 300]):
+            harr = (C.c_uint32 * len(bad))(*bad)
+            out = torch.full((len(bad), hidden), 2.0, dtype=torch.float16, device="cuda")
+            rc = be.L.apk_embed_rows_host_ids(be.h, fmt, table.data_ptr(), vocab, hidden, harr, len(bad), out.data_ptr(), apklib.F16)
+            be.sync()
+            assert rc == apklib.DECLINE_RANGE and torch.all(out == 2.0) and be.take_faults() == 0
+
+
 def test_embed_errors_and_declines(be, ora):
     import allpaka_amd as apk
 
