@@ -179,7 +179,9 @@ int apk_embed_rows(apk_ctx* ctx, int fmt, const void* table, size_t vocab, size_
 int apk_embed_rows_scaled(apk_ctx* ctx, int fmt, const void* table, size_t vocab, size_t n_in, const uint32_t* ids,
                           size_t t, float scale, void* out, int out_dtype);
 /* Same with the ids on the host: range-checked BEFORE anything is enqueued
- * (APK_DECLINE_RANGE), as the reference's callers reject token >= vocab first. */
+ * (APK_DECLINE_RANGE), as the reference's callers reject token >= vocab first.  One id (a decode
+ * step whose sampler runs on the host) travels as a kernel argument; more are staged through a
+ * pinned buffer of the context, which waits for the previous use of that buffer. */
 int apk_embed_rows_host_ids(apk_ctx* ctx, int fmt, const void* table, size_t vocab, size_t n_in,
                             const uint32_t* ids_host, size_t t, void* out, int out_dtype);
 /* The rows [row0, row0 + count) of a quantized matrix of n_rows rows, dequantized in place of a
