@@ -314,6 +314,32 @@ class Backend:
             return table, tok, tok_off, hit_row, hit_w
         return table[: int(n_used.item())], tok, tok_off, hit_row, hit_w
 
+    def route_group(self, logits, k, n_expert=None, gating=Gating.Softmax, norm=True, scale=1.0, bias=None):
+        """route_rows then moe_permute with the same results; one launch for a decode-sized batch
+        (the router and the grouping of Ffn::moe_batch, moe.rs:204-271, :298-309).
+        Returns (ids, w), (table, tok, tok_off, hit_row, hit_w)."""
+        rows, n = logits.shape
+        n_expert = n if n_expert is None else n_expert
+        k = min(k, n)
+        dev = self.device
+        assert logits.dtype == torch.float32 and n_expert == n
+        ids = torch.empty((rows, k), dtype=torch.int32, device=dev)
+        w = torch.empty((rows, k), dtype=torch.float32, device=dev)
+        table = torch.zeros((n_expert, 3), dtype=torch.int32, device=dev)
+        n_used = torch.zeros(1, dtype=torch.int32, device=dev)
+        tok = torch.empty(rows * k, dtype=torch.int32, device=dev)
+        tok_off = torch.empty(rows + 1, dtype=torch.int32, device=dev)
+        hit_row = torch.empty(rows * k, dtype=torch.int32, device=dev)
+        hit_w = torch.empty(rows * k, dtype=torch.float32, device=dev)
+        self._enter()
+        check(self.L.apk_route_group(self.h, _ptr(logits), _ptr(bias), rows, n_expert, k, int(norm), scale,
+                                     int(gating == Gating.Sigmoid), _ptr(ids), _ptr(w), _ptr(table), _ptr(n_used), _ptr(tok),
+                                     _ptr(tok_off), _ptr(hit_row), _ptr(hit_w)))
+        self._leave()
+        if self._recording:
+            return (ids, w), (table, tok, tok_off, hit_row, hit_w)
+        return (ids, w), (table[: int(n_used.item())], tok, tok_off, hit_row, hit_w)
+
     def gather_rows(self, src, tok):
         """xe rows in tok order (moe.rs:348-352)."""
         total = tok.numel()

@@ -65,7 +65,8 @@ std::vector<std::string> all_kernel_names() {
     std::vector<std::string> v = {"apk_swiglu_f32", "apk_swiglu_f16", "apk_rope_table", "apk_embed_q4k_f32",
                                   "apk_embed_q4k_f16", "apk_embed_q8_0_f32", "apk_embed_q8_0_f16", "apk_route_topk",
                                   "apk_moe_permute", "apk_gather_rows", "apk_scatter_rows_t1", "apk_scatter_rows_t2", "apk_argmax_rows", "apk_add_rmsnorm_ragged_f32", "apk_add_rmsnorm_ragged_f16", "apk_copy",
-                                  "apk_qknorm_rope_generic_f32", "apk_qknorm_rope_generic_f16", "apk_route_topk_wide", "apk_route_topk_e64", "apk_route_topk_e128", "apk_add_assign_f32", "apk_add_assign_f16", "apk_softmax_rows", "apk_moe_count", "apk_moe_rank"};
+                                  "apk_qknorm_rope_generic_f32", "apk_qknorm_rope_generic_f16", "apk_route_topk_wide", "apk_route_topk_e64", "apk_route_topk_e128", "apk_route_group_small_e64", "apk_route_group_small_e128",
+                                  "apk_route_group_small_e256", "apk_route_group_small_e1024", "apk_add_assign_f32", "apk_add_assign_f16", "apk_softmax_rows", "apk_moe_count", "apk_moe_rank"};
     for (const char* t : {"f32", "f16"}) {
         for (const char* f : {"q5k", "q6k", "q2k", "q3k", "q5_0", "f16", "f32", "bf16"}) v.push_back(std::string("apk_embed_") + f + "_" + t);
         for (int c : kAddnormTiles) v.push_back(std::string("apk_add_rmsnorm_") + t + "_c" + std::to_string(c));
@@ -1063,6 +1064,29 @@ int apk_moe_permute(apk_ctx* c, const uint32_t* ids, const float* w, size_t rows
     if (int rc = launch(c, "apk_moe_count", (unsigned)parts, 512, 0, cargs)) return rc;
     void* rargs[] = {&ids, &w, &rows_i, &k_i, &ne_i, &parts_i, &c->permute_counts, &table, &n_used, &tok, &tok_off, &hit_row, &hit_w};
     return launch(c, "apk_moe_rank", (unsigned)(n_expert * parts), 512, 0, rargs);
+}
+
+int apk_route_group(apk_ctx* c, const float* logits, const float* bias, size_t rows, size_t n_expert, size_t k, int norm,
+                    float scale, int sigmoid, uint32_t* ids, float* w, uint32_t* table, uint32_t* n_used, uint32_t* tok,
+                    uint32_t* tok_off, uint32_t* hit_row, float* hit_w) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_route_group: ctx is NULL");
+    if (n_expert == 0 || n_expert > 1024) return fail(APK_DECLINE_UNSUPPORTED, "apk_route_group: n_expert %zu (1..1024)", n_expert);
+    if (k == 0 || k > n_expert || k > 64) return fail(APK_DECLINE_UNSUPPORTED, "apk_route_group: k %zu", k);
+    if (!table || !n_used || !tok_off) return fail(APK_DECLINE_NULL, "apk_route_group: NULL tensor");
+    if (rows && (!logits || !ids || !w || !tok || !hit_row || !hit_w)) return fail(APK_DECLINE_NULL, "apk_route_group: NULL tensor");
+    if (rows == 0 || rows > 16) {
+        // beyond a decode-sized batch the two launches are bound by their work, not by the launch:
+        // the same results from the two entries (every decline is theirs; nothing above can fail below)
+        if (int rc = apk_route_topk(c, logits, bias, rows, n_expert, k, norm, scale, sigmoid, ids, w)) return rc;
+        return apk_moe_permute(c, ids, w, rows, k, n_expert, table, n_used, tok, tok_off, hit_row, hit_w);
+    }
+    CallScope s(c);
+    if (int rc = set_device(c)) return rc;
+    int rows_i = (int)rows, ne_i = (int)n_expert, k_i = (int)k;
+    void* args[] = {&logits, &bias, &rows_i, &ne_i, &k_i, &norm, &scale, &sigmoid, &ids, &w, &table, &n_used, &tok, &tok_off, &hit_row, &hit_w};
+    const char* which = n_expert <= 64 ? "apk_route_group_small_e64" : n_expert <= 128 ? "apk_route_group_small_e128"
+                      : n_expert <= 256 ? "apk_route_group_small_e256" : "apk_route_group_small_e1024";
+    return launch(c, which, 1, 1024, 0, args);
 }
 
 int apk_gather_rows(apk_ctx* c, const void* src, const uint32_t* tok, size_t src_rows, size_t total_rows, size_t cols,

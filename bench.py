@@ -397,6 +397,15 @@ def other_shapes(args, L, h, apklib, synth, torch, gen, dev, randn, pool, p, tim
     us = timed(lambda i: check(L.apk_moe_permute(h, p(ids_m), p(w_m), TM, K, NE, p(tbl), p(n_used), p(tok), p(tok_off),
                                                  p(hit_row), p(hit_w))), 200)
     record("moe_permute (tables)", tagm, us, TM * K * 8 + TM * K * 12 + TM * 4, note="launch-bound")
+    # a decode step of the same router: one token, router and grouping as two launches and as one
+    def two_launches(i):
+        check(L.apk_route_topk(h, p(logits[i % 8]), None, 1, NE, K, 1, 1.0, 0, p(ids_m), p(w_m)))
+        check(L.apk_moe_permute(h, p(ids_m), p(w_m), 1, K, NE, p(tbl), p(n_used), p(tok), p(tok_off), p(hit_row), p(hit_w)))
+    us = timed(two_launches, 200)
+    record("route_topk + moe_permute (two launches)", "qwen3-30b-a3b decode T=1 f32", us, NE * 4 + K * 28 + 8, launches=2, note="launch-bound")
+    us = timed(lambda i: check(L.apk_route_group(h, p(logits[i % 8]), None, 1, NE, K, 1, 1.0, 0, p(ids_m), p(w_m), p(tbl), p(n_used),
+                                                 p(tok), p(tok_off), p(hit_row), p(hit_w))), 200)
+    record("route_group (router + grouping, one launch)", "qwen3-30b-a3b decode T=1 f32", us, NE * 4 + K * 28 + 8, note="launch-bound")
     us = timed(lambda i: check(L.apk_gather_rows(h, p(ga[i % len(ga)]["hs"]), p(tok), TM, TM * K, HM, p(ga[i % len(ga)]["xe"]), F32)), reps)
     record("gather_rows (permute, row-side)", tagm, us, TM * HM * 4 + TM * K * HM * 4 + TM * K * 4)
     us = timed(lambda i: check(L.apk_scatter_rows(h, p(ga[i % len(ga)]["hs"]), p(hit_row), TM, K, TM * K, HM, p(ga[i % len(ga)]["xe"]), F32)), reps)

@@ -295,6 +295,16 @@ int apk_moe_permute(apk_ctx* ctx, const uint32_t* ids, const float* w, size_t ro
                     uint32_t* table, uint32_t* n_used, uint32_t* tok, uint32_t* tok_off, uint32_t* hit_row,
                     float* hit_w);
 
+/* apk_route_topk followed by apk_moe_permute, with the same arguments and the same results bit for
+ * bit; ONE launch for a decode-sized batch (rows <= 16), where the two launches
+ * cost a launch latency each and the second waits for the first.  The reference's accelerators route
+ * and group inside one command buffer as well (GroupedRoute of a GroupedFfnReq, gpu/types.rs:406-416,
+ * :446-467; the Metal route_scatter kernel, gpu/shaders/kernels.metal:2223).  Larger batches run the
+ * two entries. */
+int apk_route_group(apk_ctx* ctx, const float* logits, const float* bias, size_t rows, size_t n_expert, size_t k,
+                    int norm, float scale, int sigmoid, uint32_t* ids, float* w, uint32_t* table, uint32_t* n_used,
+                    uint32_t* tok, uint32_t* tok_off, uint32_t* hit_row, float* hit_w);
+
 /* dst[r,:] = src[tok[r],:] -- the gathered expert activations (model/moe.rs:348-352).
  * src: [src_rows][cols], dst: [total_rows][cols] of dtype; cols*sizeof(dtype) must
  * be a multiple of 16. */

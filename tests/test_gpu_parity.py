@@ -813,6 +813,37 @@ def test_route_reference_vectors_ties_sigmoid_bias(be, ora):
         be.route_gated(dev(np.zeros(1025, np.float32)), 4)
 
 
+@pytest.mark.parametrize("rows,n_expert,k", [(1, 128, 8), (6, 128, 8), (16, 128, 8), (16, 64, 6), (13, 256, 8), (16, 1024, 64), (5, 512, 10),
+                                            (16, 16, 16), (1, 4, 4), (15, 60, 3), (9, 128, 16), (12, 1000, 25), (2, 64, 64), (16, 65, 1),
+                                            # beyond one launch: the two entries run
+                                            (17, 128, 8), (64, 128, 8), (300, 24, 5)])
+@pytest.mark.parametrize("gating", ["softmax", "sigmoid_bias"])
+def test_route_group_equals_router_then_grouping(be, ora, rows, n_expert, k, gating):
+    """The one-launch router + grouping of a decode-sized batch against the oracle, and bit for bit against
+    apk_route_topk followed by apk_moe_permute."""
+    import allpaka_amd as apk
+
+    s = synth()
+    g = s.rng(4, rows * 131 + n_expert + k)
+    logits = s.normal_f32(g, (rows, n_expert))
+    if n_expert > 8:
+        logits[:, n_expert // 3] = -60.0  # an expert nobody picks (k < n_expert - 1 in these cases)
+    bias = s.normal_f32(g, n_expert, 0.0, 0.01) if gating == "sigmoid_bias" else None
+    kind = apk.Gating.Sigmoid if bias is not None else apk.Gating.Softmax
+    args = dict(gating=kind, norm=True, scale=1.25, bias=None if bias is None else dev(bias))
+    (ids, w), got = be.route_group(dev(logits), k, **args)
+    ids2, w2 = be.route_rows(dev(logits), k, **args)
+    want = be.moe_permute(ids2, w2, n_expert)
+    assert torch.equal(ids, ids2) and torch.equal(w, w2)
+    for name, a, b in zip(["table", "tok", "tok_off", "hit_row", "hit_w"], got, want):
+        assert a.shape == b.shape and torch.equal(a, b), name
+    o_ids, o_w = ora.route_rows(logits, k, ora.SIGMOID if bias is not None else ora.SOFTMAX, True, 1.25, bias, threads=4)
+    assert np.array_equal(host(ids), o_ids) and rel_err_f32(host(w), o_w) <= TOL_F32
+    for name, a, b in zip(["table", "tok", "tok_off", "hit_row"], got, ora.moe_group(o_ids, o_w, n_expert)):
+        assert np.array_equal(host(a), b), name
+    assert be.take_faults() == 0
+
+
 # ------------------------------------------------------- grouping and gather
 @pytest.mark.parametrize("rows,k,n_expert", [(1024, 8, 128), (1, 8, 128), (5, 2, 4), (600, 8, 16), (64, 1, 256), (777, 3, 7), (2048, 8, 128),
                                              # beyond 2048 tokens: the two-launch form (parts of 1024 tokens)

@@ -361,3 +361,29 @@ def test_grouping_scratch_cannot_move_under_a_graph(be, ora):
         assert b2.moe_permute(big_ids, dev(np.ones((9000, 4), np.float32)), ne)[1].numel() == 36000
     finally:
         b2.close()
+
+
+def test_recorded_router_and_grouping_follow_the_logits_of_every_replay(be, ora):
+    """The one-launch router + grouping of a decode step inside a recording: one node, and every replay
+    routes the logits that are in the buffer at that time."""
+    from allpaka_amd import synth as s
+
+    rows, ne, k = 4, 128, 8
+    logits = torch.zeros((rows, ne), device="cuda")
+    with be.record() as rec:
+        (ids, w), outs = be.route_group(logits, k)
+    assert rec.graph.nodes == 1
+    for step in range(4):
+        fresh = s.normal_f32(s.rng(4, 700 + step), (rows, ne))
+        logits.copy_(dev(fresh))
+        for t in (ids, w) + tuple(outs):
+            t.zero_()
+        be.swiglu(torch.ones(64, device="cuda"), torch.ones(64, device="cuda"))  # unrecorded work in between
+        rec.graph.launch()
+        be.sync()
+        o_ids, o_w = ora.route_rows(fresh, k, threads=2)
+        assert np.array_equal(host(ids), o_ids) and rel_err_f32(host(w), o_w) <= 1e-5
+        want = ora.moe_group(o_ids, host(w), ne)  # grouped with the device's own weights: bit for bit
+        for name, a, b in zip(["table", "tok", "tok_off", "hit_row", "hit_w"], outs, want):
+            assert np.array_equal(host(a)[: b.shape[0]].view(np.uint32), b.view(np.uint32)), (step, name)
+    rec.graph.destroy()
