@@ -1106,7 +1106,10 @@ int apk_gather_rows(apk_ctx* c, const void* src, const uint32_t* tok, size_t src
     int row_vecs = (int)(cols * es / 16);
     uint32_t total32 = (uint32_t)total_rows;
     void* args[] = {&src, &tok, &src_rows32, &total32, &row_vecs, &dst, &c->fault_dev};
-    return launch(c, "apk_gather_rows", (unsigned)((total_rows + 3) / 4), 256, 0, args);  // 4 rows per workgroup
+    // groups of 32 destination rows, eight workgroups per group (one per XCD)
+    const uint64_t grid = (total_rows + 31) / 32 * 8;
+    if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_gather_rows: too large");
+    return launch(c, "apk_gather_rows", (unsigned)grid, 256, 0, args);
 }
 
 int apk_scatter_rows(apk_ctx* c, const void* src, const uint32_t* hit_row, size_t rows, size_t k, size_t total_rows,

@@ -1917,44 +1917,30 @@ extern "C" __global__ __launch_bounds__(APK_PERMUTE_THREADS) void apk_moe_rank(
 }
 
 // Gathered activations in tok order (moe.rs:348-352): dst[r,:] = src[tok[r],:].
-// One workgroup per APK_GATHER_ROWS destination rows, 16-byte tiles; row_vecs = row bytes / 16.
-// The source row numbers of the group are read first (uniform for the workgroup), then the
-// tiles of all its rows are in flight together: one index latency per group, not per row.
-#define APK_GATHER_ROWS 4
+// Every source row is wanted k times, by destination rows that lie far apart (one per expert that the
+// token picked).  Taken in destination order the k reads of a row come from any of the 8 XCDs, each with
+// an L2 of its own, and the row crosses the fabric up to 8 times (T=4096, 2048 f32 columns: 75 us).  Here
+// workgroup b runs on XCD b % 8 and takes, of the 32 destination rows of group b / 8, those whose SOURCE
+// row number is b % 8 modulo 8: a source row is then only ever read through one L2, which holds that
+// XCD's eighth of the source for batches of a few thousand tokens (53 us; the token-side scatter 44 us).
+#define APK_GATHER_GROUP 32
 extern "C" __global__ __launch_bounds__(256) void apk_gather_rows(const u32x4* src, const uint32_t* tok,
                                                                  uint32_t src_rows, uint32_t total_rows, int row_vecs,
                                                                  u32x4* dst, uint32_t* fault) {
-    const uint32_t r0 = blockIdx.x * APK_GATHER_ROWS;
-    uint32_t s[APK_GATHER_ROWS];
-    bool ok[APK_GATHER_ROWS];
-    bool bad = false;
-#pragma unroll
-    for (int j = 0; j < APK_GATHER_ROWS; j++) {
-        const bool in = r0 + j < total_rows;
-        s[j] = tok[min(r0 + (uint32_t)j, total_rows - 1u)];
-        ok[j] = in && s[j] < src_rows;
-        bad |= in && s[j] >= src_rows;
-        s[j] = s[j] < src_rows ? s[j] : 0u;
-    }
-    if (bad && threadIdx.x == 0) atomicOr(fault, APK_FAULT_ROW_RANGE);
-    for (int c = threadIdx.x; c < row_vecs; c += 2 * blockDim.x) {
-        const int c2 = c + blockDim.x;
-        const bool two = c2 < row_vecs;
-        u32x4 a[APK_GATHER_ROWS], b[APK_GATHER_ROWS];
-#pragma unroll
-        for (int j = 0; j < APK_GATHER_ROWS; j++) {
-            const u32x4* sp = src + (uint64_t)s[j] * row_vecs;
-            a[j] = sp[c];
-            b[j] = sp[two ? c2 : c];
-        }
-#pragma unroll
-        for (int j = 0; j < APK_GATHER_ROWS; j++) {
-            if (ok[j]) {  // uniform
-                u32x4* dp = dst + (uint64_t)(r0 + j) * row_vecs;
-                __builtin_nontemporal_store(a[j], dp + c);
-                if (two) __builtin_nontemporal_store(b[j], dp + c2);
-            }
-        }
+    const uint32_t xcd = blockIdx.x & 7u, r0 = (blockIdx.x >> 3) * APK_GATHER_GROUP;
+    const int lane = threadIdx.x & 63;
+    const uint32_t r = r0 + (uint32_t)lane;
+    const bool mine_to_check = lane < APK_GATHER_GROUP && r < total_rows;
+    const uint32_t t = mine_to_check ? tok[r] : 0u;
+    const bool mine = mine_to_check && (t & 7u) == xcd;
+    if (__ballot(mine && t >= src_rows) != 0 && threadIdx.x == 0) atomicOr(fault, APK_FAULT_ROW_RANGE);
+    uint64_t m = __ballot(mine && t < src_rows);  // the same in every wave of the workgroup
+    while (m) {
+        const int j = __builtin_ctzll(m);
+        m &= m - 1;
+        const u32x4* sp = src + (uint64_t)__shfl(t, j, 64) * row_vecs;
+        u32x4* dp = dst + (uint64_t)(r0 + (uint32_t)j) * row_vecs;
+        for (int c = threadIdx.x; c < row_vecs; c += blockDim.x) __builtin_nontemporal_store(sp[c], dp + c);
     }
 }
 
