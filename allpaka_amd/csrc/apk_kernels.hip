@@ -869,8 +869,7 @@ DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const fl
     const int lane = threadIdx.x & 63;
     const int l = lane % LPH, sub = lane / LPH;
     const int gq = (n_q + HPW * ITERQ - 1) / (HPW * ITERQ), gk = (n_kv + HPW - 1) / HPW;
-    // all q items first (the long ones), then the k items: the k waves, one pass each,
-    // fill in behind the resident round of q waves instead of delaying part of it
+    // all q items first (the longer ones, up to two passes), then the k items, one pass each
     const uint64_t wid = ((uint64_t)vblock * blockDim.x + threadIdx.x) >> 6;
     const uint64_t nq_items = (uint64_t)rows * gq;
     if (wid >= nq_items + (uint64_t)rows * gk) return;  // whole wave
