@@ -185,6 +185,14 @@ class Backend:
         check(self.L.apk_add_rmsnorm_rows(self.h, _ptr(x), _ptr(delta), _ptr(h), _ptr(gamma), n, rows, eps, _dt(x)))
         self._leave()
 
+    def rope_inv_freq(self, rot_dim, base):
+        """ops::rope_inv_freq (rope.rs:8-12): the f32 inverse frequencies, computed on the host, as a device tensor."""
+        import numpy as np
+
+        inv = np.empty(rot_dim // 2, np.float32)
+        check(self.L.apk_rope_inv_freq(rot_dim, base, inv.ctypes.data))
+        return torch.from_numpy(inv).to(self.device)
+
     def rope_table(self, positions, inv_freq):
         """ops::rope_sin_cos per position -> [rows, half, 2] = [sin, cos] (rope.rs:18-22)."""
         rows, half = positions.numel(), inv_freq.numel()

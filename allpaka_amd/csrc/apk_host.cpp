@@ -13,6 +13,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
+#include <cmath>
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -906,6 +907,12 @@ int apk_layer_prologue(apk_ctx* c, void* x, const void* delta, void* h, const fl
     return launch_keyed(c, OP_PROLOGUE, (uint32_t)dtype << 16 | (uint32_t)head_dim,
                         [&] { return std::string("apk_layer_prologue_") + (dtype == APK_F32 ? "f32" : "f16") + "_hd" + std::to_string(head_dim); },
                         (unsigned)grid, (unsigned)threads, 0, args);
+}
+
+int apk_rope_inv_freq(size_t rot_dim, float base, float* inv_freq) {
+    if (rot_dim >= 2 && !inv_freq) return fail(APK_DECLINE_NULL, "apk_rope_inv_freq: inv_freq is NULL");
+    for (size_t i = 0; i < rot_dim / 2; i++) inv_freq[i] = powf(base, -2.0f * (float)i / (float)rot_dim);
+    return APK_OK;
 }
 
 int apk_rope_table(apk_ctx* c, const uint32_t* positions, const float* inv_freq, size_t rows, size_t half, float* table) {

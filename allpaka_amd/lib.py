@@ -68,6 +68,7 @@ SYMBOLS = {
     "apk_moe_combine_add_rmsnorm": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _sz, _sz, _f, _i]),
     "apk_argmax_rows": (_i, [_vp, _vp, _sz, _sz, _vp]),
     "apk_copy": (_i, [_vp, _vp, _vp, _sz]),
+    "apk_rope_inv_freq": (_i, [_sz, _f, _vp]),
     "apk_route_group": (_i, [_vp, _vp, _vp, _sz, _sz, _sz, _i, _f, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "apk_plan_add_rmsnorm_rows": (_i, [_sz, _sz, _i, _plan]),
     "apk_plan_qknorm_rope": (_i, [_sz, _sz, _sz, _sz, _sz, _i, _i, _i, _plan]),

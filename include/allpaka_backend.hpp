@@ -126,8 +126,13 @@ inline void add_assign_then_rmsnorm_into(std::vector<float>& a, const std::vecto
     std::copy(out.begin(), out.end(), h.begin());
 }
 
-// ops::rope_inv_freq / rope_sin_cos (rope.rs:8-22) stay host-side one-liners in the reference; the table rows
-// for a batch of positions can be built on the device:
+// ops::rope_inv_freq(head_dim, base) (rope.rs:8-12): host-side, as in the reference.
+inline std::vector<float> rope_inv_freq(size_t head_dim, float base) {
+    std::vector<float> inv(head_dim / 2);
+    check(apk_rope_inv_freq(head_dim, base, inv.data()));
+    return inv;
+}
+// ops::rope_sin_cos (rope.rs:18-22) per position; the table rows for a batch of positions are built on the device:
 inline std::vector<std::array<float, 2>> rope_sin_cos_rows(const std::vector<uint32_t>& positions, const std::vector<float>& inv_freq) {
     Dev<uint32_t> dp(positions.data(), positions.size());
     Dev<float> di(inv_freq.data(), inv_freq.size()), dt(positions.size() * inv_freq.size() * 2);

@@ -263,6 +263,11 @@ int apk_layer_prologue(apk_ctx* ctx, void* x, const void* delta, void* h, const 
                        void* k, const float* qw, const float* kw, const float* rope, size_t rows, size_t n_q,
                        size_t n_kv, size_t head_dim, size_t rot_dim, float eps, int dtype);
 
+/* inv_freq[i] = base.powf(-2 i / rot_dim) for i < rot_dim / 2, in f32 on the host: ops::rope_inv_freq
+ * (ops/rope.rs:8-12), which the reference computes once at load with the platform's powf -- the
+ * same libm symbol this uses.  No context, no GPU. */
+int apk_rope_inv_freq(size_t rot_dim, float base, float* inv_freq);
+
 /* Builds RoPE table rows on the device: table[r][i] = [sin, cos](pos[r] as f32 *
  * inv_freq[i]).  Replaces ops::rope_sin_cos per position (ops/rope.rs:18-22;
  * Session::ensure_rope_cache, model/session.rs:34-50; gpu::multi_stage's staging

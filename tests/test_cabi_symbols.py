@@ -90,3 +90,19 @@ def test_package_has_no_cpu_fallback_and_never_touches_the_oracle():
             if f.endswith((".py", ".cpp", ".hip", ".h", ".S")):
                 src = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in src.lower().replace("no oracle", ""), f"{f} mentions the oracle"
+
+
+def test_rope_inv_freq_is_the_reference_powf_series():
+    """ops::rope_inv_freq (ops/rope.rs:8-12) on the host: base^(-2i/d) in f32 with libm's powf, the oracle's
+    series bit for bit; the reference's own checks: inv[0] == 1, strictly decreasing (ops/mod.rs:250-257)."""
+    import numpy as np
+
+    import oracle as ora
+
+    lib, L = _lib()
+    for d, base in ((128, 1e6), (64, 1e4), (256, 1e6), (96, 5e5), (2, 10.0)):
+        inv = np.zeros(d // 2, np.float32)
+        assert L.apk_rope_inv_freq(d, base, inv.ctypes.data) == 0
+        assert np.array_equal(inv.view(np.uint32), ora.rope_inv_freq(d, base).view(np.uint32))
+        assert inv[0] == 1.0 and np.all(np.diff(inv) < 0)
+    assert L.apk_rope_inv_freq(0, 1e4, None) == 0 and L.apk_rope_inv_freq(8, 1e4, None) == 3
