@@ -1,0 +1,113 @@
+// gfx950 device code, part of apk_kernels.hip (one translation unit, one code object): SwiGLU, residual add, row softmax.
+#pragma once
+
+// =========================================================================
+// SwiGLU: gate[i] = silu(gate[i]) * up[i], silu(x) = x / (1 + exp(-x))
+// (activation.rs:19-22, :116-119).  Pure stream: 2 reads + 1 write / element.
+// =========================================================================
+template <typename T> DEV float silu_mul(float g, float u);
+// f32 activations: exp(-g) by Cody-Waite reduction around the hardware exp2 (log2(e) carried in
+// two parts, so the reduced argument is exact to the last bit: about 1 ulp over the whole range,
+// where a bare exp2(-g*log2e) loses |g| ulps), then the hardware reciprocal (1 ulp): the result is
+// within a few ulp of the reference's g / (1 + exp(-g)) * u -- 1e-6 of the 1e-5 bar -- at a third
+// of the instructions of libm expf + IEEE division, which at 32 per element no longer hid behind
+// the stream.
+template <> __device__ __forceinline__ float silu_mul<float>(float g, float u) {
+    const float L2E_HI = 1.44269502162933349609375f, L2E_LO = 1.925963033500011e-08f;  // hi + lo = log2(e)
+    const float n = fminf(fmaxf(-g, -104.0f), 89.0f);  // beyond: e underflows to 0 / overflows to inf anyway
+    const float k = __builtin_rintf(n * L2E_HI);
+    float r = __builtin_fmaf(n, L2E_HI, -k);
+    r = __builtin_fmaf(n, L2E_LO, r);
+    const float e = __builtin_amdgcn_ldexpf(__builtin_amdgcn_exp2f(r), (int)k);
+    // the hardware reciprocal flushes subnormal results: keep 1/(1+e) normal for e up to FLT_MAX by
+    // taking it of (1+e) * 2^-32 and applying the 2^-32 after the multiplication by g (all exact)
+    const float sc = e > 0x1p96f ? 0x1p-32f : 1.0f;
+    return g * __builtin_amdgcn_rcpf((1.0f + e) * sc) * sc * u;  // NaN in g still gives NaN
+}
+// fp16 activations: the result is rounded to 11 bits, so the hardware exp2 /
+// rcp approximations (about 1 ulp of f32 each) are far inside the 2-ulp-of-fp16
+// budget and keep the kernel under its ALU ceiling.
+template <> __device__ __forceinline__ float silu_mul<f16_t>(float g, float u) {
+    float e = __builtin_amdgcn_exp2f(g * -1.4426950408889634f);
+    return g * __builtin_amdgcn_rcpf(1.0f + e) * u;
+}
+
+template <typename T, int UNR> DEV void swiglu_body(T* gate, const T* up, uint64_t n) {
+    constexpr int VEC = io<T>::VEC;
+    const uint64_t nvec = n / VEC;
+    const uint64_t base = (uint64_t)blockIdx.x * (blockDim.x * UNR) + threadIdx.x;
+    float g[UNR][VEC], u[UNR][VEC];
+#pragma unroll
+    for (int j = 0; j < UNR; j++) {
+        uint64_t c = base + (uint64_t)j * blockDim.x;
+        if (c < nvec) {
+            io<T>::load_nt(gate + c * VEC, g[j]);
+            io<T>::load_nt(up + c * VEC, u[j]);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < UNR; j++) {
+        uint64_t c = base + (uint64_t)j * blockDim.x;
+        if (c < nvec) {
+#pragma unroll
+            for (int i = 0; i < VEC; i++) g[j][i] = silu_mul<T>(g[j][i], u[j][i]);
+            io<T>::store_nt(gate + c * VEC, g[j]);
+        }
+    }
+    // ragged tail (n not a multiple of the 16-byte tile): last block, scalar
+    if (blockIdx.x == gridDim.x - 1) {
+        for (uint64_t i = nvec * VEC + threadIdx.x; i < n; i += blockDim.x)
+            gate[i] = (T)silu_mul<T>((float)gate[i], (float)up[i]);
+    }
+}
+#define APK_SWIGLU_UNR 1  // measured: 1 tile per lane streams best (most waves in flight)
+extern "C" __global__ __launch_bounds__(256) void apk_swiglu_f32(float* gate, const float* up, uint64_t n) {
+    swiglu_body<float, APK_SWIGLU_UNR>(gate, up, n);
+}
+extern "C" __global__ __launch_bounds__(256) void apk_swiglu_f16(f16_t* gate, const f16_t* up, uint64_t n) {
+    swiglu_body<f16_t, APK_SWIGLU_UNR>(gate, up, n);
+}
+
+// Residual add on its own: a[i] += b[i] (ops::add_assign_slice, blas.rs:105-178), for the
+// places where no norm follows.  One 16-byte tile per lane, a scalar tail for ragged n.
+template <typename T> DEV void add_assign_body(T* a, const T* b, uint64_t n) {
+    constexpr int VEC = io<T>::VEC;
+    const uint64_t nvec = n / VEC, c = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c < nvec) {
+        float x[VEC], y[VEC];
+        io<T>::load_nt(a + c * VEC, x);
+        io<T>::load_nt(b + c * VEC, y);
+#pragma unroll
+        for (int i = 0; i < VEC; i++) x[i] += y[i];
+        io<T>::store_nt(a + c * VEC, x);
+    }
+    if (blockIdx.x == gridDim.x - 1)
+        for (uint64_t i = nvec * VEC + threadIdx.x; i < n; i += blockDim.x) a[i] = (T)((float)a[i] + (float)b[i]);
+}
+extern "C" __global__ __launch_bounds__(256) void apk_add_assign_f32(float* a, const float* b, uint64_t n) {
+    add_assign_body<float>(a, b, n);
+}
+extern "C" __global__ __launch_bounds__(256) void apk_add_assign_f16(f16_t* a, const f16_t* b, uint64_t n) {
+    add_assign_body<f16_t>(a, b, n);
+}
+
+// Softmax over rows in place (ops::softmax, activation.rs:5-16): max, exp(v - max), sum,
+// times 1/sum.  A wave per row, any row length; the sum runs in lane order, not index order.
+extern "C" __global__ __launch_bounds__(256) void apk_softmax_rows(float* x, int rows, int n) {
+    const int lane = threadIdx.x & 63;
+    const uint64_t r = ((uint64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    if (r >= (uint64_t)rows) return;  // whole wave
+    float* row = x + r * (uint64_t)n;
+    float mx = -INFINITY;
+    for (int i = lane; i < n; i += 64) mx = fmaxf(mx, row[i]);
+    mx = wave_max_f32(mx);
+    float sum = 0.0f;
+    for (int i = lane; i < n; i += 64) {
+        const float e = expf(row[i] - mx);
+        row[i] = e;
+        sum += e;
+    }
+    sum = group_sum<64>(sum);
+    const float inv = 1.0f / sum;
+    for (int i = lane; i < n; i += 64) row[i] *= inv;  // each lane re-reads only what it wrote
+}

@@ -1,0 +1,253 @@
+// gfx950 device code, part of apk_kernels.hip (one translation unit, one code object): per-head QK-norm + RoPE, K/V cache store, layer prologue, rotary table.
+#pragma once
+
+// =========================================================================
+// Per-head QK-norm + NeoX RoPE, in place on q [rows, n_q*HD] and k [rows, n_kv*HD]
+// (caller loop attention.rs:131-165: rmsnorm(head, w, eps) then the NeoX
+// rotation with the row's [sin, cos] table, rope.rs:70-81).
+// Lane mapping: a lane holds one 16-byte tile of the first half of a head and
+// the tile of its NeoX partners in the second half (EPL = 8 fp16 / 4 f32
+// elements each), so the rotation needs no cross-lane traffic, every global
+// access is a full 16-byte tile and the LPH = HD/2/EPL lanes of a head cover
+// contiguous runs.  A wave owns (row, q or k, group of HPW*ITER consecutive
+// heads), HPW = 64/LPH heads per pass: one tensor per wave means one norm
+// weight per wave and no per-element selects; the row's [sin, cos] tile and
+// the weight are loaded once and reused over ITER passes (q: ITERQ passes,
+// k: 1 pass -- under GQA k has few heads).  Waves are kept short (ITERQ 1 or 2, about
+// 4 KB of heads each): a wave that carries a row's 64 q heads in 8 passes lives as long as
+// the whole launch, and a batch a few rows beyond one resident round of such waves
+// (2061 rows instead of 2048) then takes 15 % longer; short waves fill in evenly.
+// Arithmetic: the reference's, for both activation types (see `headstat`): f64 statistics,
+// (x as f64 * scale) as f32 * w, then the four products and two sums of the rotation,
+// not contracted.  fp16 results are that f32 result rounded once.
+// =========================================================================
+// KV = true (k items only): the rotated k tiles are also narrowed to fp16 into the cache row
+// kc, and the same tiles of the row's v are narrowed into vc (KvCache::store_at,
+// crates/allpaka-model/src/kv.rs:682-697: k and v rows as f16 at pos*kv_dim).
+template <typename T, int HD, int ITER, bool KV = false>
+DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, float eps, int l, int sub,
+                 f16_t* kc = nullptr, const T* vrow = nullptr, f16_t* vc = nullptr) {
+    constexpr int EPL = io<T>::VEC;   // elements per lane per half
+    constexpr int HALF = HD / 2;
+    constexpr int LPH = HALF / EPL;   // lanes per head
+    constexpr int HPW = 64 / LPH;     // heads per wave pass
+    typedef typename headstat<T>::acc_t acc_t;
+    // Loads return in issue order, so the small cached ones go first and the first pass
+    // can start as soon as its own two tiles arrive.  No branch, no conversion here: a
+    // lane of a pass beyond the last head re-reads the last head and stores nothing; a
+    // missing norm weight is read from the [sin, cos] tile instead and never used.
+    float sc[2 * EPL], wa[EPL], wb[EPL];
+#pragma unroll
+    for (int i = 0; i < 2 * EPL; i += 4) io<float>::load(trow + 2 * EPL * l + i, sc + i);
+    const float* wp = w ? w : trow;
+#pragma unroll
+    for (int i = 0; i < EPL; i += 4) {
+        io<float>::load(wp + EPL * l + i, wa + i);
+        io<float>::load(wp + HALF + EPL * l + i, wb + i);
+    }
+    typename io<T>::raw_t araw[ITER], braw[ITER], varaw[ITER], vbraw[ITER];
+    // head of pass `it` and its element offset: recomputed where needed (a few integer
+    // operations) rather than kept in registers across the loads
+    const int hh_first = g * ITER * HPW + sub;
+    auto head_off = [&](int it) { return min(hh_first + it * HPW, nheads - 1) * HD + EPL * l; };
+#pragma unroll
+    for (int it = 0; it < ITER; it++) {
+        const int off = head_off(it);
+        __builtin_amdgcn_sched_barrier(0);  // loads stay in program order (returns are in order)
+        araw[it] = io<T>::ldraw_nt(base + off);
+        braw[it] = io<T>::ldraw_nt(base + off + HALF);
+        if constexpr (KV) {
+            varaw[it] = io<T>::ldraw_nt(vrow + off);
+            vbraw[it] = io<T>::ldraw_nt(vrow + off + HALF);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);  // every load above; all uses below
+    const bool normed = w != nullptr;  // uniform for the wave
+#pragma unroll
+    for (int it = 0; it < ITER; it++) {
+        float a[EPL], b[EPL], oa[EPL], ob[EPL];
+        io<T>::widen(araw[it], a);
+        io<T>::widen(braw[it], b);
+        acc_t ss = 0;
+#pragma unroll
+        for (int i = 0; i < EPL; i++) {
+            ss = headstat<T>::sq(ss, a[i]);
+            ss = headstat<T>::sq(ss, b[i]);
+        }
+        ss = group_sum<LPH>(ss);
+        const typename headstat<T>::scale_t scale = headstat<T>::rscale(ss, HD, eps);
+#pragma unroll
+        for (int i = 0; i < EPL; i++) {
+            float x = a[i], y = b[i];
+            if (normed) {
+                x = headstat<T>::apply(x, scale, wa[i]);
+                y = headstat<T>::apply(y, scale, wb[i]);
+            }
+            const float s = sc[2 * i], c = sc[2 * i + 1];
+            oa[i] = x * c - y * s;  // not contracted: the reference's four products and two sums
+            ob[i] = x * s + y * c;
+        }
+        const bool live = hh_first + it * HPW < nheads;
+        const int off = head_off(it);
+        if (live) {
+            io<T>::store_nt(base + off, oa);
+            io<T>::store_nt(base + off + HALF, ob);
+        }
+        if constexpr (KV) {
+            if (live && kc != nullptr) {  // kc == nullptr: cache position out of range, row skipped
+                float va[EPL], vb[EPL];
+                io<T>::widen(varaw[it], va);
+                io<T>::widen(vbraw[it], vb);
+                store_f16_tile<T>(kc + off, oa);
+                store_f16_tile<T>(kc + off + HALF, ob);
+                store_f16_tile<T>(vc + off, va);
+                store_f16_tile<T>(vc + off + HALF, vb);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);  // pass by pass: pass it+1 waits only for its own tiles
+    }
+}
+
+template <typename T, int HD, int ITERQ, bool KV = false>
+DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv,
+                          float eps, uint32_t vblock, const T* v = nullptr, const uint32_t* cache_pos = nullptr,
+                          f16_t* k_cache = nullptr, f16_t* v_cache = nullptr, uint32_t capacity = 0,
+                          uint32_t* fault = nullptr) {
+    constexpr int LPH = HD / 2 / io<T>::VEC, HPW = 64 / LPH;
+    const int lane = threadIdx.x & 63;
+    const int l = lane % LPH, sub = lane / LPH;
+    const int gq = (n_q + HPW * ITERQ - 1) / (HPW * ITERQ), gk = (n_kv + HPW - 1) / HPW;
+    // all q items first (the longer ones, up to two passes), then the k items, one pass each
+    const uint64_t wid = ((uint64_t)vblock * blockDim.x + threadIdx.x) >> 6;
+    const uint64_t nq_items = (uint64_t)rows * gq;
+    if (wid >= nq_items + (uint64_t)rows * gk) return;  // whole wave
+    if (wid < nq_items) {
+        const uint64_t row = wid / gq;
+        qk_item<T, HD, ITERQ>(q + row * (uint64_t)n_q * HD, n_q, (int)(wid % gq), qw, rope + row * HD, eps, l, sub);
+    } else {
+        const uint64_t w2 = wid - nq_items, row = w2 / gk;
+        const uint64_t kv_dim = (uint64_t)n_kv * HD;
+        if constexpr (KV) {
+            const uint32_t pos = cache_pos[row];
+            const bool ok = pos < capacity;
+            if (!ok && lane == 0 && w2 % gk == 0) atomicOr(fault, APK_FAULT_CACHE_RANGE);
+            qk_item<T, HD, 1, true>(k + row * kv_dim, n_kv, (int)(w2 % gk), kw, rope + row * HD, eps, l, sub,
+                                    ok ? k_cache + pos * kv_dim : nullptr, v + row * kv_dim,
+                                    ok ? v_cache + pos * kv_dim : nullptr);
+        } else {
+            qk_item<T, HD, 1>(k + row * kv_dim, n_kv, (int)(w2 % gk), kw, rope + row * HD, eps, l, sub);
+        }
+    }
+}
+// At most 128 VGPRs (at least 4 waves per SIMD).
+#define APK_QK_OCC __attribute__((amdgpu_waves_per_eu(4)))
+#define APK_QKROPE(T, TN, HD, ITER)                                                                          \
+    extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void apk_qknorm_rope_##TN##_hd##HD##_i##ITER(   \
+        T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv, float eps) { \
+        qknorm_rope_body<T, HD, ITER>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, blockIdx.x);                  \
+    }
+#define APK_QKROPE_ALL(T, TN)                                                                                          \
+    APK_QKROPE(T, TN, 64, 1) APK_QKROPE(T, TN, 64, 2) APK_QKROPE(T, TN, 128, 1) APK_QKROPE(T, TN, 128, 2)              \
+    APK_QKROPE(T, TN, 256, 1) APK_QKROPE(T, TN, 256, 2)
+APK_QKROPE_ALL(float, f32)
+APK_QKROPE_ALL(f16_t, f16)
+
+// The same with the K/V cache store fused in: rotated k and the row's v narrowed to fp16
+// at cache row cache_pos[row] (one launch instead of QK-norm+RoPE, then two narrowing copies).
+#define APK_QKROPE_KV(T, TN, HD, ITER)                                                                            \
+    extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void apk_qknorm_rope_kv_##TN##_hd##HD##_i##ITER(     \
+        T* q, T* k, const T* v, const float* qw, const float* kw, const float* rope, const uint32_t* cache_pos,  \
+        f16_t* k_cache, f16_t* v_cache, uint32_t capacity, int rows, int n_q, int n_kv, float eps, uint32_t* fault) { \
+        qknorm_rope_body<T, HD, ITER, true>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, blockIdx.x, v, cache_pos,   \
+                                            k_cache, v_cache, capacity, fault);                                   \
+    }
+#define APK_QKROPE_KV_ALL(T, TN)                                                                                       \
+    APK_QKROPE_KV(T, TN, 64, 1) APK_QKROPE_KV(T, TN, 64, 2) APK_QKROPE_KV(T, TN, 128, 1) APK_QKROPE_KV(T, TN, 128, 2)  \
+    APK_QKROPE_KV(T, TN, 256, 1) APK_QKROPE_KV(T, TN, 256, 2)
+APK_QKROPE_KV_ALL(float, f32)
+APK_QKROPE_KV_ALL(f16_t, f16)
+
+// Any other head geometry: head_dim not 64/128/256, a rotary table that covers only the
+// leading rot_half pairs of a head (partial rotary: channels >= 2*rot_half are normalised
+// and pass through, rope.rs:52-81), or the adjacent-pair style (RopeStyle::Norm, pairs
+// (2i, 2i+1), rope.rs:52-64; chosen per model in attention.rs:62-67).  A wave per head,
+// element-wise; same arithmetic as the tiled kernels minus the coefficient folding.
+template <typename T>
+DEV void qknorm_rope_generic_body(T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q,
+                                  int n_kv, int hd, int rot_half, int norm_style, float eps) {
+    typedef typename headstat<T>::acc_t acc_t;
+    const int lane = threadIdx.x & 63;
+    const uint64_t wid = ((uint64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const uint64_t heads = (uint64_t)n_q + n_kv;
+    if (wid >= (uint64_t)rows * heads) return;  // whole wave
+    const uint64_t row = wid / heads;
+    const int hh = (int)(wid % heads);
+    const bool isq = hh < n_q;
+    T* x = isq ? q + (row * n_q + hh) * (uint64_t)hd : k + (row * n_kv + (hh - n_q)) * (uint64_t)hd;
+    const float* w = isq ? qw : kw;
+    const float* t = rope + row * (uint64_t)rot_half * 2;
+    typename headstat<T>::scale_t scale{};
+    if (w) {
+        acc_t ss = 0;
+        for (int i = lane; i < hd; i += 64) ss = headstat<T>::sq(ss, (float)x[i]);
+        ss = group_sum<64>(ss);  // every lane's loads are consumed here, before any store below
+        scale = headstat<T>::rscale(ss, hd, eps);
+    }
+    for (int i = lane; i < rot_half; i += 64) {
+        const int ia = norm_style ? 2 * i : i, ib = norm_style ? 2 * i + 1 : i + rot_half;
+        float a = (float)x[ia], b = (float)x[ib];
+        if (w) {
+            a = headstat<T>::apply(a, scale, w[ia]);
+            b = headstat<T>::apply(b, scale, w[ib]);
+        }
+        const float sn = t[2 * i], cs = t[2 * i + 1];
+        x[ia] = (T)(a * cs - b * sn);
+        x[ib] = (T)(a * sn + b * cs);
+    }
+    if (w)
+        for (int i = 2 * rot_half + lane; i < hd; i += 64) x[i] = (T)headstat<T>::apply((float)x[i], scale, w[i]);
+}
+extern "C" __global__ __launch_bounds__(256) void apk_qknorm_rope_generic_f32(
+    float* q, float* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv, int hd,
+    int rot_half, int norm_style, float eps) {
+    qknorm_rope_generic_body<float>(q, k, qw, kw, rope, rows, n_q, n_kv, hd, rot_half, norm_style, eps);
+}
+extern "C" __global__ __launch_bounds__(256) void apk_qknorm_rope_generic_f16(
+    f16_t* q, f16_t* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv, int hd,
+    int rot_half, int norm_style, float eps) {
+    qknorm_rope_generic_body<f16_t>(q, k, qw, kw, rope, rows, n_q, n_kv, hd, rot_half, norm_style, eps);
+}
+
+// Layer prologue for small decode batches: the residual add + RMSNorm of the hidden
+// rows and the QK-norm + RoPE of the q/k rows as ONE launch.  They are two independent
+// jobs sharing a grid (workgroups [0, rows) normalise one hidden row each, the rest
+// own 8-head groups of q/k); in a layer a QKV projection sits between them, so this
+// removes a launch, not a pass over memory.  One tile per lane (NCH = 1), one pass per
+// wave (ITER = 1): the shapes where launch latency, not bandwidth, is the cost.
+#define APK_PROLOGUE(T, TN, HD)                                                                                   \
+    extern "C" __global__ __launch_bounds__(1024) void apk_layer_prologue_##TN##_hd##HD(                         \
+        T* x, const T* delta, T* h, const float* gamma, int n, T* q, T* k, const float* qw, const float* kw,     \
+        const float* rope, int rows, int n_q, int n_kv, float eps) {                                             \
+        if (blockIdx.x < (uint32_t)rows) add_rmsnorm_body<T, 1>(x, delta, h, gamma, n, eps, blockIdx.x);         \
+        else qknorm_rope_body<T, HD, 1>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, blockIdx.x - (uint32_t)rows);  \
+    }
+APK_PROLOGUE(float, f32, 64) APK_PROLOGUE(float, f32, 128) APK_PROLOGUE(float, f32, 256)
+APK_PROLOGUE(f16_t, f16, 64) APK_PROLOGUE(f16_t, f16, 128) APK_PROLOGUE(f16_t, f16, 256)
+
+// RoPE table rows from per-row positions (rope.rs:18-22, session.rs:34-50):
+// table[r][i] = [sin, cos]((pos[r] as f32) * inv_freq[i]).  One f32 rounding of
+// the angle, as the reference; then sine and cosine of that f32 angle in double
+// precision, rounded once to f32: the correctly rounded values, which is what the
+// reference's libm returns in all but rare cases -- a 2-ulp sincosf here would
+// show as 1e-5 in rotated outputs that nearly cancel.  (The table is rows*half
+// values: the cost of the double evaluation does not register.)
+extern "C" __global__ __launch_bounds__(256) void apk_rope_table(const uint32_t* pos, const float* inv_freq, int rows,
+                                                                int half, float* table) {
+    const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (uint64_t)rows * half) return;
+    const float ang = (float)pos[i / half] * inv_freq[i % half];
+    double s, c;
+    sincos((double)ang, &s, &c);
+    table[2 * i] = (float)s;
+    table[2 * i + 1] = (float)c;
+}
