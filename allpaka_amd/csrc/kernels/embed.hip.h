@@ -38,7 +38,8 @@ DEV void k4_scale_min(const u32x4 hdr, int s, float& sc, float& mn) {
 // The embedding multiplier of models that scale their token embeddings (`*v *= embed_scale`
 // after the dequant, only when it is not 1: model/prefill.rs:107-109, model/decode.rs:427-429).
 template <int N> DEV void embed_scale(float* v, float scale) {
-    if (scale != 1.0f) {
+    // compared as bits: as floats the compiler drops the test (v * 1.0f == v) and multiplies every time
+    if (__builtin_bit_cast(uint32_t, scale) != 0x3f800000u) {
 #pragma unroll
         for (int i = 0; i < N; i++) v[i] *= scale;
     }
@@ -129,12 +130,21 @@ template <> struct qbytes<8> {
     u32x2 v;
     DEV qbytes<8> at(const uint8_t* p) { return qbytes<8>{*(const u32x2_a2*)p}; }
     DEV uint32_t byte(const qbytes<8>& q, int i) { return (q.v[i >> 2] >> (8 * (i & 3))) & 0xffu; }
+    DEV uint32_t word(const qbytes<8>& q, int w) { return q.v[w]; }  // bytes 4w .. 4w+3
 };
 template <> struct qbytes<4> {
     uint32_t v;
     DEV qbytes<4> at(const uint8_t* p) { return qbytes<4>{*(const u32_a2*)p}; }
     DEV uint32_t byte(const qbytes<4>& q, int i) { return (q.v >> (8 * i)) & 0xffu; }
+    DEV uint32_t word(const qbytes<4>& q, int) { return q.v; }
 };
+// The four bytes of a word as floats (each a single byte-to-float conversion of the hardware).
+DEV void bytes_to_f32(uint32_t w, float* f) {
+    f[0] = (float)(w & 0xffu);
+    f[1] = (float)((w >> 8) & 0xffu);
+    f[2] = (float)((w >> 16) & 0xffu);
+    f[3] = (float)(w >> 24);
+}
 template <int FMT> struct dqd;  // tile<N>(row, e0, o): outputs e0 .. e0+N-1 of the row, e0 a multiple of N
 template <> struct dqd<3> {     // Q8_0 (dequant.rs:94-126): 34-byte block = f16 scale + 32 int8; out = d * q
     static constexpr int BE = 32, BB = 34;
@@ -174,7 +184,12 @@ template <> struct dqd<4> {  // Q2_K (dequant.rs:150-174): scales[16] qs[64] d d
         const float dl = h2f(dd & 0xffffu) * (float)(sc & 0xfu), ml = h2f(dd >> 16) * (float)(sc >> 4);
         const qbytes<N> qs = qbytes<N>::at(b + 16 + half * 32 + group * 16 + l0);
 #pragma unroll
-        for (int i = 0; i < N; i++) o[i] = dl * (float)((qbytes<N>::byte(qs, i) >> (2 * si)) & 3u) - ml;
+        for (int w = 0; w < N / 4; w++) {  // four 2-bit quants at a time, in the bytes of one word
+            float f[4];
+            bytes_to_f32((qbytes<N>::word(qs, w) >> (2 * si)) & 0x03030303u, f);
+#pragma unroll
+            for (int i = 0; i < 4; i++) o[4 * w + i] = dl * f[i] - ml;
+        }
     }
 };
 template <> struct dqd<5> {  // Q3_K (dequant.rs:176-204; scales: allpaka-dtype lib.rs:395-422): hmask[32] qs[64] scales[12] d
@@ -191,11 +206,17 @@ template <> struct dqd<5> {  // Q3_K (dequant.rs:176-204; scales: allpaka-dtype 
         const int idx0 = group * 16 + l0;
         const qbytes<N> hm = qbytes<N>::at(b + idx0);
         const qbytes<N> qs = qbytes<N>::at(b + 32 + half * 32 + idx0);
-        const uint32_t m = 1u << (half * 4 + si);
+        // four quants at a time, in the bytes of one word: the two low bits | the mask bit << 2 = 0 .. 7, which is
+        // the reference's (low bits - (mask bit ? 0 : 4)) plus 4
+        const int mbit = half * 4 + si;
 #pragma unroll
-        for (int i = 0; i < N; i++) {
-            const int quant = (int)((qbytes<N>::byte(qs, i) >> (2 * si)) & 3u) - ((qbytes<N>::byte(hm, i) & m) ? 0 : 4);
-            o[i] = dl * (float)quant;
+        for (int w = 0; w < N / 4; w++) {
+            const uint32_t low = (qbytes<N>::word(qs, w) >> (2 * si)) & 0x03030303u;
+            const uint32_t top = (qbytes<N>::word(hm, w) >> mbit) & 0x01010101u;
+            float f[4];
+            bytes_to_f32(low | (top << 2), f);
+#pragma unroll
+            for (int i = 0; i < 4; i++) o[4 * w + i] = dl * (f[i] - 4.0f);
         }
     }
 };
@@ -211,11 +232,14 @@ template <> struct dqd<1> {  // Q5_K (dequant.rs:238-263): d dmin scales[12] qh[
         k4_scale_min(hdr, sub, sc, mn);
         const float dsc = h2f(hdr.x & 0xffffu) * sc, dm = h2f(hdr.x >> 16) * mn;
 #pragma unroll
-        for (int i = 0; i < N; i++) {
-            const uint32_t byte = qbytes<N>::byte(qs, i);
-            const uint32_t q4 = hn ? (byte >> 4) : (byte & 0xfu);
-            const uint32_t hb = (qbytes<N>::byte(qh, i) >> sub) & 1u;
-            o[i] = dsc * (float)(q4 + 16u * hb) - dm;
+        for (int w = 0; w < N / 4; w++) {  // four quants at a time, in the bytes of one word: nibble | fifth bit << 4
+            const uint32_t lo = qbytes<N>::word(qs, w);
+            const uint32_t nib = (hn ? lo >> 4 : lo) & 0x0f0f0f0fu;
+            const uint32_t top = (qbytes<N>::word(qh, w) >> sub) & 0x01010101u;
+            float f[4];
+            bytes_to_f32(nib | (top << 4), f);
+#pragma unroll
+            for (int i = 0; i < 4; i++) o[4 * w + i] = dsc * f[i] - dm;
         }
     }
 };
@@ -228,12 +252,17 @@ template <> struct dqd<2> {  // Q6_K (dequant.rs:271-295): ql[128] qh[64] scales
         const qbytes<N> qh = qbytes<N>::at(b + 128 + half * 32 + l0);
         const float sc = (float)(int8_t)b[192 + half * 8 + is + 2 * quarter];
         const float dl = h2f(*(const uint16_t*)(b + 208)) * sc;
+        // four quants at a time, in the bytes of one word: low nibbles | high bit pairs << 4 = 0 .. 63; the
+        // reference's (q as i8 - 32) as f32 is that byte as a float minus 32 (both exact)
 #pragma unroll
-        for (int i = 0; i < N; i++) {
-            const uint32_t lo = qbytes<N>::byte(ql, i);
-            const uint32_t nib = quarter < 2 ? (lo & 0xfu) : (lo >> 4);
-            const int qv = (int)(nib | (((qbytes<N>::byte(qh, i) >> (2 * quarter)) & 3u) << 4)) - 32;
-            o[i] = dl * (float)qv;
+        for (int w = 0; w < N / 4; w++) {
+            const uint32_t lo = qbytes<N>::word(ql, w);
+            const uint32_t nib = (quarter < 2 ? lo : lo >> 4) & 0x0f0f0f0fu;
+            const uint32_t q4 = nib | (((qbytes<N>::word(qh, w) >> (2 * quarter)) & 0x03030303u) << 4);
+            float f[4];
+            bytes_to_f32(q4, f);
+#pragma unroll
+            for (int i = 0; i < 4; i++) o[4 * w + i] = dl * (f[i] - 32.0f);
         }
     }
 };
