@@ -1083,7 +1083,15 @@ int apk_route_group(apk_ctx* c, const float* logits, const float* bias, size_t r
     if (rows && (!logits || !ids || !w || !tok || !hit_row || !hit_w)) return fail(APK_DECLINE_NULL, "apk_route_group: NULL tensor");
     if (rows == 0 || rows > 16) {
         // beyond a decode-sized batch the two launches are bound by their work, not by the launch:
-        // the same results from the two entries (every decline is theirs; nothing above can fail below)
+        // the same results from the two entries.  What the second could still decline after the first has
+        // run -- its scratch having to grow inside a recording or under a recorded graph -- is checked first.
+        if (rows > 2048) {
+            std::lock_guard<std::mutex> lock(c->mu);
+            if ((rows + 1023) / 1024 * n_expert > c->permute_counts_cap && (c->capturing || c->graphs_with_permute))
+                return fail(APK_DECLINE_CAPTURE, "apk_route_group: the grouping scratch would have to grow %s",
+                            c->capturing ? "inside a recording (run once unrecorded first)"
+                                         : "while a recorded graph holds its address (destroy the graph first)");
+        }
         if (int rc = apk_route_topk(c, logits, bias, rows, n_expert, k, norm, scale, sigmoid, ids, w)) return rc;
         return apk_moe_permute(c, ids, w, rows, k, n_expert, table, n_used, tok, tok_off, hit_row, hit_w);
     }
