@@ -76,8 +76,9 @@ std::vector<std::string> all_kernel_names() {
         for (int hd : kQkHeadDims) v.push_back(std::string("apk_layer_prologue_") + t + "_hd" + std::to_string(hd));
         for (int hd : kQkHeadDims)
             for (int it : kQkIters) {
-                v.push_back(std::string("apk_qknorm_rope_") + t + "_hd" + std::to_string(hd) + "_i" + std::to_string(it));
-                v.push_back(std::string("apk_qknorm_rope_kv_") + t + "_hd" + std::to_string(hd) + "_i" + std::to_string(it));
+                for (const char* style : {"", "pairs_"})
+                    for (const char* kv : {"", "kv_"})
+                        v.push_back(std::string("apk_qknorm_rope_") + style + kv + t + "_hd" + std::to_string(hd) + "_i" + std::to_string(it));
             }
     }
     return v;
@@ -201,9 +202,9 @@ int plan_qknorm_rope(size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size
     if (!es) return fail(APK_DECLINE_UNSUPPORTED, "apk_qknorm_rope: dtype %d", dtype);
     if (head_dim == 0 || head_dim > 65536 || rot_dim % 2 || rot_dim > head_dim)
         return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope: head_dim %zu, rot_dim %zu", head_dim, rot_dim);
-    const bool tiled = style == 0 && rot_dim == head_dim && (head_dim == 64 || head_dim == 128 || head_dim == 256);
+    const bool tiled = rot_dim == head_dim && (head_dim == 64 || head_dim == 128 || head_dim == 256);
     if (with_kv && !tiled)
-        return fail(APK_DECLINE_UNSUPPORTED, "apk_qknorm_rope_kv_store: NeoX over a whole head of 64/128/256 only (head_dim %zu, rot_dim %zu)",
+        return fail(APK_DECLINE_UNSUPPORTED, "apk_qknorm_rope_kv_store: rotation over a whole head of 64/128/256 only (head_dim %zu, rot_dim %zu)",
                     head_dim, rot_dim);
     if (rows == 0 || n_q + n_kv == 0) return APK_OK;
     if (with_kv && n_kv == 0) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_kv_store: no k heads");
@@ -235,8 +236,8 @@ int plan_qknorm_rope(size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size
     const uint64_t grid = (waves * 64 + block - 1) / block;
     if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope: too large");
     p->variant = QK_TILED;
-    plan_name(p, std::string(with_kv ? "apk_qknorm_rope_kv_" : "apk_qknorm_rope_") + t + "_hd" + std::to_string(head_dim) + "_i" +
-                     std::to_string(iter));
+    plan_name(p, std::string("apk_qknorm_rope_") + (style ? "pairs_" : "") + (with_kv ? "kv_" : "") + t + "_hd" + std::to_string(head_dim) +
+                     "_i" + std::to_string(iter));
     p->grid = (unsigned)grid;
     p->block = block;
     p->tiles_per_lane = iter;
@@ -835,7 +836,7 @@ static int qknorm_rope_common(apk_ctx* c, void* q, void* k, const float* qw, con
         return launch(c, p.kernel, p.grid, p.block, 0, gargs);
     }
     auto which = [&] { return std::string(p.kernel); };
-    const uint32_t variant = (uint32_t)dtype << 16 | (uint32_t)head_dim << 4 | p.tiles_per_lane;
+    const uint32_t variant = (uint32_t)style << 20 | (uint32_t)dtype << 16 | (uint32_t)head_dim << 4 | p.tiles_per_lane;
     if (kv) {
         uint32_t cap32 = (uint32_t)kv->capacity;
         void* kargs[] = {&q, &k, (void*)&kv->v, &qw, &kw, &rope, (void*)&kv->cache_pos, (void*)&kv->k_cache, (void*)&kv->v_cache,
@@ -868,6 +869,16 @@ int apk_qknorm_rope_kv_store(apk_ctx* c, void* q, void* k, const void* v, const 
     KvStore kv;
     kv.v = v; kv.cache_pos = cache_pos; kv.k_cache = k_cache; kv.v_cache = v_cache; kv.capacity = capacity;
     return qknorm_rope_common(c, q, k, qw, kw, rope, rows, n_q, n_kv, head_dim, rot_dim, eps, dtype, &kv);
+}
+
+int apk_qknorm_rope_norm_kv_store(apk_ctx* c, void* q, void* k, const void* v, const float* qw, const float* kw,
+                                  const float* rope, const uint32_t* cache_pos, void* k_cache, void* v_cache, size_t capacity,
+                                  size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim, float eps, int dtype) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_qknorm_rope_norm_kv_store: ctx is NULL");
+    CallScope s(c);
+    KvStore kv;
+    kv.v = v; kv.cache_pos = cache_pos; kv.k_cache = k_cache; kv.v_cache = v_cache; kv.capacity = capacity;
+    return qknorm_rope_common(c, q, k, qw, kw, rope, rows, n_q, n_kv, head_dim, rot_dim, eps, dtype, &kv, 1);
 }
 
 int apk_layer_prologue(apk_ctx* c, void* x, const void* delta, void* h, const float* gamma, size_t n, void* q, void* k,

@@ -24,7 +24,11 @@
 // KV = true (k items only): the rotated k tiles are also narrowed to fp16 into the cache row
 // kc, and the same tiles of the row's v are narrowed into vc (KvCache::store_at,
 // crates/allpaka-model/src/kv.rs:682-697: k and v rows as f16 at pos*kv_dim).
-template <typename T, int HD, int ITER, bool KV = false>
+// PAIRS = false: NeoX pairs (i, i + HD/2), one from each of the lane's two tiles; the lane's [sin, cos]
+// entries are l*EPL .. l*EPL+EPL-1.  PAIRS = true: adjacent pairs (2i, 2i+1) (RopeStyle::Norm, rope.rs:52-64,
+// the Llama-family layout, chosen per model in attention.rs:62-67), both inside one tile; the lane's
+// entries are the EPL/2 pairs of each of its two tiles.  Same loads, same bytes, same statistics.
+template <typename T, int HD, int ITER, bool KV = false, bool PAIRS = false>
 DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, float eps, int l, int sub,
                  f16_t* kc = nullptr, const T* vrow = nullptr, f16_t* vc = nullptr) {
     constexpr int EPL = io<T>::VEC;   // elements per lane per half
@@ -38,7 +42,10 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
     // missing norm weight is read from the [sin, cos] tile instead and never used.
     float sc[2 * EPL], wa[EPL], wb[EPL];
 #pragma unroll
-    for (int i = 0; i < 2 * EPL; i += 4) io<float>::load(trow + 2 * EPL * l + i, sc + i);
+    for (int i = 0; i < 2 * EPL; i += 4) {
+        if constexpr (PAIRS) io<float>::load(trow + (i < EPL ? EPL * l + i : HALF + EPL * l + i - EPL), sc + i);
+        else io<float>::load(trow + 2 * EPL * l + i, sc + i);
+    }
     const float* wp = w ? w : trow;
 #pragma unroll
     for (int i = 0; i < EPL; i += 4) {
@@ -76,16 +83,34 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
         }
         ss = group_sum<LPH>(ss);
         const typename headstat<T>::scale_t scale = headstat<T>::rscale(ss, HD, eps);
+        if constexpr (PAIRS) {
 #pragma unroll
-        for (int i = 0; i < EPL; i++) {
-            float x = a[i], y = b[i];
-            if (normed) {
-                x = headstat<T>::apply(x, scale, wa[i]);
-                y = headstat<T>::apply(y, scale, wb[i]);
+            for (int i = 0; i < EPL; i++) {
+                if (normed) {
+                    a[i] = headstat<T>::apply(a[i], scale, wa[i]);
+                    b[i] = headstat<T>::apply(b[i], scale, wb[i]);
+                }
             }
-            const float s = sc[2 * i], c = sc[2 * i + 1];
-            oa[i] = x * c - y * s;  // not contracted: the reference's four products and two sums
-            ob[i] = x * s + y * c;
+#pragma unroll
+            for (int m = 0; m < EPL / 2; m++) {  // sc[0 .. EPL): the pairs of tile a, sc[EPL .. 2 EPL): of tile b
+                const float sa = sc[2 * m], ca = sc[2 * m + 1], sb = sc[EPL + 2 * m], cb = sc[EPL + 2 * m + 1];
+                oa[2 * m] = a[2 * m] * ca - a[2 * m + 1] * sa;
+                oa[2 * m + 1] = a[2 * m] * sa + a[2 * m + 1] * ca;
+                ob[2 * m] = b[2 * m] * cb - b[2 * m + 1] * sb;
+                ob[2 * m + 1] = b[2 * m] * sb + b[2 * m + 1] * cb;
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < EPL; i++) {
+                float x = a[i], y = b[i];
+                if (normed) {
+                    x = headstat<T>::apply(x, scale, wa[i]);
+                    y = headstat<T>::apply(y, scale, wb[i]);
+                }
+                const float s = sc[2 * i], c = sc[2 * i + 1];
+                oa[i] = x * c - y * s;  // not contracted: the reference's four products and two sums
+                ob[i] = x * s + y * c;
+            }
         }
         const bool live = hh_first + it * HPW < nheads;
         const int off = head_off(it);
@@ -108,7 +133,7 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
     }
 }
 
-template <typename T, int HD, int ITERQ, bool KV = false>
+template <typename T, int HD, int ITERQ, bool KV = false, bool PAIRS = false>
 DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv,
                           float eps, uint32_t vblock, const T* v = nullptr, const uint32_t* cache_pos = nullptr,
                           f16_t* k_cache = nullptr, f16_t* v_cache = nullptr, uint32_t capacity = 0,
@@ -123,7 +148,7 @@ DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const fl
     if (wid >= nq_items + (uint64_t)rows * gk) return;  // whole wave
     if (wid < nq_items) {
         const uint64_t row = wid / gq;
-        qk_item<T, HD, ITERQ>(q + row * (uint64_t)n_q * HD, n_q, (int)(wid % gq), qw, rope + row * HD, eps, l, sub);
+        qk_item<T, HD, ITERQ, false, PAIRS>(q + row * (uint64_t)n_q * HD, n_q, (int)(wid % gq), qw, rope + row * HD, eps, l, sub);
     } else {
         const uint64_t w2 = wid - nq_items, row = w2 / gk;
         const uint64_t kv_dim = (uint64_t)n_kv * HD;
@@ -131,11 +156,11 @@ DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const fl
             const uint32_t pos = cache_pos[row];
             const bool ok = pos < capacity;
             if (!ok && lane == 0 && w2 % gk == 0) atomicOr(fault, APK_FAULT_CACHE_RANGE);
-            qk_item<T, HD, 1, true>(k + row * kv_dim, n_kv, (int)(w2 % gk), kw, rope + row * HD, eps, l, sub,
+            qk_item<T, HD, 1, true, PAIRS>(k + row * kv_dim, n_kv, (int)(w2 % gk), kw, rope + row * HD, eps, l, sub,
                                     ok ? k_cache + pos * kv_dim : nullptr, v + row * kv_dim,
                                     ok ? v_cache + pos * kv_dim : nullptr);
         } else {
-            qk_item<T, HD, 1>(k + row * kv_dim, n_kv, (int)(w2 % gk), kw, rope + row * HD, eps, l, sub);
+            qk_item<T, HD, 1, false, PAIRS>(k + row * kv_dim, n_kv, (int)(w2 % gk), kw, rope + row * HD, eps, l, sub);
         }
     }
 }
@@ -145,6 +170,10 @@ DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const fl
     extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void apk_qknorm_rope_##TN##_hd##HD##_i##ITER(   \
         T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv, float eps) { \
         qknorm_rope_body<T, HD, ITER>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, blockIdx.x);                  \
+    }                                                                                                        \
+    extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void apk_qknorm_rope_pairs_##TN##_hd##HD##_i##ITER( \
+        T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv, float eps) { \
+        qknorm_rope_body<T, HD, ITER, false, true>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, blockIdx.x);     \
     }
 #define APK_QKROPE_ALL(T, TN)                                                                                          \
     APK_QKROPE(T, TN, 64, 1) APK_QKROPE(T, TN, 64, 2) APK_QKROPE(T, TN, 128, 1) APK_QKROPE(T, TN, 128, 2)              \
@@ -160,6 +189,12 @@ APK_QKROPE_ALL(f16_t, f16)
         f16_t* k_cache, f16_t* v_cache, uint32_t capacity, int rows, int n_q, int n_kv, float eps, uint32_t* fault) { \
         qknorm_rope_body<T, HD, ITER, true>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, blockIdx.x, v, cache_pos,   \
                                             k_cache, v_cache, capacity, fault);                                   \
+    }                                                                                                             \
+    extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void apk_qknorm_rope_pairs_kv_##TN##_hd##HD##_i##ITER( \
+        T* q, T* k, const T* v, const float* qw, const float* kw, const float* rope, const uint32_t* cache_pos,  \
+        f16_t* k_cache, f16_t* v_cache, uint32_t capacity, int rows, int n_q, int n_kv, float eps, uint32_t* fault) { \
+        qknorm_rope_body<T, HD, ITER, true, true>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, blockIdx.x, v, cache_pos, \
+                                                  k_cache, v_cache, capacity, fault);                             \
     }
 #define APK_QKROPE_KV_ALL(T, TN)                                                                                       \
     APK_QKROPE_KV(T, TN, 64, 1) APK_QKROPE_KV(T, TN, 64, 2) APK_QKROPE_KV(T, TN, 128, 1) APK_QKROPE_KV(T, TN, 128, 2)  \

@@ -235,6 +235,12 @@ def main():
             h, p(qk[i % len(qk)]["q"]), p(qk[i % len(qk)]["k"]), p(kvp[i % len(qk)]["v"]), p(qw), p(kw), p(rope), p(pos),
             p(kvp[i % len(qk)]["kc"]), p(kvp[i % len(qk)]["vc"]), T, T, NQ, NKV, HD, HD, EPS, F16)), reps)
         record("qknorm_rope_neox + K/V cache store (one launch)", tag, us, bytes_qkrope + T * NKV * HD * b + 2 * T * NKV * HD * 2 + T * 4)
+        # the same rows with the adjacent-pair rotation and no QK-norm: the prologue of the Llama-family layouts
+        # (32 q heads and 8 k heads of 128: the leading heads of the same buffers)
+        lq, lkv = 32, 8
+        us = timed(lambda i: apklib.check(L.apk_qknorm_rope_norm(h, p(qk[i % len(qk)]["q"]), p(qk[i % len(qk)]["k"]), None, None, p(rope),
+                                                                 T, lq, lkv, HD, HD, EPS, F16)), reps)
+        record("rope, adjacent pairs, no QK-norm", f"32 q + 8 k heads of 128, T={T} f16", us, 2 * T * (lq + lkv) * HD * b + T * HD * 4)
         # what fusing the residual add into the norm buys: the same result as two launches of this library's own ops
         us = timed(lambda i: (apklib.check(L.apk_add_assign(h, p(an[i % len(an)]["x"]), p(an[i % len(an)]["d"]), T * H, F16)),
                               apklib.check(L.apk_add_rmsnorm_rows(h, p(an[i % len(an)]["x"]), None, p(an[i % len(an)]["h"]), p(gamma1), H, T, EPS, F16))), reps)

@@ -229,7 +229,8 @@ int apk_qknorm_rope_neox(apk_ctx* ctx, void* q, void* k, const float* qw, const 
                          int dtype);
 /* The same with the adjacent-pair rotation (2i, 2i+1) of RopeStyle::Norm models:
  * ops::rope_norm_cached_from_array (ops/rope.rs:52-64), selected per model in
- * rope_from_arrays (model/attention.rs:62-67).  Element-wise kernel for every geometry. */
+ * rope_from_arrays (model/attention.rs:62-67).  The same kernel choice: tiled for a whole head of
+ * 64 / 128 / 256, element-wise otherwise. */
 int apk_qknorm_rope_norm(apk_ctx* ctx, void* q, void* k, const float* qw, const float* kw, const float* rope,
                          size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim, float eps,
                          int dtype);
@@ -250,6 +251,13 @@ int apk_qknorm_rope_kv_store(apk_ctx* ctx, void* q, void* k, const void* v, cons
                              const float* rope, const uint32_t* cache_pos, void* k_cache, void* v_cache,
                              size_t capacity, size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim,
                              float eps, int dtype);
+
+/* The same with adjacent rotary pairs (RopeStyle::Norm, as apk_qknorm_rope_norm): the chunk prologue of
+ * the Llama-family layouts with the cache store fused in. */
+int apk_qknorm_rope_norm_kv_store(apk_ctx* ctx, void* q, void* k, const void* v, const float* qw, const float* kw,
+                                  const float* rope, const uint32_t* cache_pos, void* k_cache, void* v_cache,
+                                  size_t capacity, size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim,
+                                  float eps, int dtype);
 
 /* Layer prologue as ONE launch: apk_add_rmsnorm_rows(x, delta, h, gamma, n, rows) and
  * apk_qknorm_rope_neox(q, k, qw, kw, rope, rows, ...) with the same arguments and the

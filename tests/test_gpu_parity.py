@@ -483,6 +483,34 @@ def test_qknorm_rope_any_geometry(be, ora, rows, n_q, n_kv, hd, rot, style, f16,
             assert rel_err_f32(got, want) <= TOL_F32 and close_idiom(got, want)
 
 
+@pytest.mark.parametrize("rows,n_q,n_kv,hd", [(1, 32, 8, 128), (6, 32, 8, 128), (64, 32, 8, 128), (300, 32, 8, 128), (2048, 8, 2, 128),
+                                            (700, 64, 8, 128), (33, 12, 2, 64), (400, 32, 8, 64), (9, 8, 1, 256), (350, 16, 4, 256),
+                                            (5, 3, 0, 128), (5, 0, 3, 64)])
+@pytest.mark.parametrize("f16", [False, True])
+@pytest.mark.parametrize("normed", [True, False])
+def test_adjacent_pair_rope_on_whole_heads(be, ora, rows, n_q, n_kv, hd, f16, normed):
+    """RopeStyle::Norm (pairs (2i, 2i+1), rope.rs:52-64: the Llama-family layout, attention.rs:62-67) over whole
+    heads of 64 / 128 / 256: the tiled kernels, one and two passes per q wave, with and without the QK-norm."""
+    s = synth()
+    g = s.rng(3, rows * 131 + n_q * 7 + hd)
+    q, k = s.normal_f32(g, (rows, n_q * hd)), s.normal_f32(g, (rows, n_kv * hd))
+    qw, kw = (s.normal_f32(g, hd, 1.0, 0.05), s.normal_f32(g, hd, 1.0, 0.05)) if normed else (None, None)
+    if f16:
+        q, k = s.to_f16_bits(q), s.to_f16_bits(k)
+    ropes = ora.rope_table([int(v) for v in g.integers(0, 32768, size=rows)], ora.rope_inv_freq(hd, 5e5))
+    wq, wk = q.copy(), k.copy()
+    ora.qknorm_rope_rows(wq, wk, n_q, n_kv, hd, qw, kw, ropes, 1e-5, style=1)
+    tq, tk = dev(q), dev(k)
+    be.qknorm_rope_norm(tq, tk, None if qw is None else dev(qw), None if kw is None else dev(kw), dev(ropes), n_q, n_kv, hd, 1e-5)
+    for got, want in ((host(tq), wq), (host(tk), wk)):
+        if f16:
+            assert np.array_equal(got, want)  # the definition, bit for bit (as the NeoX kernels)
+        elif not normed:
+            assert np.array_equal(got, want)  # rotation only: the same f32 operations
+        else:
+            assert rel_err_f32(got, want) <= TOL_F32 and close_idiom(got, want)
+
+
 def test_rope_table_on_device(be, ora):
     # table rows built on the device vs ops::rope_sin_cos: same f32 angle, device sincosf vs glibc
     inv = ora.rope_inv_freq(128, 1e6)
@@ -507,7 +535,8 @@ def test_rope_table_on_device(be, ora):
 # --------------------------------------------- fused K/V cache store
 @pytest.mark.parametrize("rows,n_q,n_kv,hd,f16", [(1, 16, 8, 128, False), (64, 64, 8, 128, True), (300, 64, 8, 128, True),
                                                    (7, 4, 4, 64, False), (5, 2, 1, 256, True), (2048, 16, 8, 128, False)])
-def test_qknorm_rope_kv_store(be, ora, rows, n_q, n_kv, hd, f16):
+@pytest.mark.parametrize("style", [0, 1])
+def test_qknorm_rope_kv_store(be, ora, rows, n_q, n_kv, hd, f16, style):
     """QK-norm + RoPE with KvCache::store_at fused: q, k as the plain op; the cache rows hold
     the rotated k and the row's v narrowed to f16 (RNE) at each row's position."""
     s = synth()
@@ -519,13 +548,14 @@ def test_qknorm_rope_kv_store(be, ora, rows, n_q, n_kv, hd, f16):
     if f16:
         v = s.to_f16_bits(v)
     wq, wk = q.copy(), k.copy()
-    ora.qknorm_rope_rows(wq, wk, n_q, n_kv, hd, qw, kw, ropes, 1e-6)
+    ora.qknorm_rope_rows(wq, wk, n_q, n_kv, hd, qw, kw, ropes, 1e-6, style=style)
     wkc, wvc = np.zeros((cap, n_kv * hd), np.uint16), np.zeros((cap, n_kv * hd), np.uint16)
     ora.kv_store_rows(wk, v, positions, wkc, wvc)
     tq, tk = dev(q), dev(k)
     kc = torch.zeros((cap, n_kv * hd), dtype=torch.float16, device="cuda")
     vc = torch.zeros_like(kc)
-    be.qknorm_rope_kv_store(tq, tk, dev(v), dev(qw), dev(kw), dev(ropes), dev(positions), kc, vc, n_q, n_kv, hd, 1e-6)
+    be.qknorm_rope_kv_store(tq, tk, dev(v), dev(qw), dev(kw), dev(ropes), dev(positions), kc, vc, n_q, n_kv, hd, 1e-6,
+                            adjacent_pairs=bool(style))
     gk = host(tk)
     for got, want in ((host(tq), wq), (gk, wk)):
         if f16:

@@ -141,7 +141,7 @@ def test_qknorm_rope_plans_cover_every_head(L, kernels, bounds):
                 for rows in (1, 6, 64, 255, 512, 2048, 2061, 8192, 100000):
                     for kv in (0, 1):
                         rc, p = plan(L.apk_plan_qknorm_rope, rows, n_q, n_kv, hd, rot, style, dtype, kv)
-                        tiled = style == 0 and rot == hd and hd in (64, 128, 256)
+                        tiled = rot == hd and hd in (64, 128, 256)
                         if kv and not tiled:
                             assert rc == 1
                             continue
@@ -154,7 +154,8 @@ def test_qknorm_rope_plans_cover_every_head(L, kernels, bounds):
                         if not tiled:
                             assert "generic" in name and waves_launched >= rows * (n_q + n_kv) > waves_launched - 4
                             continue
-                        assert name == f"apk_qknorm_rope_{'kv_' if kv else ''}{'f32' if dtype == F32 else 'f16'}_hd{hd}_i{p.tiles_per_lane}"
+                        assert name == (f"apk_qknorm_rope_{'pairs_' if style else ''}{'kv_' if kv else ''}{'f32' if dtype == F32 else 'f16'}"
+                                        f"_hd{hd}_i{p.tiles_per_lane}")
                         lph = hd // 2 // (16 // es)  # lanes per head
                         hpw = 64 // lph
                         assert p.lanes_per_row == lph and p.tiles_per_lane in (1, 2)
