@@ -241,18 +241,19 @@ class Backend:
         self._leave()
 
     def qknorm_rope_kv_store(self, q, k, v, q_norm, k_norm, rope_flat, cache_pos, k_cache, v_cache, n_q, n_kv, head_dim, eps,
-                             adjacent_pairs=False):
+                             adjacent_pairs=False, rot_dim=None):
         """qknorm_rope_neox (adjacent_pairs: qknorm_rope_norm), then KvCache::store_at of every row's k and v as
         f16 at cache row cache_pos[r] (kv.rs:682-697), in one launch.  k_cache, v_cache: fp16 [capacity, n_kv*head_dim]."""
         rows = k.numel() // (n_kv * head_dim)
         assert q.numel() == rows * n_q * head_dim and v.numel() == k.numel() == rows * n_kv * head_dim
-        assert rope_flat.numel() == rows * head_dim and q.dtype == k.dtype == v.dtype
+        rot_dim = head_dim if rot_dim is None else rot_dim
+        assert rope_flat.numel() == rows * rot_dim and q.dtype == k.dtype == v.dtype
         assert k_cache.dtype == v_cache.dtype == torch.float16 and k_cache.shape == v_cache.shape
         assert k_cache.shape[1] == n_kv * head_dim and cache_pos.numel() == rows
         self._enter()
         fn = self.L.apk_qknorm_rope_norm_kv_store if adjacent_pairs else self.L.apk_qknorm_rope_kv_store
         check(fn(self.h, _ptr(q), _ptr(k), _ptr(v), _ptr(q_norm), _ptr(k_norm), _ptr(rope_flat), _ptr(cache_pos), _ptr(k_cache),
-                 _ptr(v_cache), k_cache.shape[0], rows, n_q, n_kv, head_dim, head_dim, eps, _dt(q)))
+                 _ptr(v_cache), k_cache.shape[0], rows, n_q, n_kv, head_dim, rot_dim, eps, _dt(q)))
         self._leave()
         # (inside a recording nothing has run yet: the caller reads take_faults() after a replay)
         if not self._recording and self.take_faults() & _l.FAULT_CACHE_RANGE:

@@ -202,9 +202,14 @@ int plan_qknorm_rope(size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size
     if (!es) return fail(APK_DECLINE_UNSUPPORTED, "apk_qknorm_rope: dtype %d", dtype);
     if (head_dim == 0 || head_dim > 65536 || rot_dim % 2 || rot_dim > head_dim)
         return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope: head_dim %zu, rot_dim %zu", head_dim, rot_dim);
-    const bool tiled = rot_dim == head_dim && (head_dim == 64 || head_dim == 128 || head_dim == 256);
+    // the tiled kernels: heads of 64 / 128 / 256 whose rotary width is a whole number of the lanes' 16-byte tiles
+    // (adjacent pairs: a tile rotates or it does not; NeoX: the partner halves are whole tiles); no rotation at
+    // all and every other geometry take the element-wise kernel
+    const size_t epl_t = 16 / es;
+    const bool tiled = (head_dim == 64 || head_dim == 128 || head_dim == 256) && rot_dim > 0 &&
+                       (style ? rot_dim % epl_t == 0 : (rot_dim / 2) % epl_t == 0);
     if (with_kv && !tiled)
-        return fail(APK_DECLINE_UNSUPPORTED, "apk_qknorm_rope_kv_store: rotation over a whole head of 64/128/256 only (head_dim %zu, rot_dim %zu)",
+        return fail(APK_DECLINE_UNSUPPORTED, "apk_qknorm_rope_kv_store: heads of 64/128/256 with a rotary width of whole tiles only (head_dim %zu, rot_dim %zu)",
                     head_dim, rot_dim);
     if (rows == 0 || n_q + n_kv == 0) return APK_OK;
     if (with_kv && n_kv == 0) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_kv_store: no k heads");
@@ -829,7 +834,7 @@ static int qknorm_rope_common(apk_ctx* c, void* q, void* k, const float* qw, con
     }
     if (validate_only) return APK_OK;
     if (int rc = set_device(c)) return rc;
-    int rows_i = (int)rows, nq_i = (int)n_q, nkv_i = (int)n_kv;
+    int rows_i = (int)rows, nq_i = (int)n_q, nkv_i = (int)n_kv, rot_i = (int)rot_dim;
     if (p.variant == QK_GENERIC) {
         int hd_i = (int)head_dim, half_i = (int)(rot_dim / 2);
         void* gargs[] = {&q, &k, &qw, &kw, &rope, &rows_i, &nq_i, &nkv_i, &hd_i, &half_i, &style, &eps};
@@ -840,10 +845,10 @@ static int qknorm_rope_common(apk_ctx* c, void* q, void* k, const float* qw, con
     if (kv) {
         uint32_t cap32 = (uint32_t)kv->capacity;
         void* kargs[] = {&q, &k, (void*)&kv->v, &qw, &kw, &rope, (void*)&kv->cache_pos, (void*)&kv->k_cache, (void*)&kv->v_cache,
-                         &cap32, &rows_i, &nq_i, &nkv_i, &eps, &c->fault_dev};
+                         &cap32, &rows_i, &nq_i, &nkv_i, &eps, &c->fault_dev, &rot_i};
         return launch_keyed(c, OP_QKROPE_KV, variant, which, p.grid, p.block, 0, kargs);
     }
-    void* args[] = {&q, &k, &qw, &kw, &rope, &rows_i, &nq_i, &nkv_i, &eps};
+    void* args[] = {&q, &k, &qw, &kw, &rope, &rows_i, &nq_i, &nkv_i, &eps, &rot_i};
     return launch_keyed(c, OP_QKROPE, variant, which, p.grid, p.block, 0, args);
 }
 

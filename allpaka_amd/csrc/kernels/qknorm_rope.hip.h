@@ -28,44 +28,67 @@
 // entries are l*EPL .. l*EPL+EPL-1.  PAIRS = true: adjacent pairs (2i, 2i+1) (RopeStyle::Norm, rope.rs:52-64,
 // the Llama-family layout, chosen per model in attention.rs:62-67), both inside one tile; the lane's
 // entries are the EPL/2 pairs of each of its two tiles.  Same loads, same bytes, same statistics.
+// Partial rotary (rot < HD channels rotate, the rest is normalised and passes through, rope.rs:52-81): the
+// table row then has rot/2 entries.  With adjacent pairs a whole tile either rotates or does not (rot is a
+// multiple of the tile); with NeoX pairs (i, i + rot/2) the first rot/2/EPL lanes of a head take the partner
+// tiles at i and i + rot/2, the others two consecutive tiles of the tail.  rot == HD is the layout above.
 template <typename T, int HD, int ITER, bool KV = false, bool PAIRS = false>
-DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, float eps, int l, int sub,
+DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, float eps, int l, int sub, int rot,
                  f16_t* kc = nullptr, const T* vrow = nullptr, f16_t* vc = nullptr) {
     constexpr int EPL = io<T>::VEC;   // elements per lane per half
     constexpr int HALF = HD / 2;
     constexpr int LPH = HALF / EPL;   // lanes per head
     constexpr int HPW = 64 / LPH;     // heads per wave pass
     typedef typename headstat<T>::acc_t acc_t;
+    // the lane's two tiles inside a head, whether each rotates, and where its [sin, cos] floats start
+    int off_a, off_b, sc_a, sc_b;
+    bool rot_a, rot_b;
+    if constexpr (PAIRS) {
+        off_a = EPL * l;
+        off_b = HALF + EPL * l;
+        rot_a = off_a < rot;
+        rot_b = off_b < rot;
+        sc_a = rot_a ? off_a : 0;
+        sc_b = rot_b ? off_b : 0;
+    } else {
+        const int lr = (rot >> 1) / EPL;  // lanes of a head that hold rotating pairs
+        rot_a = rot_b = l < lr;
+        off_a = rot_a ? EPL * l : rot + 2 * EPL * (l - lr);
+        off_b = rot_a ? (rot >> 1) + EPL * l : off_a + EPL;
+        sc_a = rot_a ? 2 * EPL * l : 0;
+        sc_b = sc_a + EPL;
+    }
     // Loads return in issue order, so the small cached ones go first and the first pass
     // can start as soon as its own two tiles arrive.  No branch, no conversion here: a
     // lane of a pass beyond the last head re-reads the last head and stores nothing; a
     // missing norm weight is read from the [sin, cos] tile instead and never used.
     float sc[2 * EPL], wa[EPL], wb[EPL];
 #pragma unroll
-    for (int i = 0; i < 2 * EPL; i += 4) {
-        if constexpr (PAIRS) io<float>::load(trow + (i < EPL ? EPL * l + i : HALF + EPL * l + i - EPL), sc + i);
-        else io<float>::load(trow + 2 * EPL * l + i, sc + i);
+    for (int i = 0; i < EPL; i += 4) {  // a tile that does not rotate reads the row's first entries and ignores them
+        io<float>::load(trow + sc_a + i, sc + i);
+        io<float>::load(trow + sc_b + i, sc + EPL + i);
     }
     const float* wp = w ? w : trow;
+    const int w_a = w ? off_a : 0, w_b = w ? off_b : 0;
 #pragma unroll
     for (int i = 0; i < EPL; i += 4) {
-        io<float>::load(wp + EPL * l + i, wa + i);
-        io<float>::load(wp + HALF + EPL * l + i, wb + i);
+        io<float>::load(wp + w_a + i, wa + i);
+        io<float>::load(wp + w_b + i, wb + i);
     }
     typename io<T>::raw_t araw[ITER], braw[ITER], varaw[ITER], vbraw[ITER];
     // head of pass `it` and its element offset: recomputed where needed (a few integer
     // operations) rather than kept in registers across the loads
     const int hh_first = g * ITER * HPW + sub;
-    auto head_off = [&](int it) { return min(hh_first + it * HPW, nheads - 1) * HD + EPL * l; };
+    auto head_off = [&](int it) { return min(hh_first + it * HPW, nheads - 1) * HD; };
 #pragma unroll
     for (int it = 0; it < ITER; it++) {
         const int off = head_off(it);
         __builtin_amdgcn_sched_barrier(0);  // loads stay in program order (returns are in order)
-        araw[it] = io<T>::ldraw_nt(base + off);
-        braw[it] = io<T>::ldraw_nt(base + off + HALF);
+        araw[it] = io<T>::ldraw_nt(base + off + off_a);
+        braw[it] = io<T>::ldraw_nt(base + off + off_b);
         if constexpr (KV) {
-            varaw[it] = io<T>::ldraw_nt(vrow + off);
-            vbraw[it] = io<T>::ldraw_nt(vrow + off + HALF);
+            varaw[it] = io<T>::ldraw_nt(vrow + off + off_a);
+            vbraw[it] = io<T>::ldraw_nt(vrow + off + off_b);
         }
     }
     __builtin_amdgcn_sched_barrier(0);  // every load above; all uses below
@@ -94,10 +117,10 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
 #pragma unroll
             for (int m = 0; m < EPL / 2; m++) {  // sc[0 .. EPL): the pairs of tile a, sc[EPL .. 2 EPL): of tile b
                 const float sa = sc[2 * m], ca = sc[2 * m + 1], sb = sc[EPL + 2 * m], cb = sc[EPL + 2 * m + 1];
-                oa[2 * m] = a[2 * m] * ca - a[2 * m + 1] * sa;
-                oa[2 * m + 1] = a[2 * m] * sa + a[2 * m + 1] * ca;
-                ob[2 * m] = b[2 * m] * cb - b[2 * m + 1] * sb;
-                ob[2 * m + 1] = b[2 * m] * sb + b[2 * m + 1] * cb;
+                oa[2 * m] = rot_a ? a[2 * m] * ca - a[2 * m + 1] * sa : a[2 * m];
+                oa[2 * m + 1] = rot_a ? a[2 * m] * sa + a[2 * m + 1] * ca : a[2 * m + 1];
+                ob[2 * m] = rot_b ? b[2 * m] * cb - b[2 * m + 1] * sb : b[2 * m];
+                ob[2 * m + 1] = rot_b ? b[2 * m] * sb + b[2 * m + 1] * cb : b[2 * m + 1];
             }
         } else {
 #pragma unroll
@@ -108,25 +131,25 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
                     y = headstat<T>::apply(y, scale, wb[i]);
                 }
                 const float s = sc[2 * i], c = sc[2 * i + 1];
-                oa[i] = x * c - y * s;  // not contracted: the reference's four products and two sums
-                ob[i] = x * s + y * c;
+                oa[i] = rot_a ? x * c - y * s : x;  // not contracted: the reference's four products and two sums
+                ob[i] = rot_a ? x * s + y * c : y;
             }
         }
         const bool live = hh_first + it * HPW < nheads;
         const int off = head_off(it);
         if (live) {
-            io<T>::store_nt(base + off, oa);
-            io<T>::store_nt(base + off + HALF, ob);
+            io<T>::store_nt(base + off + off_a, oa);
+            io<T>::store_nt(base + off + off_b, ob);
         }
         if constexpr (KV) {
             if (live && kc != nullptr) {  // kc == nullptr: cache position out of range, row skipped
                 float va[EPL], vb[EPL];
                 io<T>::widen(varaw[it], va);
                 io<T>::widen(vbraw[it], vb);
-                store_f16_tile<T>(kc + off, oa);
-                store_f16_tile<T>(kc + off + HALF, ob);
-                store_f16_tile<T>(vc + off, va);
-                store_f16_tile<T>(vc + off + HALF, vb);
+                store_f16_tile<T>(kc + off + off_a, oa);
+                store_f16_tile<T>(kc + off + off_b, ob);
+                store_f16_tile<T>(vc + off + off_a, va);
+                store_f16_tile<T>(vc + off + off_b, vb);
             }
         }
         __builtin_amdgcn_sched_barrier(0);  // pass by pass: pass it+1 waits only for its own tiles
@@ -135,7 +158,7 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
 
 template <typename T, int HD, int ITERQ, bool KV = false, bool PAIRS = false>
 DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv,
-                          float eps, uint32_t vblock, const T* v = nullptr, const uint32_t* cache_pos = nullptr,
+                          float eps, int rot, uint32_t vblock, const T* v = nullptr, const uint32_t* cache_pos = nullptr,
                           f16_t* k_cache = nullptr, f16_t* v_cache = nullptr, uint32_t capacity = 0,
                           uint32_t* fault = nullptr) {
     constexpr int LPH = HD / 2 / io<T>::VEC, HPW = 64 / LPH;
@@ -148,7 +171,7 @@ DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const fl
     if (wid >= nq_items + (uint64_t)rows * gk) return;  // whole wave
     if (wid < nq_items) {
         const uint64_t row = wid / gq;
-        qk_item<T, HD, ITERQ, false, PAIRS>(q + row * (uint64_t)n_q * HD, n_q, (int)(wid % gq), qw, rope + row * HD, eps, l, sub);
+        qk_item<T, HD, ITERQ, false, PAIRS>(q + row * (uint64_t)n_q * HD, n_q, (int)(wid % gq), qw, rope + row * (uint64_t)rot, eps, l, sub, rot);
     } else {
         const uint64_t w2 = wid - nq_items, row = w2 / gk;
         const uint64_t kv_dim = (uint64_t)n_kv * HD;
@@ -156,11 +179,11 @@ DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const fl
             const uint32_t pos = cache_pos[row];
             const bool ok = pos < capacity;
             if (!ok && lane == 0 && w2 % gk == 0) atomicOr(fault, APK_FAULT_CACHE_RANGE);
-            qk_item<T, HD, 1, true, PAIRS>(k + row * kv_dim, n_kv, (int)(w2 % gk), kw, rope + row * HD, eps, l, sub,
-                                    ok ? k_cache + pos * kv_dim : nullptr, v + row * kv_dim,
-                                    ok ? v_cache + pos * kv_dim : nullptr);
+            qk_item<T, HD, 1, true, PAIRS>(k + row * kv_dim, n_kv, (int)(w2 % gk), kw, rope + row * (uint64_t)rot, eps, l, sub, rot,
+                                           ok ? k_cache + pos * kv_dim : nullptr, v + row * kv_dim,
+                                           ok ? v_cache + pos * kv_dim : nullptr);
         } else {
-            qk_item<T, HD, 1, false, PAIRS>(k + row * kv_dim, n_kv, (int)(w2 % gk), kw, rope + row * HD, eps, l, sub);
+            qk_item<T, HD, 1, false, PAIRS>(k + row * kv_dim, n_kv, (int)(w2 % gk), kw, rope + row * (uint64_t)rot, eps, l, sub, rot);
         }
     }
 }
@@ -168,12 +191,12 @@ DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const fl
 #define APK_QK_OCC __attribute__((amdgpu_waves_per_eu(4)))
 #define APK_QKROPE(T, TN, HD, ITER)                                                                          \
     extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void apk_qknorm_rope_##TN##_hd##HD##_i##ITER(   \
-        T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv, float eps) { \
-        qknorm_rope_body<T, HD, ITER>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, blockIdx.x);                  \
+        T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv, float eps, int rot) { \
+        qknorm_rope_body<T, HD, ITER>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x);                  \
     }                                                                                                        \
     extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void apk_qknorm_rope_pairs_##TN##_hd##HD##_i##ITER( \
-        T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv, float eps) { \
-        qknorm_rope_body<T, HD, ITER, false, true>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, blockIdx.x);     \
+        T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv, float eps, int rot) { \
+        qknorm_rope_body<T, HD, ITER, false, true>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x);     \
     }
 #define APK_QKROPE_ALL(T, TN)                                                                                          \
     APK_QKROPE(T, TN, 64, 1) APK_QKROPE(T, TN, 64, 2) APK_QKROPE(T, TN, 128, 1) APK_QKROPE(T, TN, 128, 2)              \
@@ -186,14 +209,14 @@ APK_QKROPE_ALL(f16_t, f16)
 #define APK_QKROPE_KV(T, TN, HD, ITER)                                                                            \
     extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void apk_qknorm_rope_kv_##TN##_hd##HD##_i##ITER(     \
         T* q, T* k, const T* v, const float* qw, const float* kw, const float* rope, const uint32_t* cache_pos,  \
-        f16_t* k_cache, f16_t* v_cache, uint32_t capacity, int rows, int n_q, int n_kv, float eps, uint32_t* fault) { \
-        qknorm_rope_body<T, HD, ITER, true>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, blockIdx.x, v, cache_pos,   \
+        f16_t* k_cache, f16_t* v_cache, uint32_t capacity, int rows, int n_q, int n_kv, float eps, uint32_t* fault, int rot) { \
+        qknorm_rope_body<T, HD, ITER, true>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x, v, cache_pos,   \
                                             k_cache, v_cache, capacity, fault);                                   \
     }                                                                                                             \
     extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void apk_qknorm_rope_pairs_kv_##TN##_hd##HD##_i##ITER( \
         T* q, T* k, const T* v, const float* qw, const float* kw, const float* rope, const uint32_t* cache_pos,  \
-        f16_t* k_cache, f16_t* v_cache, uint32_t capacity, int rows, int n_q, int n_kv, float eps, uint32_t* fault) { \
-        qknorm_rope_body<T, HD, ITER, true, true>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, blockIdx.x, v, cache_pos, \
+        f16_t* k_cache, f16_t* v_cache, uint32_t capacity, int rows, int n_q, int n_kv, float eps, uint32_t* fault, int rot) { \
+        qknorm_rope_body<T, HD, ITER, true, true>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x, v, cache_pos, \
                                                   k_cache, v_cache, capacity, fault);                             \
     }
 #define APK_QKROPE_KV_ALL(T, TN)                                                                                       \
@@ -264,7 +287,7 @@ extern "C" __global__ __launch_bounds__(256) void apk_qknorm_rope_generic_f16(
         T* x, const T* delta, T* h, const float* gamma, int n, T* q, T* k, const float* qw, const float* kw,     \
         const float* rope, int rows, int n_q, int n_kv, float eps) {                                             \
         if (blockIdx.x < (uint32_t)rows) add_rmsnorm_body<T, 1>(x, delta, h, gamma, n, eps, blockIdx.x);         \
-        else qknorm_rope_body<T, HD, 1>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, blockIdx.x - (uint32_t)rows);  \
+        else qknorm_rope_body<T, HD, 1>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, HD, blockIdx.x - (uint32_t)rows);  \
     }
 APK_PROLOGUE(float, f32, 64) APK_PROLOGUE(float, f32, 128) APK_PROLOGUE(float, f32, 256)
 APK_PROLOGUE(f16_t, f16, 64) APK_PROLOGUE(f16_t, f16, 128) APK_PROLOGUE(f16_t, f16, 256)

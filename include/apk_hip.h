@@ -222,8 +222,9 @@ int apk_add_rmsnorm_rows(apk_ctx* ctx, void* x, const void* delta, void* h, cons
  * per row (the session table rows, model/session.rs:34-50).
  * rot_dim (even, <= head_dim) is the rotary width: pairs (i, i + rot_dim/2) rotate and
  * channels >= rot_dim are normalised and pass through (partial rotary, rope.rs:66-81).
- * head_dim in {64,128,256} with rot_dim == head_dim takes the tiled kernels; any other
- * geometry takes an element-wise kernel (a wave per head). */
+ * head_dim in {64,128,256} with a rotary width of whole 16-byte tiles (rot_dim/2 a multiple of
+ * 8 fp16 / 4 f32 elements; rot_dim itself for adjacent pairs) takes the tiled kernels; rot_dim = 0
+ * and any other geometry take an element-wise kernel (a wave per head, 2.5-4x slower). */
 int apk_qknorm_rope_neox(apk_ctx* ctx, void* q, void* k, const float* qw, const float* kw, const float* rope,
                          size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim, float eps,
                          int dtype);

@@ -450,6 +450,10 @@ def test_rope_only_and_reference_vectors(be, ora):
 @pytest.mark.parametrize("rows,n_q,n_kv,hd,rot", [
     (5, 4, 2, 128, 64),   # partial rotary on a tiled head size (GLM style)
     (3, 6, 2, 96, 96), (7, 5, 1, 80, 32), (2, 2, 2, 192, 192), (4, 3, 3, 32, 16), (1, 1, 1, 576, 64), (3, 2, 1, 128, 0),
+    # partial rotary over heads of 64 / 128 / 256: the tiled kernels where the rotary width is whole tiles, one and
+    # two passes per q wave; (128, 8) is whole tiles only for some of the style / type combinations
+    (300, 32, 8, 128, 64), (9, 8, 2, 256, 64), (33, 12, 2, 64, 32), (7, 4, 4, 128, 32), (5, 4, 2, 128, 96), (4, 3, 1, 128, 8),
+    (6, 2, 2, 64, 48), (700, 16, 2, 256, 128), (40, 20, 0, 128, 16),
 ])
 @pytest.mark.parametrize("style", [0, 1])
 @pytest.mark.parametrize("f16", [False, True])
@@ -536,7 +540,8 @@ def test_rope_table_on_device(be, ora):
 @pytest.mark.parametrize("rows,n_q,n_kv,hd,f16", [(1, 16, 8, 128, False), (64, 64, 8, 128, True), (300, 64, 8, 128, True),
                                                    (7, 4, 4, 64, False), (5, 2, 1, 256, True), (2048, 16, 8, 128, False)])
 @pytest.mark.parametrize("style", [0, 1])
-def test_qknorm_rope_kv_store(be, ora, rows, n_q, n_kv, hd, f16, style):
+@pytest.mark.parametrize("partial", [False, True])
+def test_qknorm_rope_kv_store(be, ora, rows, n_q, n_kv, hd, f16, style, partial):
     """QK-norm + RoPE with KvCache::store_at fused: q, k as the plain op; the cache rows hold
     the rotated k and the row's v narrowed to f16 (RNE) at each row's position."""
     s = synth()
@@ -544,6 +549,9 @@ def test_qknorm_rope_kv_store(be, ora, rows, n_q, n_kv, hd, f16, style):
     cap = max(rows + 9, 40)
     positions = g.permutation(cap)[:rows].astype(np.uint32)  # distinct cache rows, any order
     q, k, qw, kw, inv, ropes = _qk_case(ora, 3, rows, n_q, n_kv, hd, f16, [int(p) for p in positions])
+    rot = hd // 2 if partial else hd
+    if partial:  # only the leading half of every head rotates
+        ropes = ora.rope_table([int(p) for p in positions], ora.rope_inv_freq(rot, 1e6))
     v = s.normal_f32(g, (rows, n_kv * hd))
     if f16:
         v = s.to_f16_bits(v)
@@ -555,7 +563,7 @@ def test_qknorm_rope_kv_store(be, ora, rows, n_q, n_kv, hd, f16, style):
     kc = torch.zeros((cap, n_kv * hd), dtype=torch.float16, device="cuda")
     vc = torch.zeros_like(kc)
     be.qknorm_rope_kv_store(tq, tk, dev(v), dev(qw), dev(kw), dev(ropes), dev(positions), kc, vc, n_q, n_kv, hd, 1e-6,
-                            adjacent_pairs=bool(style))
+                            adjacent_pairs=bool(style), rot_dim=rot)
     gk = host(tk)
     for got, want in ((host(tq), wq), (gk, wk)):
         if f16:

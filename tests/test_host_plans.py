@@ -136,12 +136,14 @@ def test_add_rmsnorm_plans_cover_every_row_once(L, kernels, bounds):
 
 def test_qknorm_rope_plans_cover_every_head(L, kernels, bounds):
     for dtype, es in ((F32, 4), (F16, 2)):
-        for hd, rot, style in ((64, 64, 0), (128, 128, 0), (256, 256, 0), (128, 64, 0), (96, 96, 0), (128, 128, 1), (80, 0, 0), (2, 2, 1)):
+        for hd, rot, style in ((64, 64, 0), (128, 128, 0), (256, 256, 0), (128, 64, 0), (96, 96, 0), (128, 128, 1), (80, 0, 0), (2, 2, 1),
+                               (128, 64, 1), (256, 64, 0), (128, 8, 0), (128, 8, 1), (128, 0, 0), (64, 36, 1), (64, 48, 0)):
             for n_q, n_kv in ((64, 8), (32, 8), (16, 8), (40, 8), (28, 4), (8, 1), (1, 0), (0, 3), (12, 2), (96, 8), (5, 5)):
                 for rows in (1, 6, 64, 255, 512, 2048, 2061, 8192, 100000):
                     for kv in (0, 1):
                         rc, p = plan(L.apk_plan_qknorm_rope, rows, n_q, n_kv, hd, rot, style, dtype, kv)
-                        tiled = rot == hd and hd in (64, 128, 256)
+                        epl = 16 // es  # elements of a lane's 16-byte tile
+                        tiled = hd in (64, 128, 256) and rot > 0 and (rot % epl == 0 if style else (rot // 2) % epl == 0)
                         if kv and not tiled:
                             assert rc == 1
                             continue
