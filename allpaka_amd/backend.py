@@ -285,6 +285,14 @@ class Backend:
         check(self.L.apk_swiglu(self.h, _ptr(gate), _ptr(up), gate.numel(), _dt(gate)))
         self._leave()
 
+    def geglu_tanh(self, gate, up):
+        """ops::geglu_tanh (activation.rs:44-51): gate = gelu_tanh(gate) * up, the Gemma-family FFN gate."""
+        assert gate.numel() == up.numel()
+        assert gate.dtype == up.dtype
+        self._enter()
+        check(self.L.apk_geglu_tanh(self.h, _ptr(gate), _ptr(up), gate.numel(), _dt(gate)))
+        self._leave()
+
     # ---- model::route_gated (crates/allpaka-model/src/model/moe.rs:601)
     def route_rows(self, logits, k, gating=Gating.Softmax, norm=True, scale=1.0, bias=None):
         """route_gated_into_slice for every row of logits [rows, n_expert] -> (ids u32, w f32) [rows, k]."""

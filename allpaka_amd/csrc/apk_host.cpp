@@ -63,7 +63,7 @@ const int kQkIters[] = {1, 2};
 const int kQkHeadDims[] = {64, 128, 256};
 
 std::vector<std::string> all_kernel_names() {
-    std::vector<std::string> v = {"apk_swiglu_f32", "apk_swiglu_f16", "apk_rope_table", "apk_embed_q4k_f32",
+    std::vector<std::string> v = {"apk_swiglu_f32", "apk_swiglu_f16", "apk_geglu_tanh_f32", "apk_geglu_tanh_f16", "apk_rope_table", "apk_embed_q4k_f32",
                                   "apk_embed_q4k_f16", "apk_embed_q8_0_f32", "apk_embed_q8_0_f16", "apk_route_topk",
                                   "apk_moe_permute", "apk_gather_rows", "apk_scatter_rows_t1", "apk_scatter_rows_t2", "apk_argmax_rows", "apk_add_rmsnorm_ragged_f32", "apk_add_rmsnorm_ragged_f16", "apk_copy",
                                   "apk_qknorm_rope_generic_f32", "apk_qknorm_rope_generic_f16", "apk_route_topk_wide", "apk_route_topk_e64", "apk_route_topk_e128", "apk_route_group_small_e64", "apk_route_group_small_e128",
@@ -148,7 +148,7 @@ int launch(apk_ctx* c, const std::string& k, unsigned grid, unsigned block, unsi
 // The same for the ops of the decode chain, where the host's cost per launch is what bounds
 // the chain: the kernel of an (op, variant) pair is looked up by an integer; its name is built
 // only the first time.
-enum OpId : uint32_t { OP_SWIGLU = 1, OP_ADDNORM, OP_QKROPE, OP_QKROPE_KV, OP_PROLOGUE, OP_ADD_ASSIGN, OP_EMBED, OP_ARGMAX };
+enum OpId : uint32_t { OP_GEGLU = 20, OP_SWIGLU = 1, OP_ADDNORM, OP_QKROPE, OP_QKROPE_KV, OP_PROLOGUE, OP_ADD_ASSIGN, OP_EMBED, OP_ARGMAX };
 template <typename NameFn>
 int launch_keyed(apk_ctx* c, OpId op, uint32_t variant, NameFn&& name, unsigned grid, unsigned block, unsigned shmem,
                  void** args) {
@@ -740,6 +740,26 @@ int apk_swiglu(apk_ctx* c, void* gate, const void* up, size_t n, int dtype) {
     uint64_t n64 = n;
     void* args[] = {&gate, &up, &n64};
     return launch_keyed(c, OP_SWIGLU, (uint32_t)dtype, [&] { return std::string(dtype == APK_F32 ? "apk_swiglu_f32" : "apk_swiglu_f16"); },
+                        (unsigned)grid, block, 0, args);
+}
+
+int apk_geglu_tanh(apk_ctx* c, void* gate, const void* up, size_t n, int dtype) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_geglu_tanh: ctx is NULL");
+    CallScope s(c);
+    const int es = elem_size(dtype);
+    if (!es) return fail(APK_DECLINE_UNSUPPORTED, "apk_geglu_tanh: dtype %d", dtype);
+    if (n == 0) return APK_OK;
+    if (!gate || !up) return fail(APK_DECLINE_NULL, "apk_geglu_tanh: NULL tensor");
+    if (!aligned16(gate) || !aligned16(up)) return fail(APK_DECLINE_SHAPE, "apk_geglu_tanh: tensors must be 16-byte aligned");
+    if (int rc = set_device(c)) return rc;
+    const uint64_t vec = 16 / es, nvec = n / vec;
+    const unsigned block = 256, per_block = block;  // one 16-byte tile per lane
+    uint64_t grid = (nvec + per_block - 1) / per_block;
+    if (grid == 0) grid = 1;
+    if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_geglu_tanh: n too large");
+    uint64_t n64 = n;
+    void* args[] = {&gate, &up, &n64};
+    return launch_keyed(c, OP_GEGLU, (uint32_t)dtype, [&] { return std::string(dtype == APK_F32 ? "apk_geglu_tanh_f32" : "apk_geglu_tanh_f16"); },
                         (unsigned)grid, block, 0, args);
 }
 

@@ -1,20 +1,24 @@
-// gfx950 device code, part of apk_kernels.hip (one translation unit, one code object): SwiGLU, residual add, row softmax.
+// gfx950 device code, part of apk_kernels.hip (one translation unit, one code object): SwiGLU, GeGLU, residual add, row softmax.
 #pragma once
 
 // =========================================================================
 // SwiGLU: gate[i] = silu(gate[i]) * up[i], silu(x) = x / (1 + exp(-x))
 // (activation.rs:19-22, :116-119).  Pure stream: 2 reads + 1 write / element.
 // =========================================================================
-template <typename T> DEV float silu_mul(float g, float u);
+// Both gates are g * sigmoid(a) * u: a = g for SiLU; for the tanh GELU of GeGLU (activation.rs:44-51)
+// 0.5 g (1 + tanh z) = g * sigmoid(2z), z = sqrt(2/pi) g (1 + 0.044715 g^2) -- the form without the
+// cancellation of 1 + tanh z for negative z (there the reference's own f32 result carries the rounding of
+// its tanh, up to a few 1e-5 relative; this one stays within a few ulp of the exact value).
+template <typename T> DEV float sigmoid_gate(float g, float a, float u);
 // f32 activations: exp(-g) by Cody-Waite reduction around the hardware exp2 (log2(e) carried in
 // two parts, so the reduced argument is exact to the last bit: about 1 ulp over the whole range,
 // where a bare exp2(-g*log2e) loses |g| ulps), then the hardware reciprocal (1 ulp): the result is
 // within a few ulp of the reference's g / (1 + exp(-g)) * u -- 1e-6 of the 1e-5 bar -- at a third
 // of the instructions of libm expf + IEEE division, which at 32 per element no longer hid behind
 // the stream.
-template <> __device__ __forceinline__ float silu_mul<float>(float g, float u) {
+template <> __device__ __forceinline__ float sigmoid_gate<float>(float g, float a, float u) {
     const float L2E_HI = 1.44269502162933349609375f, L2E_LO = 1.925963033500011e-08f;  // hi + lo = log2(e)
-    const float n = fminf(fmaxf(-g, -104.0f), 89.0f);  // beyond: e underflows to 0 / overflows to inf anyway
+    const float n = fminf(fmaxf(-a, -104.0f), 89.0f);  // beyond: e underflows to 0 / overflows to inf anyway
     const float k = __builtin_rintf(n * L2E_HI);
     float r = __builtin_fmaf(n, L2E_HI, -k);
     r = __builtin_fmaf(n, L2E_LO, r);
@@ -22,17 +26,21 @@ template <> __device__ __forceinline__ float silu_mul<float>(float g, float u) {
     // the hardware reciprocal flushes subnormal results: keep 1/(1+e) normal for e up to FLT_MAX by
     // taking it of (1+e) * 2^-32 and applying the 2^-32 after the multiplication by g (all exact)
     const float sc = e > 0x1p96f ? 0x1p-32f : 1.0f;
-    return g * __builtin_amdgcn_rcpf((1.0f + e) * sc) * sc * u;  // NaN in g still gives NaN
+    return g * __builtin_amdgcn_rcpf((1.0f + e) * sc) * sc * u;  // NaN in g still gives NaN (a is a function of g)
 }
 // fp16 activations: the result is rounded to 11 bits, so the hardware exp2 /
 // rcp approximations (about 1 ulp of f32 each) are far inside the 2-ulp-of-fp16
 // budget and keep the kernel under its ALU ceiling.
-template <> __device__ __forceinline__ float silu_mul<f16_t>(float g, float u) {
-    float e = __builtin_amdgcn_exp2f(g * -1.4426950408889634f);
+template <> __device__ __forceinline__ float sigmoid_gate<f16_t>(float g, float a, float u) {
+    float e = __builtin_amdgcn_exp2f(a * -1.4426950408889634f);
     return g * __builtin_amdgcn_rcpf(1.0f + e) * u;
 }
+template <typename T, bool GELU> DEV float gate_mul(float g, float u) {
+    if constexpr (GELU) return sigmoid_gate<T>(g, 2.0f * (0.7978846f * g * (1.0f + 0.044715f * g * g)), u);
+    else return sigmoid_gate<T>(g, g, u);
+}
 
-template <typename T, int UNR> DEV void swiglu_body(T* gate, const T* up, uint64_t n) {
+template <typename T, int UNR, bool GELU = false> DEV void swiglu_body(T* gate, const T* up, uint64_t n) {
     constexpr int VEC = io<T>::VEC;
     const uint64_t nvec = n / VEC;
     const uint64_t base = (uint64_t)blockIdx.x * (blockDim.x * UNR) + threadIdx.x;
@@ -50,14 +58,14 @@ template <typename T, int UNR> DEV void swiglu_body(T* gate, const T* up, uint64
         uint64_t c = base + (uint64_t)j * blockDim.x;
         if (c < nvec) {
 #pragma unroll
-            for (int i = 0; i < VEC; i++) g[j][i] = silu_mul<T>(g[j][i], u[j][i]);
+            for (int i = 0; i < VEC; i++) g[j][i] = gate_mul<T, GELU>(g[j][i], u[j][i]);
             io<T>::store_nt(gate + c * VEC, g[j]);
         }
     }
     // ragged tail (n not a multiple of the 16-byte tile): last block, scalar
     if (blockIdx.x == gridDim.x - 1) {
         for (uint64_t i = nvec * VEC + threadIdx.x; i < n; i += blockDim.x)
-            gate[i] = (T)silu_mul<T>((float)gate[i], (float)up[i]);
+            gate[i] = (T)gate_mul<T, GELU>((float)gate[i], (float)up[i]);
     }
 }
 #define APK_SWIGLU_UNR 1  // measured: 1 tile per lane streams best (most waves in flight)
@@ -66,6 +74,13 @@ extern "C" __global__ __launch_bounds__(256) void apk_swiglu_f32(float* gate, co
 }
 extern "C" __global__ __launch_bounds__(256) void apk_swiglu_f16(f16_t* gate, const f16_t* up, uint64_t n) {
     swiglu_body<f16_t, APK_SWIGLU_UNR>(gate, up, n);
+}
+// GeGLU with the tanh GELU, the FFN gate of the Gemma family: gate[i] = gelu_tanh(gate[i]) * up[i].
+extern "C" __global__ __launch_bounds__(256) void apk_geglu_tanh_f32(float* gate, const float* up, uint64_t n) {
+    swiglu_body<float, APK_SWIGLU_UNR, true>(gate, up, n);
+}
+extern "C" __global__ __launch_bounds__(256) void apk_geglu_tanh_f16(f16_t* gate, const f16_t* up, uint64_t n) {
+    swiglu_body<f16_t, APK_SWIGLU_UNR, true>(gate, up, n);
 }
 
 // Residual add on its own: a[i] += b[i] (ops::add_assign_slice, blas.rs:105-178), for the

@@ -62,6 +62,7 @@ SYMBOLS = {
     "apk_layer_prologue": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _f, _i]),
     "apk_rope_table": (_i, [_vp, _vp, _vp, _sz, _sz, _vp]),
     "apk_swiglu": (_i, [_vp, _vp, _vp, _sz, _i]),
+    "apk_geglu_tanh": (_i, [_vp, _vp, _vp, _sz, _i]),
     "apk_route_topk": (_i, [_vp, _vp, _vp, _sz, _sz, _sz, _i, _f, _i, _vp, _vp]),
     "apk_moe_permute": (_i, [_vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp]),
     "apk_gather_rows": (_i, [_vp, _vp, _vp, _sz, _sz, _sz, _vp, _i]),

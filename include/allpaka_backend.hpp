@@ -197,6 +197,14 @@ inline void swiglu(std::vector<float>& gate, const std::vector<float>& up) {
     dg.read_back(gate.data());
 }
 
+// ops::geglu_tanh(gate, up): gate = gelu_tanh(gate) * up (activation.rs:44-51).
+inline void geglu_tanh(std::vector<float>& gate, const std::vector<float>& up) {
+    if (gate.size() != up.size()) throw Panic("assertion failed: gate.len() == up.len()");
+    Dev<float> dg(gate.data(), gate.size()), du(up.data(), up.size());
+    check(apk_geglu_tanh(Gpu::get().ctx(), dg.ptr(), du.ptr(), gate.size(), APK_F32));
+    dg.read_back(gate.data());
+}
+
 }  // namespace ops
 
 // QuantMat::{new,row,row_into} (quantmat/mod.rs:39-89): a quantised matrix whose rows are the embedding rows.

@@ -287,6 +287,15 @@ int apk_rope_table(apk_ctx* ctx, const uint32_t* positions, const float* inv_fre
 /* SwiGLU in place: gate[i] = silu(gate[i]) * up[i].  Replaces ops::swiglu
  * (ops/activation.rs:57-120, non-aarch64 arm). */
 int apk_swiglu(apk_ctx* ctx, void* gate, const void* up, size_t n, int dtype);
+/* gate[i] = gelu_tanh(gate[i]) * up[i] in place: GeGLU with the tanh GELU, the FFN gate of the Gemma
+ * family.  Replaces ops::geglu_tanh (ops/activation.rs:44-51; chosen instead of swiglu where
+ * GroupedCombine.gelu is set, model/moe.rs:122-127, gpu/types.rs:440-443; the reference's CUDA kernel of
+ * the same name, gpu/cuda/kernels.rs:361).  Computed as gate * sigmoid(2z) * up, which is the same
+ * function without the cancellation of 1 + tanh z: f32 results agree with the reference's to 1e-5
+ * relative where 1 + tanh z >= 0.1 and to the reference's own tolerance idiom |a-b| < 1e-5 (1 + |b|)
+ * everywhere (for very negative gates its f32 result carries the rounding of its tanh); fp16: 2 ulp
+ * where 1 + tanh z >= 0.1, the same idiom on the values elsewhere. */
+int apk_geglu_tanh(apk_ctx* ctx, void* gate, const void* up, size_t n, int dtype);
 
 /* MoE router: softmax (sigmoid != 0: sigmoid) over n_expert logits, top-k by
  * descending selection score (+ bias when given), ties -> lower expert id,

@@ -72,6 +72,10 @@ def lib():
         L.ora_silu.argtypes = [f32]
         L.ora_swiglu.argtypes = [vp, sz, vp, sz]
         L.ora_swiglu_f16.argtypes = [vp, vp, sz]
+        L.ora_geglu_tanh.argtypes = [vp, sz, vp, sz]
+        L.ora_geglu_tanh_f16.argtypes = [vp, vp, sz]
+        L.ora_gelu_tanh_mul.restype = f32
+        L.ora_gelu_tanh_mul.argtypes = [f32, f32]
         L.ora_softmax.argtypes = [vp, sz]
         L.ora_sigmoid.argtypes = [vp, sz]
         L.ora_route_gated.restype = sz
@@ -312,6 +316,23 @@ def swiglu(gate, up):
         if gate.size != up.size:
             raise OracleError("assert_eq!(gate.len(), up.len())")
         lib().ora_swiglu_f16(_p(gate), _p(up), gate.size)
+
+
+def gelu_tanh_mul(x, u):
+    return float(lib().ora_gelu_tanh_mul(float(np.float32(x)), float(np.float32(u))))
+
+
+def geglu_tanh(gate, up):
+    """ops::geglu_tanh (activation.rs:44-51) in place into gate; uint16 arrays: the fp16 storage form."""
+    if gate.dtype == np.float32:
+        _chk(up, np.float32)
+        if lib().ora_geglu_tanh(_p(gate), gate.size, _p(up), up.size):
+            raise OracleError("assert_eq!(gate.len(), up.len())")
+    else:
+        _chk(gate, np.uint16), _chk(up, np.uint16)
+        if gate.size != up.size:
+            raise OracleError("assert_eq!(gate.len(), up.len())")
+        lib().ora_geglu_tanh_f16(_p(gate), _p(up), gate.size)
 
 
 def softmax(x):

@@ -565,6 +565,17 @@ ORA_API int ora_swiglu(float *gate, size_t g_len, const float *up, size_t u_len)
     for (size_t i = 0; i < g_len; i++) gate[i] = ora_silu(gate[i]) * up[i];
     return 0;
 }
+/* activation.rs:44-51: GeGLU with the tanh GELU (Gemma's FFN), the same formula as ggml_gelu; every product
+ * in the reference's left-to-right order, tanhf from libm as Rust's f32::tanh.  1 = length assert. */
+ORA_API float ora_gelu_tanh_mul(float x, float u) {
+    const float SQRT_2_OVER_PI = 0.7978846f;
+    return 0.5f * x * (1.0f + tanhf(SQRT_2_OVER_PI * x * (1.0f + 0.044715f * x * x))) * u;
+}
+ORA_API int ora_geglu_tanh(float *gate, size_t g_len, const float *up, size_t u_len) {
+    if (g_len != u_len) return 1;
+    for (size_t i = 0; i < g_len; i++) gate[i] = ora_gelu_tanh_mul(gate[i], up[i]);
+    return 0;
+}
 /* activation.rs:5-16 (f32::max fold: a NaN operand is ignored) */
 ORA_API void ora_softmax(float *x, size_t n) {
     float mx = -INFINITY;
@@ -798,6 +809,10 @@ ORA_API void ora_qknorm_rope_rows_f16(uint16_t *q, uint16_t *k, size_t rows, siz
 ORA_API void ora_swiglu_f16(uint16_t *gate, const uint16_t *up, size_t n) {
     for (size_t i = 0; i < n; i++)
         gate[i] = ora_f32_to_f16(ora_silu(ora_f16_to_f32(gate[i])) * ora_f16_to_f32(up[i]));
+}
+ORA_API void ora_geglu_tanh_f16(uint16_t *gate, const uint16_t *up, size_t n) {
+    for (size_t i = 0; i < n; i++)
+        gate[i] = ora_f32_to_f16(ora_gelu_tanh_mul(ora_f16_to_f32(gate[i]), ora_f16_to_f32(up[i])));
 }
 ORA_API int ora_embed_rows_f16(const uint8_t *data, size_t data_len, int fmt, size_t vocab, size_t n_in,
                                const uint32_t *ids, size_t t, uint16_t *out) {

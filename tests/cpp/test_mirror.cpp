@@ -76,6 +76,22 @@ static void swiglu_is_silu_of_gate_times_up() {  // :172-185, silu fixed points 
     CHECK(g[0] == 0.0f && close(g[1], 1.0f / (1.0f + std::exp(-1.0f))) && std::fabs(g[2]) < 1e-7f && close(g[3], 20.0f));
     CHECK(throws<Panic>([] { std::vector<float> g(4), u(3); ops::swiglu(g, u); }));
 }
+static void geglu_tanh_is_the_tanh_gelu_of_gate_times_up() {  // activation.rs:44-51
+    auto gelu = [](float x) { return 0.5f * x * (1.0f + std::tanh(0.7978846f * x * (1.0f + 0.044715f * x * x))); };
+    std::vector<float> gate, up;
+    for (int i = -40; i <= 40; i++) { gate.push_back(0.25f * (float)i); up.push_back(1.0f + 0.01f * (float)i); }
+    std::vector<float> want(gate.size());
+    for (size_t i = 0; i < gate.size(); i++) want[i] = gelu(gate[i]) * up[i];
+    ops::geglu_tanh(gate, up);
+    for (size_t i = 0; i < gate.size(); i++) CHECK(close(gate[i], want[i]));
+    std::vector<float> z = {0.0f}, one = {3.0f};
+    ops::geglu_tanh(z, one);
+    CHECK(z[0] == 0.0f);  // gelu(0) = 0
+    std::vector<float> big = {30.0f, -30.0f}, u2 = {2.0f, 2.0f};
+    ops::geglu_tanh(big, u2);
+    CHECK(big[0] == 60.0f && std::fabs(big[1]) < 1e-20f);  // identity far right, zero far left
+    CHECK(throws<Panic>([] { std::vector<float> a(4), b(3); ops::geglu_tanh(a, b); }));
+}
 static void softmax_sums_to_one_and_survives_huge_logits() {  // ops/mod.rs:147-161
     std::vector<float> x = {1.0f, 3.0f, 2.0f};
     ops::softmax(x);
@@ -336,6 +352,7 @@ int main() {
         {"rmsnorm_rows_into_rejects_a_short_destination", rmsnorm_rows_into_rejects_a_short_destination},
         {"add_assign_then_norm_matches_the_two_ops", add_assign_then_norm_matches_the_two_ops},
         {"swiglu_is_silu_of_gate_times_up", swiglu_is_silu_of_gate_times_up},
+        {"geglu_tanh_is_the_tanh_gelu_of_gate_times_up", geglu_tanh_is_the_tanh_gelu_of_gate_times_up},
         {"softmax_sums_to_one_and_survives_huge_logits", softmax_sums_to_one_and_survives_huge_logits},
         {"add_assign_slice_adds_and_rejects_length_mismatch", add_assign_slice_adds_and_rejects_length_mismatch},
         {"rope_is_norm_preserving_and_identity_at_position_zero", rope_is_norm_preserving_and_identity_at_position_zero},

@@ -683,6 +683,51 @@ def test_swiglu_reference_sweep_and_assert(be, ora):
         be.swiglu(torch.zeros(4, device="cuda"), torch.zeros(3, device="cuda"))
 
 
+# --------------------------------------------------------------------- GeGLU (tanh)
+@pytest.mark.parametrize("n", [2304 * 4, 512 * 9216, 64 * 9216, 1, 5, 1031])
+@pytest.mark.parametrize("f16", [False, True])
+def test_geglu_tanh(be, ora, n, f16):
+    """ops::geglu_tanh (activation.rs:44-51), the FFN gate of the Gemma family.  The device computes
+    g * sigmoid(2z) * u, the same function as the reference's 0.5 g (1 + tanh z) u without the cancellation of
+    1 + tanh z: to 1e-5 relative where the reference's own rounding of tanh cannot show (1 + tanh z >= 0.1, i.e.
+    gates above about -0.9) and to the reference's tolerance idiom |a - b| < 1e-5 (1 + |b|) everywhere."""
+    s = synth()
+    g = s.rng(4, n + 77)
+    gate, up = s.normal_f32(g, n, 0.0, 2.0), s.normal_f32(g, n)
+    gate[: min(n, 8)] = np.float32([0.0, 1.0, -20.0, 20.0, -6.0, 6.0, -0.0, 1e-30])[: min(n, 8)]
+    if f16:
+        gate, up = s.to_f16_bits(gate), s.to_f16_bits(up)
+    want = gate.copy()
+    ora.geglu_tanh(want, up)
+    tg = dev(gate)
+    be.geglu_tanh(tg, dev(up))
+    got = host(tg)
+    if f16:
+        # where the reference's rounding of tanh cannot show: 2 ulp; further left its own f32 result is off by
+        # parts in 1e3 and more before it is rounded to fp16, so there the reference's tolerance idiom on the values
+        gv = gate.view(np.float16).astype(np.float32)
+        right = gv >= -0.9
+        assert not right.any() or f16_ulp_diff(got[right], want[right]) <= TOL_F16_ULP
+        key = lambda b: np.where(b.astype(np.int32) & 0x8000, 0x8000 - b.astype(np.int32), b.astype(np.int32))  # noqa: E731
+        a, b = got.view(np.float16).astype(np.float64), want.view(np.float16).astype(np.float64)
+        assert np.all((np.abs(key(got) - key(want)) <= TOL_F16_ULP) | (np.abs(a - b) < 1e-5 * (1.0 + np.abs(b))))
+    else:
+        assert close_idiom(got, want)
+        right = gate >= -0.9
+        assert not right.any() or rel_err_f32(got[right], want[right]) <= TOL_F32
+        # and against the closed form in float64, over the whole range, the device keeps the bar
+        gd, ud = gate.astype(np.float64), up.astype(np.float64)
+        with np.errstate(over="ignore"):  # 0.5 (1 + tanh z) = 1 / (1 + exp(-2z)), the form that does not cancel in float64 either
+            exact = gd * ud / (1.0 + np.exp(-2.0 * np.float64(np.float32(0.7978846)) * gd * (1.0 + np.float64(np.float32(0.044715)) * gd * gd)))
+        big = np.abs(exact) > 1e-30
+        assert not big.any() or np.max(np.abs(got[big] - exact[big]) / np.abs(exact[big])) <= TOL_F32  # z itself is an f32 product: |2z| ulps in exp(-2z)
+
+
+def test_geglu_tanh_asserts_equal_lengths(be):
+    with pytest.raises(AssertionError):
+        be.geglu_tanh(torch.zeros(4, device="cuda"), torch.zeros(3, device="cuda"))
+
+
 def test_fp16_special_values_follow_the_oracle(be, ora):
     """fp16 edges: sums that overflow to infinity, subnormal inputs and outputs, all-zero rows, signed zeros."""
     n = 1024

@@ -529,6 +529,43 @@ def test_silu_fixed_points_and_swiglu_sweep(ora):
         ora.swiglu(np.zeros(4, np.float32), np.zeros(3, np.float32))
 
 
+def test_geglu_tanh_vs_the_closed_form(ora):
+    """ops::geglu_tanh (activation.rs:44-51) has no known-answer test in the reference; pinned by its closed form
+    0.5 x (1 + tanh(sqrt(2/pi) x (1 + 0.044715 x^2))) u in float64 (the f32 result carries at most the rounding of
+    tanhf, 1 ulp of a value near 1, times |0.5 x u|), by gelu(0) = 0, the identity far right and zero far left, by
+    gelu(x) - gelu(-x) = x, and by a transposed-operand check (gate and up are not interchangeable)."""
+    x = np.float32([i * 0.173 for i in range(-60, 61)])
+    u = np.float32([1.5 - 0.02 * i for i in range(121)])
+    got = x.copy()
+    ora.geglu_tanh(got, u)
+    xd, ud = x.astype(np.float64), u.astype(np.float64)
+    want = 0.5 * xd * (1.0 + np.tanh(0.7978846 * xd * (1.0 + 0.044715 * xd * xd))) * ud
+    assert np.all(np.abs(got - want) <= 1.3e-7 * np.abs(xd * ud) + 4e-7 * np.abs(want))
+    right = x >= -1.0
+    assert np.allclose(got[right], want[right], rtol=5e-7, atol=0)
+    z = np.float32([0.0, 30.0, -30.0])
+    ora.geglu_tanh(z, np.float32([7.0, 2.0, 2.0]))
+    assert z[0] == 0.0 and z[1] == 60.0 and abs(z[2]) < 1e-20
+    a, b = x.copy(), (-x).copy()
+    one = np.ones_like(x)
+    ora.geglu_tanh(a, one)
+    ora.geglu_tanh(b, one)
+    assert np.allclose(a - b, x, rtol=0, atol=2e-6)  # gelu(x) - gelu(-x) = x
+    swapped = u.copy()
+    ora.geglu_tanh(swapped, x)
+    assert not np.allclose(swapped, got, rtol=1e-3, atol=1e-3)
+    assert ora.gelu_tanh_mul(1.0, 1.0) == pytest.approx(0.8411919906082768, rel=3e-7)  # gelu_tanh(1)
+    h = np.float32([0.5, -1.25, 3.0]).astype(np.float16).view(np.uint16)
+    hu = np.float32([2.0, 1.0, -0.5]).astype(np.float16).view(np.uint16)
+    hg = h.copy()
+    ora.geglu_tanh(hg, hu)
+    f = h.view(np.float16).astype(np.float32)
+    ora.geglu_tanh(f, hu.view(np.float16).astype(np.float32))
+    assert np.array_equal(hg, f.astype(np.float16).view(np.uint16))  # fp16: widen, the f32 op, one rounding
+    with pytest.raises(ora.OracleError):
+        ora.geglu_tanh(np.zeros(4, np.float32), np.zeros(3, np.float32))
+
+
 def test_softmax_known_answers(ora):
     # ops/mod.rs:146-161
     x = np.float32([1, 3, 2])
