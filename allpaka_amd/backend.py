@@ -179,6 +179,18 @@ class Backend:
         assert h.dtype == x.dtype
         self._rows(x, delta, h, gamma, n, rows, eps)
 
+    def postnorm_add_rmsnorm_rows(self, x, delta, post_gamma, h, gamma, eps):
+        """The sandwich norm of the Gemma family and the next norm in one pass: x += rmsnorm(delta) * post_gamma
+        (ops::rmsnorm on the projected rows, then add_assign_slice: decode.rs:581-584, :771-775), h = rmsnorm(x) * gamma.
+        delta may be overwritten with its normalised form."""
+        n = gamma.numel()
+        rows = x.numel() // n
+        assert x.numel() == rows * n == delta.numel() and h.numel() >= rows * n and post_gamma.numel() == n
+        assert x.dtype == delta.dtype == h.dtype
+        self._enter()
+        check(self.L.apk_postnorm_add_rmsnorm_rows(self.h, _ptr(x), _ptr(delta), _ptr(post_gamma), _ptr(h), _ptr(gamma), n, rows, eps, _dt(x)))
+        self._leave()
+
     def _rows(self, x, delta, h, gamma, n, rows, eps):
         assert gamma.dtype == torch.float32
         self._enter()

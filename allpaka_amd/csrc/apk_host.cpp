@@ -71,6 +71,7 @@ std::vector<std::string> all_kernel_names() {
     for (const char* t : {"f32", "f16"}) {
         for (const char* f : {"q5k", "q6k", "q2k", "q3k", "q5_0", "f16", "f32", "bf16"}) v.push_back(std::string("apk_embed_") + f + "_" + t);
         for (int c : kAddnormTiles) v.push_back(std::string("apk_add_rmsnorm_") + t + "_c" + std::to_string(c));
+        for (int c : kAddnormTiles) v.push_back(std::string("apk_postnorm_add_rmsnorm_") + t + "_c" + std::to_string(c));
         for (int l : {4, 8, 16, 32}) v.push_back(std::string("apk_add_rmsnorm_small_") + t + "_l" + std::to_string(l));
         for (int c : {1, 2, 4}) v.push_back(std::string("apk_combine_add_rmsnorm_") + t + "_c" + std::to_string(c));
         for (int hd : kQkHeadDims) v.push_back(std::string("apk_layer_prologue_") + t + "_hd" + std::to_string(hd));
@@ -302,7 +303,7 @@ int plan_embed(int fmt, size_t n_in, size_t t, int out_dtype, apk_plan* p) {
 }
 
 enum { ADDNORM_RAGGED = 0, ADDNORM_SMALL = 1, ADDNORM_TILED = 2 };
-int plan_add_rmsnorm(size_t n, size_t rows, int dtype, apk_plan* p) {
+int plan_add_rmsnorm(size_t n, size_t rows, int dtype, apk_plan* p, bool post = false) {
     plan_reset(p);
     const int es = elem_size(dtype);
     if (!es) return fail(APK_DECLINE_UNSUPPORTED, "apk_add_rmsnorm_rows: dtype %d", dtype);
@@ -320,7 +321,9 @@ int plan_add_rmsnorm(size_t n, size_t rows, int dtype, apk_plan* p) {
     // Resident waves: 16 per CU up to 10 tiles per lane (<= 128 VGPRs), 12 at 12 tiles (144 VGPRs),
     // 8 at 16 and 20 tiles (187 / 233 VGPRs).
     const size_t nchunks = n / vec;
-    const int max_nch = dtype == APK_F16 ? 10 : 20;
+    // (the sandwich-norm kernels hold the delta tiles through one more reduction: up to 10 tiles per lane,
+    // 140 / 176 VGPRs there, so fewer resident waves)
+    const int max_nch = (dtype == APK_F16 || post) ? 10 : 20;
     int nch = 0;
     size_t waves = 0;
     if (n % vec == 0) {
@@ -334,7 +337,8 @@ int plan_add_rmsnorm(size_t n, size_t rows, int dtype, apk_plan* p) {
             waves = w;
             if (rows * w <= 2048) break;
         }
-        const size_t resident = nch >= 16 ? 2048 : nch >= 12 ? 3072 : 4096;
+        const size_t resident = post ? (nch >= 10 ? (dtype == APK_F16 ? 3072 : 2048) : nch >= 8 ? 3072 : 4096)
+                                     : nch >= 16 ? 2048 : nch >= 12 ? 3072 : 4096;
         if (nch > 2 && rows * waves > resident) {
             const size_t w2 = (nchunks + 127) / 128;
             if (w2 * 64 <= 1024) {
@@ -374,7 +378,7 @@ int plan_add_rmsnorm(size_t n, size_t rows, int dtype, apk_plan* p) {
     // and four rows (waves) to a workgroup measure 1-3 % faster
     const unsigned rpb = (waves == 1 && rows >= 8192) ? 4 : 1;
     p->variant = ADDNORM_TILED;
-    plan_name(p, std::string("apk_add_rmsnorm_") + t + "_c" + std::to_string(nch));
+    plan_name(p, std::string(post ? "apk_postnorm_add_rmsnorm_" : "apk_add_rmsnorm_") + t + "_c" + std::to_string(nch));
     p->grid = (unsigned)(rpb > 1 ? (rows + rpb - 1) / rpb : rows);
     p->block = (unsigned)(rpb > 1 ? 256 : waves * 64);
     p->tiles_per_lane = (unsigned)nch;
@@ -827,6 +831,31 @@ int apk_add_rmsnorm_rows(apk_ctx* c, void* x, const void* delta, void* h, const 
                         args);
 }
 
+int apk_postnorm_add_rmsnorm_rows(apk_ctx* c, void* x, void* delta, const float* post_gamma, void* h, const float* gamma,
+                                  size_t n, size_t rows, float eps, int dtype) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_postnorm_add_rmsnorm_rows: ctx is NULL");
+    if (!elem_size(dtype)) return fail(APK_DECLINE_UNSUPPORTED, "apk_postnorm_add_rmsnorm_rows: dtype %d", dtype);
+    if (rows == 0) return APK_OK;
+    if (!x || !delta || !post_gamma || !h || !gamma) return fail(APK_DECLINE_NULL, "apk_postnorm_add_rmsnorm_rows: NULL tensor");
+    if (h == x || h == delta || x == delta) return fail(APK_DECLINE_SHAPE, "apk_postnorm_add_rmsnorm_rows: x, delta and h must be distinct");
+    apk_plan p;
+    if (int rc = plan_add_rmsnorm(n, rows, dtype, &p, true)) return rc;
+    if (p.variant != ADDNORM_TILED) {
+        // rows outside the tiled kernels (not whole 16-byte tiles, longer than they hold, short rows in bulk):
+        // the reference's own two steps, the delta normalised in place first
+        if (int rc = apk_add_rmsnorm_rows(c, delta, nullptr, delta, post_gamma, n, rows, eps, dtype)) return rc;
+        return apk_add_rmsnorm_rows(c, x, delta, h, gamma, n, rows, eps, dtype);
+    }
+    CallScope s(c);
+    if (!aligned16(x) || !aligned16(h) || !aligned16(gamma) || !aligned16(delta) || !aligned16(post_gamma))
+        return fail(APK_DECLINE_SHAPE, "apk_postnorm_add_rmsnorm_rows: tensors must be 16-byte aligned");
+    if (int rc = set_device(c)) return rc;
+    int n_i = (int)n;
+    uint32_t rows32 = (uint32_t)rows;
+    void* args[] = {&x, &delta, &h, &gamma, &n_i, &eps, &p.rows_per_block, &rows32, &post_gamma};
+    return launch(c, p.kernel, p.grid, p.block, 0, args);
+}
+
 struct KvStore {  // the fused K/V cache store of apk_qknorm_rope_kv_store (all NULL/0: plain op)
     const void* v = nullptr;
     const uint32_t* cache_pos = nullptr;
@@ -1256,6 +1285,11 @@ int apk_argmax_rows(apk_ctx* c, const float* logits, size_t rows, size_t n, uint
 int apk_plan_add_rmsnorm_rows(size_t n, size_t rows, int dtype, apk_plan* plan) {
     if (!plan) return fail(APK_DECLINE_NULL, "apk_plan_add_rmsnorm_rows: plan is NULL");
     return plan_add_rmsnorm(n, rows, dtype, plan);
+}
+
+int apk_plan_postnorm_add_rmsnorm_rows(size_t n, size_t rows, int dtype, apk_plan* plan) {
+    if (!plan) return fail(APK_DECLINE_NULL, "apk_plan_postnorm_add_rmsnorm_rows: plan is NULL");
+    return plan_add_rmsnorm(n, rows, dtype, plan, true);
 }
 
 int apk_plan_qknorm_rope(size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim, int adjacent_pairs, int dtype,

@@ -62,12 +62,18 @@ template <> struct headstat<f16_t> {
     }
 };
 
-template <typename T, int NCH, bool HAS_DELTA>
+// POST (with a delta): the delta is normalised first, x' = x + rmsnorm(delta) * post_gamma -- the sandwich
+// norm of the Gemma family (ops::rmsnorm on the projected row, then add_assign_slice: model/decode.rs:581-584,
+// :771-775; the reference's CUDA rmsnorm_add_f32, gpu/cuda/kernels.rs:376-406) -- one more reduction over the
+// row's delta tiles, which are in registers already; the delta itself is left as it was.
+template <typename T, int NCH, bool HAS_DELTA, bool POST = false>
 DEV void add_rmsnorm_impl(T* x, const T* delta, T* h, const float* gamma, int n, float eps, uint32_t vblock,
-                          uint32_t rows_per_block, uint32_t rows) {
+                          uint32_t rows_per_block, uint32_t rows, const float* post_gamma = nullptr) {
     constexpr int VEC = io<T>::VEC;
     typedef typename stat<T>::acc_t acc_t;
     __shared__ acc_t part[16];
+    typedef typename headstat<T>::acc_t dacc_t;  // the delta's norm feeds an addition that can cancel: the reference's values
+    __shared__ dacc_t part_d[POST ? 16 : 1];
     const int nchunks = n / VEC;
     // Two shapes of workgroup: all its waves share one row (rows_per_block == 1: few long rows), or
     // every wave has a row of its own (a wave covers the row with NCH tiles per lane; the workgroup
@@ -105,6 +111,28 @@ DEV void add_rmsnorm_impl(T* x, const T* delta, T* h, const float* gamma, int n,
     }
     __builtin_amdgcn_sched_barrier(0);  // keep every load above; all uses below
     float v[NCH][VEC];
+    typename headstat<T>::scale_t dscale{};
+    if constexpr (POST) {  // the delta's own statistics
+        dacc_t sd = 0;
+#pragma unroll
+        for (int j = 0; j < NCH; j++) {
+            const int c = tid + j * stride;
+            float d[VEC];
+            io<T>::widen(draw[j], d);
+            dacc_t s8 = 0;
+#pragma unroll
+            for (int i = 0; i < VEC; i++) s8 = headstat<T>::sq(s8, d[i]);
+            sd += c < nchunks ? s8 : (dacc_t)0;
+        }
+        sd = group_sum<64>(sd);
+        if (!own_row && blockDim.x > 64) {
+            if ((threadIdx.x & 63) == 0) part_d[threadIdx.x >> 6] = sd;
+            __syncthreads();
+            sd = 0;
+            for (int w = 0; w < (int)((blockDim.x + 63) >> 6); w++) sd += part_d[w];
+        }
+        dscale = headstat<T>::rscale(sd, n, eps);
+    }
     acc_t ss = 0;
 #pragma unroll
     for (int j = 0; j < NCH; j++) {
@@ -113,6 +141,25 @@ DEV void add_rmsnorm_impl(T* x, const T* delta, T* h, const float* gamma, int n,
         if constexpr (HAS_DELTA) {
             float d[VEC];
             io<T>::widen(draw[j], d);
+            if constexpr (POST) {
+                float pg[VEC];
+                const int cc = min(c, nchunks - 1);
+#pragma unroll
+                for (int q = 0; q < VEC; q += 4) io<float>::load(post_gamma + cc * VEC + q, pg + q);
+#pragma unroll
+                for (int i = 0; i < VEC; i++) d[i] = headstat<T>::apply(d[i], dscale, pg[i]);
+                if constexpr (sizeof(T) == 2) {  // the reference's projected row is an activation: rounded to the storage type
+                    // The f32 product is pinned in a register first: left alone the compiler folds "* post_gamma" and
+                    // the conversion into one mixed-precision fma that rounds the exact product once to fp16, which
+                    // differs from the f32 product rounded to fp16 wherever that product lands on an fp16 tie.
+#pragma unroll
+                    for (int i = 0; i < VEC; i++) {
+                        float r = d[i];
+                        asm volatile("" : "+v"(r));
+                        d[i] = (float)(T)r;
+                    }
+                }
+            }
 #pragma unroll
             for (int i = 0; i < VEC; i++) v[j][i] = v[j][i] + d[i];
             if (c < nchunks) io<T>::store(xr + c * VEC, v[j]);
@@ -251,9 +298,18 @@ extern "C" __global__ __launch_bounds__(256) void apk_add_rmsnorm_ragged_f16(f16
         T* x, const T* delta, T* h, const float* gamma, int n, float eps, uint32_t rows_per_block, uint32_t rows) { \
         add_rmsnorm_body<T, NCH>(x, delta, h, gamma, n, eps, blockIdx.x, rows_per_block, rows);              \
     }
+#define APK_POSTNORM(T, TN, NCH, MAXT)                                                                       \
+    extern "C" __global__ __launch_bounds__(MAXT) void apk_postnorm_add_rmsnorm_##TN##_c##NCH(               \
+        T* x, const T* delta, T* h, const float* gamma, int n, float eps, uint32_t rows_per_block, uint32_t rows, \
+        const float* post_gamma) {                                                                           \
+        add_rmsnorm_impl<T, NCH, true, true>(x, delta, h, gamma, n, eps, blockIdx.x, rows_per_block, rows, post_gamma); \
+    }
 #define APK_ADDNORM_ALL(T, TN)                                                                                   \
     APK_ADDNORM(T, TN, 1, 1024) APK_ADDNORM(T, TN, 2, 1024) APK_ADDNORM(T, TN, 3, 512) APK_ADDNORM(T, TN, 4, 512) \
     APK_ADDNORM(T, TN, 5, 256) APK_ADDNORM(T, TN, 6, 256) APK_ADDNORM(T, TN, 8, 256) APK_ADDNORM(T, TN, 10, 256)  \
-    APK_ADDNORM(T, TN, 12, 256) APK_ADDNORM(T, TN, 16, 256) APK_ADDNORM(T, TN, 20, 256)
+    APK_ADDNORM(T, TN, 12, 256) APK_ADDNORM(T, TN, 16, 256) APK_ADDNORM(T, TN, 20, 256)                          \
+    APK_POSTNORM(T, TN, 1, 1024) APK_POSTNORM(T, TN, 2, 1024) APK_POSTNORM(T, TN, 3, 512) APK_POSTNORM(T, TN, 4, 512) \
+    APK_POSTNORM(T, TN, 5, 256) APK_POSTNORM(T, TN, 6, 256) APK_POSTNORM(T, TN, 8, 256) APK_POSTNORM(T, TN, 10, 256) \
+    APK_POSTNORM(T, TN, 12, 256) APK_POSTNORM(T, TN, 16, 256) APK_POSTNORM(T, TN, 20, 256)
 APK_ADDNORM_ALL(float, f32)
 APK_ADDNORM_ALL(f16_t, f16)

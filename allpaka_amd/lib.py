@@ -73,6 +73,8 @@ SYMBOLS = {
     "apk_rope_inv_freq": (_i, [_sz, _f, _vp]),
     "apk_route_group": (_i, [_vp, _vp, _vp, _sz, _sz, _sz, _i, _f, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "apk_plan_add_rmsnorm_rows": (_i, [_sz, _sz, _i, _plan]),
+    "apk_plan_postnorm_add_rmsnorm_rows": (_i, [_sz, _sz, _i, _plan]),
+    "apk_postnorm_add_rmsnorm_rows": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _f, _i]),
     "apk_plan_qknorm_rope": (_i, [_sz, _sz, _sz, _sz, _sz, _i, _i, _i, _plan]),
     "apk_plan_scatter_rows": (_i, [_sz, _sz, _sz, _i, _plan]),
     "apk_plan_embed_rows": (_i, [_i, _sz, _sz, _i, _plan]),

@@ -126,6 +126,24 @@ inline void add_assign_then_rmsnorm_into(std::vector<float>& a, const std::vecto
     std::copy(out.begin(), out.end(), h.begin());
 }
 
+// The sandwich norm of the Gemma family and the norm that follows it (decode.rs:581-584 / :771-775, then :762-764):
+// ops::rmsnorm(delta, post_weight, eps); ops::add_assign_slice(a, delta); ops::rmsnorm_into(h, a, weight, eps) as one
+// launch.  `delta` itself is left as it was (the reference normalises it in place; nothing reads it afterwards).
+inline void postnorm_add_assign_then_rmsnorm_into(std::vector<float>& a, const std::vector<float>& delta,
+                                                  const std::vector<float>& post_weight, std::vector<float>& h,
+                                                  const std::vector<float>& weight, float eps) {
+    if (a.size() != delta.size()) throw Panic("assertion failed: a.len() == b.len()");
+    if (post_weight.size() != weight.size()) throw Panic("assertion failed: x.len() == weight.len()");
+    const size_t n = weight.size(), rows = a.size() / n;
+    if (h.size() < rows * n) throw Panic("dst holds fewer rows than src");
+    Dev<float> da(a.data(), a.size()), dd(delta.data(), delta.size()), dh(rows * n), dw(weight.data(), n), dp(post_weight.data(), n);
+    check(apk_postnorm_add_rmsnorm_rows(Gpu::get().ctx(), da.ptr(), dd.ptr(), dp.ptr(), dh.ptr(), dw.ptr(), n, rows, eps, APK_F32));
+    da.read_back(a.data());
+    std::vector<float> out(rows * n);
+    dh.read_back(out.data());
+    std::copy(out.begin(), out.end(), h.begin());
+}
+
 // ops::rope_inv_freq(head_dim, base) (rope.rs:8-12): host-side, as in the reference.
 inline std::vector<float> rope_inv_freq(size_t head_dim, float base) {
     std::vector<float> inv(head_dim / 2);

@@ -213,6 +213,18 @@ int apk_softmax_rows(apk_ctx* ctx, float* x, size_t rows, size_t n);
 int apk_add_rmsnorm_rows(apk_ctx* ctx, void* x, const void* delta, void* h, const float* gamma, size_t n,
                          size_t rows, float eps, int dtype);
 
+/* The sandwich norm of the Gemma family, then the next norm, in one pass:
+ *   x[r] += rmsnorm(delta[r]) * post_gamma;   h[r] = rmsnorm(x[r]) * gamma.
+ * Replaces ops::rmsnorm(projected, post_norm, eps); ops::add_assign_slice(x, projected) and the
+ * ops::rmsnorm_into that follows (model/decode.rs:581-584 and :771-775 with :762-764; the reference's CUDA
+ * rmsnorm_add_f32, gpu/cuda/kernels.rs:376-406; GroupedCombine.post_norm, gpu/types.rs:437-440).  Same
+ * arithmetic as apk_add_rmsnorm_rows for both norms; with fp16 activations the normalised delta is
+ * rounded to fp16 before the add, as the reference's in-place row would be.  One launch where
+ * apk_add_rmsnorm_rows would take its tiled kernels (the delta is then left unchanged); other rows run
+ * the reference's two steps and overwrite delta with its normalised form.  x, delta, h distinct. */
+int apk_postnorm_add_rmsnorm_rows(apk_ctx* ctx, void* x, void* delta, const float* post_gamma, void* h, const float* gamma,
+                                  size_t n, size_t rows, float eps, int dtype);
+
 /* Per-head QK-norm then NeoX RoPE, in place.  Replaces the loop
  * ops::rmsnorm(head, w, eps); ops::rope_neox_cached_from_array(head, rope_row)
  * over every q and k head of every row (model/attention.rs:131-165,
@@ -369,12 +381,13 @@ int apk_argmax_rows(apk_ctx* ctx, const float* logits, size_t rows, size_t n, ui
  * figures of the other kernels are calibrated against. */
 int apk_copy(apk_ctx* ctx, const void* src, void* dst, size_t bytes);
 
-/* Launch plans (no context, no GPU; see apk_plan): what apk_add_rmsnorm_rows, apk_qknorm_rope_neox /
+/* Launch plans (no context, no GPU; see apk_plan): what apk_add_rmsnorm_rows, apk_postnorm_add_rmsnorm_rows, apk_qknorm_rope_neox /
  * _norm (adjacent_pairs != 0) / _kv_store (with_kv_store != 0), apk_scatter_rows and apk_embed_rows /
  * apk_dequant_rows launch for these sizes.  Return APK_OK with plan filled (kernel "" and grid 0 when
  * the call would be a no-op), or the decline the entry itself would return for the sizes.  They have no
  * counterpart in the reference: its hosts size their dispatches inline (e.g. gpu/cuda/runtime/gemm.rs:218-233). */
 int apk_plan_add_rmsnorm_rows(size_t n, size_t rows, int dtype, apk_plan* plan);
+int apk_plan_postnorm_add_rmsnorm_rows(size_t n, size_t rows, int dtype, apk_plan* plan);
 int apk_plan_qknorm_rope(size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim, int adjacent_pairs, int dtype,
                          int with_kv_store, apk_plan* plan);
 int apk_plan_scatter_rows(size_t rows, size_t k, size_t cols, int dtype, apk_plan* plan);

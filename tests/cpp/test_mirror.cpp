@@ -64,6 +64,21 @@ static void add_assign_then_norm_matches_the_two_ops() {  // decode.rs:584 then 
     for (size_t i = 0; i < h.size(); i++) CHECK(h[i] == want[i]);
     CHECK(throws<Panic>([] { std::vector<float> a(64), b(8), h(64), w(64); ops::add_assign_then_rmsnorm_into(a, b, h, w, 0.0f); }));  // :396-401
 }
+static void sandwich_norm_matches_the_three_ops() {  // decode.rs:581-584, :771-775, then :762-764
+    const size_t n = 2304, rows = 5;
+    std::vector<float> a(rows * n), d(rows * n), h(rows * n), w(n), pw(n);
+    for (size_t i = 0; i < a.size(); i++) { a[i] = std::sin(0.1f * i); d[i] = 3.0f * std::cos(0.07f * i); }
+    for (size_t i = 0; i < n; i++) { w[i] = 1.0f + 0.001f * i; pw[i] = 0.5f + 0.0003f * i; }
+    std::vector<float> nd(rows * n), sum(a), want(rows * n);
+    ops::rmsnorm_rows_into(nd, d, pw, 1e-6f);
+    for (size_t i = 0; i < a.size(); i++) sum[i] = a[i] + nd[i];
+    ops::rmsnorm_rows_into(want, sum, w, 1e-6f);
+    const std::vector<float> d0(d);
+    ops::postnorm_add_assign_then_rmsnorm_into(a, d, pw, h, w, 1e-6f);
+    for (size_t i = 0; i < a.size(); i++) CHECK(a[i] == sum[i] && d[i] == d0[i]);
+    for (size_t i = 0; i < h.size(); i++) CHECK(h[i] == want[i]);
+    CHECK(throws<Panic>([] { std::vector<float> a(64), d(64), pw(32), h(64), w(64); ops::postnorm_add_assign_then_rmsnorm_into(a, d, pw, h, w, 0.0f); }));
+}
 static void swiglu_is_silu_of_gate_times_up() {  // :172-185, silu fixed points :163-170
     std::vector<float> gate, up;
     for (int i = -25; i < 26; i++) gate.push_back(i * 0.7f);
@@ -351,6 +366,7 @@ int main() {
         {"rmsnorm_eps_keeps_zero_input_finite", rmsnorm_eps_keeps_zero_input_finite},
         {"rmsnorm_rows_into_rejects_a_short_destination", rmsnorm_rows_into_rejects_a_short_destination},
         {"add_assign_then_norm_matches_the_two_ops", add_assign_then_norm_matches_the_two_ops},
+        {"sandwich_norm_matches_the_three_ops", sandwich_norm_matches_the_three_ops},
         {"swiglu_is_silu_of_gate_times_up", swiglu_is_silu_of_gate_times_up},
         {"geglu_tanh_is_the_tanh_gelu_of_gate_times_up", geglu_tanh_is_the_tanh_gelu_of_gate_times_up},
         {"softmax_sums_to_one_and_survives_huge_logits", softmax_sums_to_one_and_survives_huge_logits},

@@ -294,6 +294,54 @@ def test_add_rmsnorm_rows(be, ora, n, rows, f16, with_delta):
         assert np.mean(gh.view(np.uint32) == wh.view(np.uint32)) > 0.999  # f64 statistics: bit-equal almost everywhere
 
 
+@pytest.mark.parametrize("n,rows", [(2304, 1), (3584, 6), (1152, 64), (2560, 300), (3840, 2100), (5376, 700), (2560, 4200), (1024, 9000),
+                                    (8192, 3), (16384, 2),
+                                    # outside the tiled kernels: the two steps run
+                                    (1001, 5), (64, 100), (20488, 2)])
+@pytest.mark.parametrize("f16", [False, True])
+def test_postnorm_add_rmsnorm_rows(be, ora, n, rows, f16):
+    """The sandwich norm of the Gemma family and the next norm in one pass (decode.rs:581-584, :771-775, :762-764):
+    x += rmsnorm(delta) * post_gamma; h = rmsnorm(x) * gamma -- against the oracle's three ops in the reference's order."""
+    s = synth()
+    g = s.rng(1, n * 3 + rows)
+    x, d = s.normal_f32(g, (rows, n)), s.normal_f32(g, (rows, n), 0.0, 3.0)
+    pg, gamma = s.normal_f32(g, n, 1.0, 0.05), s.normal_f32(g, n, 1.0, 0.05)
+    if f16:
+        x, d = s.to_f16_bits(x), s.to_f16_bits(d)
+    nd = np.zeros_like(d)
+    ora.add_rmsnorm_rows(d.copy(), None, nd, pg, 1e-6)  # ops::rmsnorm(projected, post_norm, eps)
+    wx, wh = x.copy(), np.zeros_like(x)
+    ora.add_rmsnorm_rows(wx, nd, wh, gamma, 1e-6)       # add_assign_slice, then rmsnorm_into
+    tx, td, th = dev(x), dev(d), torch.zeros_like(dev(x))
+    be.postnorm_add_rmsnorm_rows(tx, td, dev(pg), th, dev(gamma), 1e-6)
+    gx, gh = host(tx), host(th)
+    if f16:
+        # one launch: the normalised delta is the reference's f32 value rounded once, so the sum is the oracle's bit for
+        # bit; as two steps the first is the plain fp16 row norm (1 ulp of the normalised delta in rare elements, which
+        # a cancelling sum magnifies): there the sum is held to 1 ulp of its larger operand
+        import allpaka_amd.lib as apklib
+
+        p = apklib.Plan()
+        assert be.L.apk_plan_postnorm_add_rmsnorm_rows(n, rows, 1, p) == 0
+        if p.kernel.startswith(b"apk_postnorm"):
+            assert np.array_equal(gx, wx)
+        else:
+            fv = lambda a: a.view(np.float16).astype(np.float64)  # noqa: E731
+            key = lambda b: np.where(b.astype(np.int32) & 0x8000, 0x8000 - b.astype(np.int32), b.astype(np.int32))  # noqa: E731
+            slack = 2.0 ** -10 * np.maximum(np.abs(fv(x)), np.abs(fv(nd)))
+            assert np.all((np.abs(key(gx) - key(wx)) <= TOL_F16_ULP) | (np.abs(fv(gx) - fv(wx)) <= slack))
+            assert np.mean(gx == wx) > 0.999
+        assert f16_ulp_diff(gh, wh) <= TOL_F16_ULP or not p.kernel.startswith(b"apk_postnorm")
+    else:
+        assert rel_err_f32(gx, wx) <= TOL_F32 and close_idiom(gx, wx)
+        assert rel_err_f32(gh, wh) <= TOL_F32 and close_idiom(gh, wh)
+        assert np.mean(gx.view(np.uint32) == wx.view(np.uint32)) > 0.999  # f64 statistics: bit-equal almost everywhere
+    import allpaka_amd as apk
+
+    with pytest.raises(apk.Declined):  # x, delta and h must be three tensors
+        be.postnorm_add_rmsnorm_rows(tx, tx, dev(pg), th, dev(gamma), 1e-6)
+
+
 def test_rmsnorm_reference_vectors_and_asserts(be, ora):
     # ops/mod.rs:119-144, :412-419
     x = torch.tensor([3.0, -4.0, 12.0, 0.0], device="cuda")

@@ -88,19 +88,25 @@ ROW_COUNTS = [1, 2, 6, 7, 8, 15, 16, 17, 33, 64, 100, 256, 511, 512, 1000, 1024,
               6000, 8191, 8192, 8193, 20000, 100000, 2**31 - 1]
 
 
-def test_add_rmsnorm_plans_cover_every_row_once(L, kernels, bounds):
+@pytest.mark.parametrize("post", [False, True])
+def test_add_rmsnorm_plans_cover_every_row_once(L, kernels, bounds, post):
+    """post: the sandwich-norm entry (its tiled kernels hold the delta through one more reduction: at most 10 tiles
+    per lane; rows outside the tiled kernels are planned as the plain entry plans them, and run as two steps)."""
     seen = set()
+    fn = L.apk_plan_postnorm_add_rmsnorm_rows if post else L.apk_plan_add_rmsnorm_rows
     for dtype, es in ((F32, 4), (F16, 2)):
         vec = 16 // es
         for n in ROW_LENGTHS:
             for rows in ROW_COUNTS:
-                rc, p = plan(L.apk_plan_add_rmsnorm_rows, n, rows, dtype)
+                rc, p = plan(fn, n, rows, dtype)
                 assert rc == 0, (n, rows, dtype)
                 name = common(p, kernels, bounds)
-                seen.add(re.sub(r"_(c|l)\d+$", "", name))
+                seen.add(re.sub(r"_(c|l)\d+$", "", name).replace("apk_postnorm_add_rmsnorm", "apk_add_rmsnorm"))
+                if post and "ragged" not in name and "small" not in name:
+                    assert name.startswith("apk_postnorm_add_rmsnorm_") and p.tiles_per_lane <= 10
                 nchunks = n // vec
                 if "ragged" in name:  # not whole tiles, or more than the register-tiled kernels hold (20480 elements)
-                    assert n % vec or n > 20480
+                    assert n % vec or n > (20480 if not post else 10240 * (2 if dtype == F16 else 1))
                     assert p.grid == rows and p.block == 256
                     continue
                 assert n % vec == 0
@@ -126,12 +132,12 @@ def test_add_rmsnorm_plans_cover_every_row_once(L, kernels, bounds):
     assert seen == {"apk_add_rmsnorm_f32", "apk_add_rmsnorm_f16", "apk_add_rmsnorm_small_f32", "apk_add_rmsnorm_small_f16",
                     "apk_add_rmsnorm_ragged_f32", "apk_add_rmsnorm_ragged_f16"}
     # the declines of the entry, and the no-op
-    assert plan(L.apk_plan_add_rmsnorm_rows, 1024, 4, 7)[0] == 1
-    assert plan(L.apk_plan_add_rmsnorm_rows, 0, 4, F32)[0] == 2
-    assert plan(L.apk_plan_add_rmsnorm_rows, 1024, 2**31, F32)[0] == 2
-    rc, p = plan(L.apk_plan_add_rmsnorm_rows, 1024, 0, F32)
+    assert plan(fn, 1024, 4, 7)[0] == 1
+    assert plan(fn, 0, 4, F32)[0] == 2
+    assert plan(fn, 1024, 2**31, F32)[0] == 2
+    rc, p = plan(fn, 1024, 0, F32)
     assert rc == 0 and p.grid == 0 and p.kernel == b""
-    assert L.apk_plan_add_rmsnorm_rows(1024, 4, F32, None) == 3
+    assert fn(1024, 4, F32, None) == 3
 
 
 def test_qknorm_rope_plans_cover_every_head(L, kernels, bounds):
