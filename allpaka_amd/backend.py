@@ -271,6 +271,46 @@ class Backend:
         if not self._recording and self.take_faults() & _l.FAULT_CACHE_RANGE:
             raise AssertionError("position past capacity")
 
+    def add_bias_rows(self, x, bias):
+        """add_bias_rows (model/loader.rs:519-523): x[r][i] += bias[i] over rows of bias.numel() elements."""
+        n = bias.numel()
+        assert n > 0 and x.numel() % n == 0 and bias.dtype == torch.float32
+        self._enter()
+        check(self.L.apk_add_bias_rows(self.h, _ptr(x), _ptr(bias), x.numel() // n, n, _dt(x)))
+        self._leave()
+
+    def attn_prologue_args(self, q, k, v, n_q, n_kv, head_dim, eps, rope_flat, q_bias=None, k_bias=None, v_bias=None, q_norm=None,
+                           k_norm=None, cache_pos=None, k_cache=None, v_cache=None, adjacent_pairs=False, rot_dim=None):
+        """The struct apk_attn_prologue for these tensors (kept alive by the caller)."""
+        rows = q.numel() // (n_q * head_dim) if n_q else k.numel() // (n_kv * head_dim)
+        rot_dim = head_dim if rot_dim is None else rot_dim
+        assert q.numel() == rows * n_q * head_dim and k.numel() == rows * n_kv * head_dim and rope_flat.numel() == rows * rot_dim
+        assert v is None or (v.numel() == k.numel() and v.dtype == k.dtype)
+        for b, heads in ((q_bias, n_q), (k_bias, n_kv), (v_bias, n_kv)):
+            assert b is None or (b.dtype == torch.float32 and b.numel() == heads * head_dim)
+        if k_cache is not None:
+            assert k_cache.dtype == v_cache.dtype == torch.float16 and k_cache.shape == v_cache.shape
+            assert k_cache.shape[1] == n_kv * head_dim and cache_pos.numel() == rows
+        a = _l.AttnPrologue()
+        a.q, a.k, a.v = _ptr(q), _ptr(k), _ptr(v)
+        a.q_bias, a.k_bias, a.v_bias = _ptr(q_bias), _ptr(k_bias), _ptr(v_bias)
+        a.q_norm, a.k_norm, a.rope = _ptr(q_norm), _ptr(k_norm), _ptr(rope_flat)
+        a.cache_pos, a.k_cache, a.v_cache = _ptr(cache_pos), _ptr(k_cache), _ptr(v_cache)
+        a.capacity = 0 if k_cache is None else k_cache.shape[0]
+        a.rows, a.n_q, a.n_kv, a.head_dim, a.rot_dim = rows, n_q, n_kv, head_dim, rot_dim
+        a.eps, a.dtype, a.adjacent_pairs = eps, _dt(q), int(adjacent_pairs)
+        return a
+
+    def attn_prologue_rows(self, q, k, v, n_q, n_kv, head_dim, eps, rope_flat, **kw):
+        """The q/k/v rows between the QKV projection and attention (attention.rs:125-165, kv.rs:682-697): optional
+        projection biases, optional per-head norms, the rotation, and the optional K/V cache store, as one call."""
+        a = self.attn_prologue_args(q, k, v, n_q, n_kv, head_dim, eps, rope_flat, **kw)
+        self._enter()
+        check(self.L.apk_attn_prologue_rows(self.h, C.byref(a)))
+        self._leave()
+        if kw.get("k_cache") is not None and not self._recording and self.take_faults() & _l.FAULT_CACHE_RANGE:
+            raise AssertionError("position past capacity")
+
     def layer_prologue(self, x, delta, h, gamma, q, k, q_norm, k_norm, rope_flat, n_q, n_kv, head_dim, eps):
         """add_rmsnorm_rows(x, delta, h, gamma) and qknorm_rope_neox(q, k, ...) as one launch
         (small decode batches; larger ones run as the two launches)."""

@@ -67,7 +67,8 @@ std::vector<std::string> all_kernel_names() {
                                   "apk_embed_q4k_f16", "apk_embed_q8_0_f32", "apk_embed_q8_0_f16", "apk_route_topk",
                                   "apk_moe_permute", "apk_gather_rows", "apk_scatter_rows_t1", "apk_scatter_rows_t2", "apk_argmax_rows", "apk_add_rmsnorm_ragged_f32", "apk_add_rmsnorm_ragged_f16", "apk_copy",
                                   "apk_qknorm_rope_generic_f32", "apk_qknorm_rope_generic_f16", "apk_route_topk_wide", "apk_route_topk_e64", "apk_route_topk_e128", "apk_route_group_small_e64", "apk_route_group_small_e128",
-                                  "apk_route_group_small_e256", "apk_route_group_small_e1024", "apk_add_assign_f32", "apk_add_assign_f16", "apk_softmax_rows", "apk_moe_count", "apk_moe_rank"};
+                                  "apk_route_group_small_e256", "apk_route_group_small_e1024", "apk_add_assign_f32", "apk_add_assign_f16", "apk_softmax_rows", "apk_moe_count", "apk_moe_rank",
+                                  "apk_add_bias_rows_f32", "apk_add_bias_rows_f16"};
     for (const char* t : {"f32", "f16"}) {
         for (const char* f : {"q5k", "q6k", "q2k", "q3k", "q5_0", "f16", "f32", "bf16"}) v.push_back(std::string("apk_embed_") + f + "_" + t);
         for (int c : kAddnormTiles) v.push_back(std::string("apk_add_rmsnorm_") + t + "_c" + std::to_string(c));
@@ -75,6 +76,12 @@ std::vector<std::string> all_kernel_names() {
         for (int l : {4, 8, 16, 32}) v.push_back(std::string("apk_add_rmsnorm_small_") + t + "_l" + std::to_string(l));
         for (int c : {1, 2, 4}) v.push_back(std::string("apk_combine_add_rmsnorm_") + t + "_c" + std::to_string(c));
         for (int hd : kQkHeadDims) v.push_back(std::string("apk_layer_prologue_") + t + "_hd" + std::to_string(hd));
+        for (int hd : kQkHeadDims)  // with the projection biases (two passes per q wave exist in fp16 only)
+            for (int it : kQkIters)
+                for (const char* style : {"", "pairs_"})
+                    for (const char* kv : {"", "kv_"})
+                        if (it == 1 || t[1] == '1')
+                            v.push_back(std::string("apk_qknorm_rope_") + style + kv + "bias_" + t + "_hd" + std::to_string(hd) + "_i" + std::to_string(it));
         for (int hd : kQkHeadDims)
             for (int it : kQkIters) {
                 for (const char* style : {"", "pairs_"})
@@ -196,8 +203,9 @@ void plan_name(apk_plan* p, const std::string& k) { snprintf(p->kernel, sizeof p
 
 enum { QK_TILED = 0, QK_GENERIC = 1 };
 // style: 0 = NeoX pairs (i, i + rot_dim/2), 1 = adjacent pairs (2i, 2i+1); with_kv: the K/V cache store fused in
+// with_bias: the kernels that also add the projection biases
 int plan_qknorm_rope(size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim, int style, int dtype, bool with_kv,
-                     apk_plan* p) {
+                     apk_plan* p, bool with_bias = false) {
     plan_reset(p);
     const int es = elem_size(dtype);
     if (!es) return fail(APK_DECLINE_UNSUPPORTED, "apk_qknorm_rope: dtype %d", dtype);
@@ -242,8 +250,8 @@ int plan_qknorm_rope(size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size
     const uint64_t grid = (waves * 64 + block - 1) / block;
     if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope: too large");
     p->variant = QK_TILED;
-    plan_name(p, std::string("apk_qknorm_rope_") + (style ? "pairs_" : "") + (with_kv ? "kv_" : "") + t + "_hd" + std::to_string(head_dim) +
-                     "_i" + std::to_string(iter));
+    plan_name(p, std::string("apk_qknorm_rope_") + (style ? "pairs_" : "") + (with_kv ? "kv_" : "") + (with_bias ? "bias_" : "") + t + "_hd" +
+                     std::to_string(head_dim) + "_i" + std::to_string(iter));
     p->grid = (unsigned)grid;
     p->block = block;
     p->tiles_per_lane = iter;
@@ -856,6 +864,12 @@ int apk_postnorm_add_rmsnorm_rows(apk_ctx* c, void* x, void* delta, const float*
     return launch(c, p.kernel, p.grid, p.block, 0, args);
 }
 
+struct QkvBias {  // the projection biases of apk_attn_prologue_rows (f32; any of them NULL: none for that tensor)
+    const float* q = nullptr;
+    const float* k = nullptr;
+    const float* v = nullptr;  // only with the cache store: added to v in place and to the cached row
+};
+
 struct KvStore {  // the fused K/V cache store of apk_qknorm_rope_kv_store (all NULL/0: plain op)
     const void* v = nullptr;
     const uint32_t* cache_pos = nullptr;
@@ -868,9 +882,10 @@ struct KvStore {  // the fused K/V cache store of apk_qknorm_rope_kv_store (all 
 // check, no launch (so a caller that chains two ops can decline before the first one runs).
 static int qknorm_rope_common(apk_ctx* c, void* q, void* k, const float* qw, const float* kw, const float* rope, size_t rows,
                               size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim, float eps, int dtype,
-                              const KvStore* kv, int style = 0, bool validate_only = false) {
+                              const KvStore* kv, int style = 0, bool validate_only = false, const QkvBias* bias = nullptr) {
     apk_plan p;
-    if (int rc = plan_qknorm_rope(rows, n_q, n_kv, head_dim, rot_dim, style, dtype, kv != nullptr, &p)) return rc;
+    if (bias && !bias->q && !bias->k && !bias->v) bias = nullptr;
+    if (int rc = plan_qknorm_rope(rows, n_q, n_kv, head_dim, rot_dim, style, dtype, kv != nullptr, &p, bias != nullptr)) return rc;
     if (rows == 0 || n_q + n_kv == 0) return APK_OK;
     if ((n_q && !q) || (n_kv && !k) || (!rope && rot_dim)) return fail(APK_DECLINE_NULL, "apk_qknorm_rope: NULL tensor");
     if ((q && !aligned16(q)) || (k && !aligned16(k)) || !aligned16(rope) || (qw && !aligned16(qw)) || (kw && !aligned16(kw)))
@@ -881,16 +896,33 @@ static int qknorm_rope_common(apk_ctx* c, void* q, void* k, const float* qw, con
             return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_kv_store: tensors must be 16-byte aligned");
         if (kv->capacity == 0 || kv->capacity > 0xffffffffu) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_kv_store: capacity");
     }
+    QkvBias nb;
+    if (bias) {
+        nb = *bias;
+        if ((nb.q && !aligned16(nb.q)) || (nb.k && !aligned16(nb.k)) || (nb.v && !aligned16(nb.v)))
+            return fail(APK_DECLINE_SHAPE, "apk_attn_prologue_rows: biases must be 16-byte aligned");
+        if (nb.v && !kv) return fail(APK_DECLINE_SHAPE, "apk_attn_prologue_rows: v_bias rides on the cache store here");
+    }
     if (validate_only) return APK_OK;
     if (int rc = set_device(c)) return rc;
     int rows_i = (int)rows, nq_i = (int)n_q, nkv_i = (int)n_kv, rot_i = (int)rot_dim;
     if (p.variant == QK_GENERIC) {
         int hd_i = (int)head_dim, half_i = (int)(rot_dim / 2);
-        void* gargs[] = {&q, &k, &qw, &kw, &rope, &rows_i, &nq_i, &nkv_i, &hd_i, &half_i, &style, &eps};
+        void* gargs[] = {&q, &k, &qw, &kw, &rope, &rows_i, &nq_i, &nkv_i, &hd_i, &half_i, &style, &eps, &nb.q, &nb.k};
         return launch(c, p.kernel, p.grid, p.block, 0, gargs);
     }
     auto which = [&] { return std::string(p.kernel); };
-    const uint32_t variant = (uint32_t)style << 20 | (uint32_t)dtype << 16 | (uint32_t)head_dim << 4 | p.tiles_per_lane;
+    const uint32_t variant = (uint32_t)(bias != nullptr) << 21 | (uint32_t)style << 20 | (uint32_t)dtype << 16 | (uint32_t)head_dim << 4 | p.tiles_per_lane;
+    if (kv && bias) {
+        uint32_t cap32 = (uint32_t)kv->capacity;
+        void* kargs[] = {&q, &k, (void*)&kv->v, &qw, &kw, &rope, (void*)&kv->cache_pos, (void*)&kv->k_cache, (void*)&kv->v_cache,
+                         &cap32, &rows_i, &nq_i, &nkv_i, &eps, &c->fault_dev, &rot_i, &nb.q, &nb.k, &nb.v};
+        return launch_keyed(c, OP_QKROPE_KV, variant, which, p.grid, p.block, 0, kargs);
+    }
+    if (bias) {
+        void* bargs[] = {&q, &k, &qw, &kw, &rope, &rows_i, &nq_i, &nkv_i, &eps, &rot_i, &nb.q, &nb.k};
+        return launch_keyed(c, OP_QKROPE, variant, which, p.grid, p.block, 0, bargs);
+    }
     if (kv) {
         uint32_t cap32 = (uint32_t)kv->capacity;
         void* kargs[] = {&q, &k, (void*)&kv->v, &qw, &kw, &rope, (void*)&kv->cache_pos, (void*)&kv->k_cache, (void*)&kv->v_cache,
@@ -933,6 +965,55 @@ int apk_qknorm_rope_norm_kv_store(apk_ctx* c, void* q, void* k, const void* v, c
     KvStore kv;
     kv.v = v; kv.cache_pos = cache_pos; kv.k_cache = k_cache; kv.v_cache = v_cache; kv.capacity = capacity;
     return qknorm_rope_common(c, q, k, qw, kw, rope, rows, n_q, n_kv, head_dim, rot_dim, eps, dtype, &kv, 1);
+}
+
+// the caller holds the context (CallScope)
+static int add_bias_rows_locked(apk_ctx* c, void* x, const float* bias, size_t rows, size_t n, int dtype) {
+    const int es = elem_size(dtype);
+    if (!es) return fail(APK_DECLINE_UNSUPPORTED, "apk_add_bias_rows: dtype %d", dtype);
+    if (rows == 0 || n == 0) return APK_OK;
+    if (!x || !bias) return fail(APK_DECLINE_NULL, "apk_add_bias_rows: NULL tensor");
+    if (!aligned16(x) || !aligned16(bias)) return fail(APK_DECLINE_SHAPE, "apk_add_bias_rows: tensors must be 16-byte aligned");
+    if (n > 0xffffffffu || rows > ((uint64_t)1 << 40) / n) return fail(APK_DECLINE_SHAPE, "apk_add_bias_rows: sizes out of range");
+    if (int rc = set_device(c)) return rc;
+    const size_t vec = 16 / es;
+    const uint64_t lanes = n % vec == 0 ? (uint64_t)rows * (n / vec) : (uint64_t)rows * n;
+    const uint64_t grid = (lanes + 255) / 256;
+    if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_add_bias_rows: too large");
+    uint64_t rows64 = rows;
+    uint32_t n32 = (uint32_t)n;
+    void* args[] = {&x, &bias, &rows64, &n32};
+    return launch(c, dtype == APK_F32 ? "apk_add_bias_rows_f32" : "apk_add_bias_rows_f16", (unsigned)grid, 256, 0, args);
+}
+
+int apk_add_bias_rows(apk_ctx* c, void* x, const float* bias, size_t rows, size_t n, int dtype) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_add_bias_rows: ctx is NULL");
+    CallScope s(c);
+    return add_bias_rows_locked(c, x, bias, rows, n, dtype);
+}
+
+int apk_attn_prologue_rows(apk_ctx* c, const apk_attn_prologue* a) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_attn_prologue_rows: ctx is NULL");
+    if (!a) return fail(APK_DECLINE_NULL, "apk_attn_prologue_rows: args is NULL");
+    CallScope s(c);
+    const bool store = a->k_cache || a->v_cache || a->cache_pos;
+    KvStore kv;
+    kv.v = a->v; kv.cache_pos = a->cache_pos; kv.k_cache = a->k_cache; kv.v_cache = a->v_cache; kv.capacity = a->capacity;
+    QkvBias bias;
+    bias.q = a->q_bias; bias.k = a->k_bias;
+    bias.v = store ? a->v_bias : nullptr;
+    const int style = a->adjacent_pairs ? 1 : 0;
+    if (a->v_bias && !store && a->rows && a->n_kv) {
+        // no cache store: v is not read by the q/k kernel, its bias is a launch of its own -- after every check of
+        // the main op, so that a decline leaves v as it was
+        if (int rc = qknorm_rope_common(c, a->q, a->k, a->q_norm, a->k_norm, a->rope, a->rows, a->n_q, a->n_kv, a->head_dim, a->rot_dim,
+                                        a->eps, a->dtype, nullptr, style, true, &bias))
+            return rc;
+        if (!a->v) return fail(APK_DECLINE_NULL, "apk_attn_prologue_rows: v_bias without v");
+        if (int rc = add_bias_rows_locked(c, a->v, a->v_bias, a->rows, a->n_kv * a->head_dim, a->dtype)) return rc;
+    }
+    return qknorm_rope_common(c, a->q, a->k, a->q_norm, a->k_norm, a->rope, a->rows, a->n_q, a->n_kv, a->head_dim, a->rot_dim, a->eps,
+                              a->dtype, store ? &kv : nullptr, style, false, &bias);
 }
 
 int apk_layer_prologue(apk_ctx* c, void* x, const void* delta, void* h, const float* gamma, size_t n, void* q, void* k,
@@ -1296,6 +1377,13 @@ int apk_plan_qknorm_rope(size_t rows, size_t n_q, size_t n_kv, size_t head_dim, 
                          int with_kv_store, apk_plan* plan) {
     if (!plan) return fail(APK_DECLINE_NULL, "apk_plan_qknorm_rope: plan is NULL");
     return plan_qknorm_rope(rows, n_q, n_kv, head_dim, rot_dim, adjacent_pairs ? 1 : 0, dtype, with_kv_store != 0, plan);
+}
+
+int apk_plan_attn_prologue_rows(const apk_attn_prologue* a, apk_plan* plan) {
+    if (!plan || !a) return fail(APK_DECLINE_NULL, "apk_plan_attn_prologue_rows: NULL argument");
+    const bool store = a->k_cache || a->v_cache || a->cache_pos;
+    const bool bias = a->q_bias || a->k_bias || (store && a->v_bias);
+    return plan_qknorm_rope(a->rows, a->n_q, a->n_kv, a->head_dim, a->rot_dim, a->adjacent_pairs ? 1 : 0, a->dtype, store, plan, bias);
 }
 
 int apk_plan_scatter_rows(size_t rows, size_t k, size_t cols, int dtype, apk_plan* plan) {

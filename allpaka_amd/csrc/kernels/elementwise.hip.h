@@ -106,6 +106,34 @@ extern "C" __global__ __launch_bounds__(256) void apk_add_assign_f16(f16_t* a, c
     add_assign_body<f16_t>(a, b, n);
 }
 
+// A per-row bias: x[r][i] += bias[i] (add_bias_rows, crates/allpaka-model/src/model/loader.rs:519-523: the
+// projection biases of attention.rs:125-129).  Whole 16-byte tiles where the row length allows, else per element.
+template <typename T> DEV void add_bias_rows_body(T* x, const float* bias, uint64_t rows, uint32_t n) {
+    constexpr int VEC = io<T>::VEC;
+    const uint64_t c = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (n % VEC == 0) {  // uniform
+        const uint32_t tiles = n / VEC;
+        if (c >= rows * tiles) return;
+        const uint32_t col = (uint32_t)(c % tiles) * VEC;
+        float v[VEC], b[VEC];
+        io<T>::load_nt(x + c * VEC, v);
+#pragma unroll
+        for (int q = 0; q < VEC; q += 4) io<float>::load(bias + col + q, b + q);
+#pragma unroll
+        for (int i = 0; i < VEC; i++) v[i] += b[i];
+        io<T>::store_nt(x + c * VEC, v);
+    } else {
+        if (c >= rows * n) return;
+        x[c] = (T)((float)x[c] + bias[c % n]);
+    }
+}
+extern "C" __global__ __launch_bounds__(256) void apk_add_bias_rows_f32(float* x, const float* bias, uint64_t rows, uint32_t n) {
+    add_bias_rows_body<float>(x, bias, rows, n);
+}
+extern "C" __global__ __launch_bounds__(256) void apk_add_bias_rows_f16(f16_t* x, const float* bias, uint64_t rows, uint32_t n) {
+    add_bias_rows_body<f16_t>(x, bias, rows, n);
+}
+
 // Softmax over rows in place (ops::softmax, activation.rs:5-16): max, exp(v - max), sum,
 // times 1/sum.  A wave per row, any row length; the sum runs in lane order, not index order.
 extern "C" __global__ __launch_bounds__(256) void apk_softmax_rows(float* x, int rows, int n) {

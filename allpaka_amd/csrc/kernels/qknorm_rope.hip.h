@@ -32,9 +32,14 @@
 // table row then has rot/2 entries.  With adjacent pairs a whole tile either rotates or does not (rot is a
 // multiple of the tile); with NeoX pairs (i, i + rot/2) the first rot/2/EPL lanes of a head take the partner
 // tiles at i and i + rot/2, the others two consecutive tiles of the tail.  rot == HD is the layout above.
-template <typename T, int HD, int ITER, bool KV = false, bool PAIRS = false>
+// BIAS = true: the projection biases of models that carry them (attention.rs:125-129: add_bias_rows on q, k and
+// v right in front of this loop; loader.rs:519-523) are added as the tiles are widened: bias [nheads*HD] f32 for the
+// item's tensor (NULL: none); with the cache store, vbias is added to the row's v, which is written back (vout)
+// as well as narrowed into the cache.
+template <typename T, int HD, int ITER, bool KV = false, bool PAIRS = false, bool BIAS = false>
 DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, float eps, int l, int sub, int rot,
-                 f16_t* kc = nullptr, const T* vrow = nullptr, f16_t* vc = nullptr) {
+                 f16_t* kc = nullptr, const T* vrow = nullptr, f16_t* vc = nullptr, const float* bias = nullptr,
+                 const float* vbias = nullptr, T* vout = nullptr) {
     constexpr int EPL = io<T>::VEC;   // elements per lane per half
     constexpr int HALF = HD / 2;
     constexpr int LPH = HALF / EPL;   // lanes per head
@@ -76,6 +81,7 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
         io<float>::load(wp + w_b + i, wb + i);
     }
     typename io<T>::raw_t araw[ITER], braw[ITER], varaw[ITER], vbraw[ITER];
+    float ba[BIAS ? ITER : 1][EPL], bb[BIAS ? ITER : 1][EPL], bva[BIAS && KV ? ITER : 1][EPL], bvb[BIAS && KV ? ITER : 1][EPL];
     // head of pass `it` and its element offset: recomputed where needed (a few integer
     // operations) rather than kept in registers across the loads
     const int hh_first = g * ITER * HPW + sub;
@@ -84,6 +90,24 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
     for (int it = 0; it < ITER; it++) {
         const int off = head_off(it);
         __builtin_amdgcn_sched_barrier(0);  // loads stay in program order (returns are in order)
+        if constexpr (BIAS) {  // uniform branches: a tensor has a bias or it has none
+            if (bias) {
+#pragma unroll
+                for (int i = 0; i < EPL; i += 4) {
+                    io<float>::load(bias + off + off_a + i, ba[it] + i);
+                    io<float>::load(bias + off + off_b + i, bb[it] + i);
+                }
+            }
+            if constexpr (KV) {
+                if (vbias) {
+#pragma unroll
+                    for (int i = 0; i < EPL; i += 4) {
+                        io<float>::load(vbias + off + off_a + i, bva[it] + i);
+                        io<float>::load(vbias + off + off_b + i, bvb[it] + i);
+                    }
+                }
+            }
+        }
         araw[it] = io<T>::ldraw_nt(base + off + off_a);
         braw[it] = io<T>::ldraw_nt(base + off + off_b);
         if constexpr (KV) {
@@ -98,6 +122,15 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
         float a[EPL], b[EPL], oa[EPL], ob[EPL];
         io<T>::widen(araw[it], a);
         io<T>::widen(braw[it], b);
+        if constexpr (BIAS) {
+            if (bias) {
+#pragma unroll
+                for (int i = 0; i < EPL; i++) {
+                    a[i] += ba[it][i];
+                    b[i] += bb[it][i];
+                }
+            }
+        }
         acc_t ss = 0;
 #pragma unroll
         for (int i = 0; i < EPL; i++) {
@@ -142,25 +175,39 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
             io<T>::store_nt(base + off + off_b, ob);
         }
         if constexpr (KV) {
-            if (live && kc != nullptr) {  // kc == nullptr: cache position out of range, row skipped
+            if (live) {
                 float va[EPL], vb[EPL];
                 io<T>::widen(varaw[it], va);
                 io<T>::widen(vbraw[it], vb);
-                store_f16_tile<T>(kc + off + off_a, oa);
-                store_f16_tile<T>(kc + off + off_b, ob);
-                store_f16_tile<T>(vc + off + off_a, va);
-                store_f16_tile<T>(vc + off + off_b, vb);
+                if constexpr (BIAS) {
+                    if (vbias) {
+#pragma unroll
+                        for (int i = 0; i < EPL; i++) {
+                            va[i] += bva[it][i];
+                            vb[i] += bvb[it][i];
+                        }
+                        io<T>::store_nt(vout + off + off_a, va);
+                        io<T>::store_nt(vout + off + off_b, vb);
+                    }
+                }
+                if (kc != nullptr) {  // kc == nullptr: cache position out of range, the row's cache store is skipped
+                    store_f16_tile<T>(kc + off + off_a, oa);
+                    store_f16_tile<T>(kc + off + off_b, ob);
+                    store_f16_tile<T>(vc + off + off_a, va);
+                    store_f16_tile<T>(vc + off + off_b, vb);
+                }
             }
         }
         __builtin_amdgcn_sched_barrier(0);  // pass by pass: pass it+1 waits only for its own tiles
     }
 }
 
-template <typename T, int HD, int ITERQ, bool KV = false, bool PAIRS = false>
+template <typename T, int HD, int ITERQ, bool KV = false, bool PAIRS = false, bool BIAS = false>
 DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv,
-                          float eps, int rot, uint32_t vblock, const T* v = nullptr, const uint32_t* cache_pos = nullptr,
+                          float eps, int rot, uint32_t vblock, T* v = nullptr, const uint32_t* cache_pos = nullptr,
                           f16_t* k_cache = nullptr, f16_t* v_cache = nullptr, uint32_t capacity = 0,
-                          uint32_t* fault = nullptr) {
+                          uint32_t* fault = nullptr, const float* qb = nullptr, const float* kb = nullptr,
+                          const float* vb = nullptr) {
     constexpr int LPH = HD / 2 / io<T>::VEC, HPW = 64 / LPH;
     const int lane = threadIdx.x & 63;
     const int l = lane % LPH, sub = lane / LPH;
@@ -171,7 +218,8 @@ DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const fl
     if (wid >= nq_items + (uint64_t)rows * gk) return;  // whole wave
     if (wid < nq_items) {
         const uint64_t row = wid / gq;
-        qk_item<T, HD, ITERQ, false, PAIRS>(q + row * (uint64_t)n_q * HD, n_q, (int)(wid % gq), qw, rope + row * (uint64_t)rot, eps, l, sub, rot);
+        qk_item<T, HD, ITERQ, false, PAIRS, BIAS>(q + row * (uint64_t)n_q * HD, n_q, (int)(wid % gq), qw, rope + row * (uint64_t)rot, eps, l, sub,
+                                                  rot, nullptr, nullptr, nullptr, qb);
     } else {
         const uint64_t w2 = wid - nq_items, row = w2 / gk;
         const uint64_t kv_dim = (uint64_t)n_kv * HD;
@@ -179,11 +227,12 @@ DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const fl
             const uint32_t pos = cache_pos[row];
             const bool ok = pos < capacity;
             if (!ok && lane == 0 && w2 % gk == 0) atomicOr(fault, APK_FAULT_CACHE_RANGE);
-            qk_item<T, HD, 1, true, PAIRS>(k + row * kv_dim, n_kv, (int)(w2 % gk), kw, rope + row * (uint64_t)rot, eps, l, sub, rot,
-                                           ok ? k_cache + pos * kv_dim : nullptr, v + row * kv_dim,
-                                           ok ? v_cache + pos * kv_dim : nullptr);
+            qk_item<T, HD, 1, true, PAIRS, BIAS>(k + row * kv_dim, n_kv, (int)(w2 % gk), kw, rope + row * (uint64_t)rot, eps, l, sub, rot,
+                                                 ok ? k_cache + pos * kv_dim : nullptr, v + row * kv_dim,
+                                                 ok ? v_cache + pos * kv_dim : nullptr, kb, vb, v + row * kv_dim);
         } else {
-            qk_item<T, HD, 1, false, PAIRS>(k + row * kv_dim, n_kv, (int)(w2 % gk), kw, rope + row * (uint64_t)rot, eps, l, sub, rot);
+            qk_item<T, HD, 1, false, PAIRS, BIAS>(k + row * kv_dim, n_kv, (int)(w2 % gk), kw, rope + row * (uint64_t)rot, eps, l, sub, rot,
+                                                  nullptr, nullptr, nullptr, kb);
         }
     }
 }
@@ -210,13 +259,13 @@ APK_QKROPE_ALL(f16_t, f16)
     extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void apk_qknorm_rope_kv_##TN##_hd##HD##_i##ITER(     \
         T* q, T* k, const T* v, const float* qw, const float* kw, const float* rope, const uint32_t* cache_pos,  \
         f16_t* k_cache, f16_t* v_cache, uint32_t capacity, int rows, int n_q, int n_kv, float eps, uint32_t* fault, int rot) { \
-        qknorm_rope_body<T, HD, ITER, true>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x, v, cache_pos,   \
+        qknorm_rope_body<T, HD, ITER, true>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x, (T*)v, cache_pos, \
                                             k_cache, v_cache, capacity, fault);                                   \
     }                                                                                                             \
     extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void apk_qknorm_rope_pairs_kv_##TN##_hd##HD##_i##ITER( \
         T* q, T* k, const T* v, const float* qw, const float* kw, const float* rope, const uint32_t* cache_pos,  \
         f16_t* k_cache, f16_t* v_cache, uint32_t capacity, int rows, int n_q, int n_kv, float eps, uint32_t* fault, int rot) { \
-        qknorm_rope_body<T, HD, ITER, true, true>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x, v, cache_pos, \
+        qknorm_rope_body<T, HD, ITER, true, true>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x, (T*)v, cache_pos, \
                                                   k_cache, v_cache, capacity, fault);                             \
     }
 #define APK_QKROPE_KV_ALL(T, TN)                                                                                       \
@@ -225,6 +274,29 @@ APK_QKROPE_ALL(f16_t, f16)
 APK_QKROPE_KV_ALL(float, f32)
 APK_QKROPE_KV_ALL(f16_t, f16)
 
+// With the projection biases (two passes per q wave in fp16 only, as without them).  Without the
+// cache store v is not touched here; with it, v + v_bias is written back to v and narrowed into the cache.
+#define APK_QKROPE_BIAS(T, TN, HD, ITER, PAIRS, PN)                                                               \
+    extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void apk_qknorm_rope_##PN##bias_##TN##_hd##HD##_i##ITER( \
+        T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv, float eps, int rot, \
+        const float* qb, const float* kb) {                                                                       \
+        qknorm_rope_body<T, HD, ITER, false, PAIRS, true>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x, nullptr, nullptr, \
+                                                          nullptr, nullptr, 0, nullptr, qb, kb, nullptr);         \
+    }                                                                                                             \
+    extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void apk_qknorm_rope_##PN##kv_bias_##TN##_hd##HD##_i##ITER( \
+        T* q, T* k, T* v, const float* qw, const float* kw, const float* rope, const uint32_t* cache_pos,         \
+        f16_t* k_cache, f16_t* v_cache, uint32_t capacity, int rows, int n_q, int n_kv, float eps, uint32_t* fault, int rot, \
+        const float* qb, const float* kb, const float* vb) {                                                      \
+        qknorm_rope_body<T, HD, ITER, true, PAIRS, true>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x, v, cache_pos, \
+                                                         k_cache, v_cache, capacity, fault, qb, kb, vb);          \
+    }
+#define APK_QKROPE_BIAS_ALL(T, TN, ITER)                                                                           \
+    APK_QKROPE_BIAS(T, TN, 64, ITER, false, ) APK_QKROPE_BIAS(T, TN, 128, ITER, false, ) APK_QKROPE_BIAS(T, TN, 256, ITER, false, ) \
+    APK_QKROPE_BIAS(T, TN, 64, ITER, true, pairs_) APK_QKROPE_BIAS(T, TN, 128, ITER, true, pairs_) APK_QKROPE_BIAS(T, TN, 256, ITER, true, pairs_)
+APK_QKROPE_BIAS_ALL(float, f32, 1)
+APK_QKROPE_BIAS_ALL(f16_t, f16, 1)
+APK_QKROPE_BIAS_ALL(f16_t, f16, 2)
+
 // Any other head geometry: head_dim not 64/128/256, a rotary table that covers only the
 // leading rot_half pairs of a head (partial rotary: channels >= 2*rot_half are normalised
 // and pass through, rope.rs:52-81), or the adjacent-pair style (RopeStyle::Norm, pairs
@@ -232,7 +304,7 @@ APK_QKROPE_KV_ALL(f16_t, f16)
 // element-wise; same arithmetic as the tiled kernels minus the coefficient folding.
 template <typename T>
 DEV void qknorm_rope_generic_body(T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q,
-                                  int n_kv, int hd, int rot_half, int norm_style, float eps) {
+                                  int n_kv, int hd, int rot_half, int norm_style, float eps, const float* qb, const float* kb) {
     typedef typename headstat<T>::acc_t acc_t;
     const int lane = threadIdx.x & 63;
     const uint64_t wid = ((uint64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
@@ -243,17 +315,20 @@ DEV void qknorm_rope_generic_body(T* q, T* k, const float* qw, const float* kw, 
     const bool isq = hh < n_q;
     T* x = isq ? q + (row * n_q + hh) * (uint64_t)hd : k + (row * n_kv + (hh - n_q)) * (uint64_t)hd;
     const float* w = isq ? qw : kw;
+    const float* bias = isq ? qb : kb;  // the projection bias of this head's channels, or none
+    if (bias) bias += (uint64_t)(isq ? hh : hh - n_q) * hd;
+    auto ld = [&](int i) { return bias ? (float)x[i] + bias[i] : (float)x[i]; };
     const float* t = rope + row * (uint64_t)rot_half * 2;
     typename headstat<T>::scale_t scale{};
     if (w) {
         acc_t ss = 0;
-        for (int i = lane; i < hd; i += 64) ss = headstat<T>::sq(ss, (float)x[i]);
+        for (int i = lane; i < hd; i += 64) ss = headstat<T>::sq(ss, ld(i));
         ss = group_sum<64>(ss);  // every lane's loads are consumed here, before any store below
         scale = headstat<T>::rscale(ss, hd, eps);
     }
     for (int i = lane; i < rot_half; i += 64) {
         const int ia = norm_style ? 2 * i : i, ib = norm_style ? 2 * i + 1 : i + rot_half;
-        float a = (float)x[ia], b = (float)x[ib];
+        float a = ld(ia), b = ld(ib);
         if (w) {
             a = headstat<T>::apply(a, scale, w[ia]);
             b = headstat<T>::apply(b, scale, w[ib]);
@@ -262,18 +337,21 @@ DEV void qknorm_rope_generic_body(T* q, T* k, const float* qw, const float* kw, 
         x[ia] = (T)(a * cs - b * sn);
         x[ib] = (T)(a * sn + b * cs);
     }
-    if (w)
-        for (int i = 2 * rot_half + lane; i < hd; i += 64) x[i] = (T)headstat<T>::apply((float)x[i], scale, w[i]);
+    if (w) {
+        for (int i = 2 * rot_half + lane; i < hd; i += 64) x[i] = (T)headstat<T>::apply(ld(i), scale, w[i]);
+    } else if (bias) {
+        for (int i = 2 * rot_half + lane; i < hd; i += 64) x[i] = (T)ld(i);
+    }
 }
 extern "C" __global__ __launch_bounds__(256) void apk_qknorm_rope_generic_f32(
     float* q, float* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv, int hd,
-    int rot_half, int norm_style, float eps) {
-    qknorm_rope_generic_body<float>(q, k, qw, kw, rope, rows, n_q, n_kv, hd, rot_half, norm_style, eps);
+    int rot_half, int norm_style, float eps, const float* qb, const float* kb) {
+    qknorm_rope_generic_body<float>(q, k, qw, kw, rope, rows, n_q, n_kv, hd, rot_half, norm_style, eps, qb, kb);
 }
 extern "C" __global__ __launch_bounds__(256) void apk_qknorm_rope_generic_f16(
     f16_t* q, f16_t* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv, int hd,
-    int rot_half, int norm_style, float eps) {
-    qknorm_rope_generic_body<f16_t>(q, k, qw, kw, rope, rows, n_q, n_kv, hd, rot_half, norm_style, eps);
+    int rot_half, int norm_style, float eps, const float* qb, const float* kb) {
+    qknorm_rope_generic_body<f16_t>(q, k, qw, kw, rope, rows, n_q, n_kv, hd, rot_half, norm_style, eps, qb, kb);
 }
 
 // Layer prologue for small decode batches: the residual add + RMSNorm of the hidden

@@ -20,6 +20,15 @@ class Plan(C.Structure):
                 ("slices_per_row", C.c_uint), ("items", C.c_uint)]
 
 
+class AttnPrologue(C.Structure):
+    """struct apk_attn_prologue: the arguments of apk_attn_prologue_rows."""
+    _fields_ = [("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("q_bias", C.c_void_p), ("k_bias", C.c_void_p),
+                ("v_bias", C.c_void_p), ("q_norm", C.c_void_p), ("k_norm", C.c_void_p), ("rope", C.c_void_p),
+                ("cache_pos", C.c_void_p), ("k_cache", C.c_void_p), ("v_cache", C.c_void_p), ("capacity", C.c_size_t),
+                ("rows", C.c_size_t), ("n_q", C.c_size_t), ("n_kv", C.c_size_t), ("head_dim", C.c_size_t), ("rot_dim", C.c_size_t),
+                ("eps", C.c_float), ("dtype", C.c_int), ("adjacent_pairs", C.c_int)]
+
+
 # every symbol include/apk_hip.h declares: (restype, argtypes)
 _vp, _sz, _i, _f, _u64p, _u32p = C.c_void_p, C.c_size_t, C.c_int, C.c_float, C.POINTER(C.c_uint64), C.POINTER(C.c_uint32)
 _plan = C.POINTER(Plan)
@@ -77,6 +86,9 @@ SYMBOLS = {
     "apk_postnorm_add_rmsnorm_rows": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _f, _i]),
     "apk_plan_qknorm_rope": (_i, [_sz, _sz, _sz, _sz, _sz, _i, _i, _i, _plan]),
     "apk_plan_scatter_rows": (_i, [_sz, _sz, _sz, _i, _plan]),
+    "apk_plan_attn_prologue_rows": (_i, [C.POINTER(AttnPrologue), _plan]),
+    "apk_add_bias_rows": (_i, [_vp, _vp, _vp, _sz, _sz, _i]),
+    "apk_attn_prologue_rows": (_i, [_vp, C.POINTER(AttnPrologue)]),
     "apk_plan_embed_rows": (_i, [_i, _sz, _sz, _i, _plan]),
     "apk_kernel_count": (_sz, []),
     "apk_kernel_name": (_i, [_sz, C.c_char_p, _sz]),

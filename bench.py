@@ -241,11 +241,30 @@ def main():
         us = timed(lambda i: apklib.check(L.apk_qknorm_rope_norm(h, p(qk[i % len(qk)]["q"]), p(qk[i % len(qk)]["k"]), None, None, p(rope),
                                                                  T, lq, lkv, HD, HD, EPS, F16)), reps)
         record("rope, adjacent pairs, no QK-norm", f"32 q + 8 k heads of 128, T={T} f16", us, 2 * T * (lq + lkv) * HD * b + T * HD * 4)
+        # projection biases, the rotation and the K/V cache store as one call (28 q + 4 k heads of 128, biases on q, k, v,
+        # no QK-norm: the geometry of the bias-carrying Qwen2.5-7B), on the leading heads of the same buffers
+        bq, bkv = 28, 4
+        qbias, kbias, vbias = randn((bq * HD,), torch.float32), randn((bkv * HD,), torch.float32), randn((bkv * HD,), torch.float32)
+        pro = []
+        for i in range(len(qk)):
+            a = apklib.AttnPrologue()
+            a.q, a.k, a.v = p(qk[i]["q"]), p(qk[i]["k"]), p(kvp[i]["v"])
+            a.q_bias, a.k_bias, a.v_bias, a.rope = p(qbias), p(kbias), p(vbias), p(rope)
+            a.cache_pos, a.k_cache, a.v_cache, a.capacity = p(pos), p(kvp[i]["kc"]), p(kvp[i]["vc"]), T
+            a.rows, a.n_q, a.n_kv, a.head_dim, a.rot_dim, a.eps, a.dtype = T, bq, bkv, HD, HD, EPS, F16
+            pro.append(a)
+        us = timed(lambda i: apklib.check(L.apk_attn_prologue_rows(h, C.byref(pro[i % len(pro)]))), reps)
+        record("attn_prologue: q/k/v biases + rope + K/V cache store (one launch)", f"28 q + 4 k heads of 128, T={T} f16", us,
+               2 * T * (bq + 2 * bkv) * HD * b + 2 * T * bkv * HD * 2 + T * HD * 4 + T * 4 + (bq + 2 * bkv) * HD * 4)
         # what fusing the residual add into the norm buys: the same result as two launches of this library's own ops
         us = timed(lambda i: (apklib.check(L.apk_add_assign(h, p(an[i % len(an)]["x"]), p(an[i % len(an)]["d"]), T * H, F16)),
                               apklib.check(L.apk_add_rmsnorm_rows(h, p(an[i % len(an)]["x"]), None, p(an[i % len(an)]["h"]), p(gamma1), H, T, EPS, F16))), reps)
         record("UNFUSED residual add, then RMSNorm (two launches)", tag, us, 3 * T * H * b + 2 * T * H * b + 4 * H, launches=2,
                note="for comparison with add_rmsnorm")
+        # the sandwich norm (x += rmsnorm(delta) * post_gamma) and the next norm as one launch: the bytes of add_rmsnorm
+        us = timed(lambda i: apklib.check(L.apk_postnorm_add_rmsnorm_rows(h, p(an[i % len(an)]["x"]), p(an[i % len(an)]["d"]), p(gamma2),
+                                                                          p(an[i % len(an)]["h"]), p(gamma1), H, T, EPS, F16)), reps)
+        record("postnorm_add_rmsnorm (sandwich norm + next norm, one launch)", tag, us, bytes_addnorm + 4 * H)
         del an, qk, sw, kvp
         # the same headline shape with f32 activations, the reference's own activation type (f64 statistics,
         # the reference's operation order): twice the bytes per launch

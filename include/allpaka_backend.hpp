@@ -177,6 +177,17 @@ inline void add_assign_slice(std::vector<float>& a, const std::vector<float>& b)
     da.read_back(a.data());
 }
 
+// add_bias_rows(rows, bias) (model/loader.rs:519-523): every whole row of bias.len() elements gets the bias; what is
+// left of a partial last row is untouched (chunks_exact_mut).
+inline void add_bias_rows(std::vector<float>& rows, const std::vector<float>& bias) {
+    if (bias.empty()) throw Panic("chunk size must be non-zero");
+    const size_t n = bias.size(), whole = rows.size() / n;
+    if (whole == 0) return;
+    Dev<float> dx(rows.data(), whole * n), db(bias.data(), n);
+    check(apk_add_bias_rows(Gpu::get().ctx(), dx.ptr(), db.ptr(), whole, n, APK_F32));
+    dx.read_back(rows.data());
+}
+
 // ops::softmax(x) in place (activation.rs:5).
 inline void softmax(std::vector<float>& x) {
     Dev<float> dx(x.data(), x.size());

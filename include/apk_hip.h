@@ -381,6 +381,42 @@ int apk_argmax_rows(apk_ctx* ctx, const float* logits, size_t rows, size_t n, ui
  * figures of the other kernels are calibrated against. */
 int apk_copy(apk_ctx* ctx, const void* src, void* dst, size_t bytes);
 
+/* x[r][i] += bias[i] over rows of length n (add_bias_rows, crates/allpaka-model/src/model/loader.rs:519-523:
+ * ops::add_assign_slice(row, bias) per row).  x: [rows][n] of dtype, in place; bias: f32[n]. */
+int apk_add_bias_rows(apk_ctx* ctx, void* x, const float* bias, size_t rows, size_t n, int dtype);
+
+/* Everything the reference does to a batch's projected q, k, v rows between the QKV projection and
+ * attention, as one call (model/attention.rs:125-165 and the cache store kv.rs:682-697):
+ *   add_bias_rows(q, q_bias); add_bias_rows(k, k_bias); add_bias_rows(v, v_bias)      (:125-129; each optional)
+ *   per head: ops::rmsnorm(head, q_norm | k_norm, eps) (optional), then the row's rotation  (:131-165)
+ *   KvCache::store_at: k and v narrowed to f16 at cache row cache_pos[row]             (optional)
+ * Fields as in apk_qknorm_rope_neox / _norm (adjacent_pairs != 0) / _kv_store; the biases are f32
+ * [n_q*head_dim] / [n_kv*head_dim], 16-byte aligned, NULL for none.  The cache store is asked for by a
+ * non-NULL k_cache (then v, cache_pos, v_cache and capacity are required).  One launch for heads of
+ * 64/128/256 with a rotary width of whole tiles; v_bias without the cache store is one more launch
+ * (v is not otherwise read), and other head geometries take the element-wise kernel (no cache store there).
+ * With biases, fp16 rows are widened, biased, normalised and rotated in f32 and rounded once. */
+typedef struct apk_attn_prologue {
+    void* q;                 /* [rows][n_q*head_dim] of dtype, in place */
+    void* k;                 /* [rows][n_kv*head_dim] of dtype, in place */
+    void* v;                 /* [rows][n_kv*head_dim] of dtype: read for the cache store, written only with v_bias; else NULL */
+    const float* q_bias;
+    const float* k_bias;
+    const float* v_bias;
+    const float* q_norm;     /* f32[head_dim] or NULL */
+    const float* k_norm;
+    const float* rope;       /* f32 [rows][rot_dim/2][2] = [sin, cos] */
+    const uint32_t* cache_pos; /* [rows] cache row per batch row, or NULL */
+    void* k_cache;           /* f16 [capacity][n_kv*head_dim], or NULL: no store */
+    void* v_cache;
+    size_t capacity;
+    size_t rows, n_q, n_kv, head_dim, rot_dim;
+    float eps;
+    int dtype;
+    int adjacent_pairs;      /* 0: NeoX pairs (i, i + rot_dim/2); else pairs (2i, 2i+1) */
+} apk_attn_prologue;
+int apk_attn_prologue_rows(apk_ctx* ctx, const apk_attn_prologue* args);
+
 /* Launch plans (no context, no GPU; see apk_plan): what apk_add_rmsnorm_rows, apk_postnorm_add_rmsnorm_rows, apk_qknorm_rope_neox /
  * _norm (adjacent_pairs != 0) / _kv_store (with_kv_store != 0), apk_scatter_rows and apk_embed_rows /
  * apk_dequant_rows launch for these sizes.  Return APK_OK with plan filled (kernel "" and grid 0 when
@@ -390,6 +426,7 @@ int apk_plan_add_rmsnorm_rows(size_t n, size_t rows, int dtype, apk_plan* plan);
 int apk_plan_postnorm_add_rmsnorm_rows(size_t n, size_t rows, int dtype, apk_plan* plan);
 int apk_plan_qknorm_rope(size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim, int adjacent_pairs, int dtype,
                          int with_kv_store, apk_plan* plan);
+int apk_plan_attn_prologue_rows(const apk_attn_prologue* args, apk_plan* plan);
 int apk_plan_scatter_rows(size_t rows, size_t k, size_t cols, int dtype, apk_plan* plan);
 int apk_plan_embed_rows(int fmt, size_t n_in, size_t t, int out_dtype, apk_plan* plan);
 /* The kernels apk_init resolves from the embedded code object: their number, and the i-th name copied into

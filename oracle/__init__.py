@@ -56,6 +56,8 @@ def lib():
         L.ora_rmsnorm_into.argtypes = [vp, vp, vp, sz, f32]
         L.ora_rmsnorm_rows_into.argtypes = [vp, sz, vp, sz, vp, sz, f32, sz]
         L.ora_add_assign_slice.argtypes = [vp, sz, vp, sz]
+        L.ora_add_bias_rows.argtypes = [vp, sz, vp, sz]
+        L.ora_add_bias_rows.restype = None
         L.ora_add_assign_par.argtypes = [vp, sz, vp, sz, sz]
         L.ora_add_scaled_slice.argtypes = [vp, sz, vp, sz, f32]
         L.ora_rope_inv_freq.argtypes = [sz, f32, vp]
@@ -288,12 +290,33 @@ def rope_norm(x, pos, base):
     lib().ora_rope_norm(_p(x), x.size, int(pos), base)
 
 
-def qknorm_rope_rows(q, k, n_q, n_kv, head_dim, qw, kw, rope_flat, eps, style=0):
+def add_bias_rows(rows, bias):
+    """add_bias_rows (model/loader.rs:519-523), f32 in place."""
+    _chk(rows, np.float32)
+    _chk(bias, np.float32)
+    lib().ora_add_bias_rows(_p(rows), rows.size, _p(bias), bias.size)
+
+
+def qknorm_rope_rows(q, k, n_q, n_kv, head_dim, qw, kw, rope_flat, eps, style=0, q_bias=None, k_bias=None):
     """OP-C: q [rows, n_q*hd], k [rows, n_kv*hd] in place; rope_flat [rows, half, 2];
-    style 0 = NeoX pairs, 1 = adjacent (NORM) pairs."""
+    style 0 = NeoX pairs, 1 = adjacent (NORM) pairs.  q_bias / k_bias: add_bias_rows first (attention.rs:125-129);
+    fp16 rows are then widened, biased and run through the f32 op, and rounded once."""
     rows = q.shape[0]
     half = rope_flat.shape[1]
     _chk(rope_flat, np.float32)
+    if q_bias is not None or k_bias is not None:
+        f16 = q.dtype != np.float32
+        qf = f16_bits_to_f32(q) if f16 else q
+        kf = f16_bits_to_f32(k) if f16 else k
+        if q_bias is not None and qf.size:
+            add_bias_rows(qf, q_bias)
+        if k_bias is not None and kf.size:
+            add_bias_rows(kf, k_bias)
+        lib().ora_qknorm_rope_rows_style(_p(qf), _p(kf), rows, n_q, n_kv, head_dim, _p(qw), _p(kw), _p(rope_flat), half, eps, style)
+        if f16:
+            q[...] = f32_to_f16_bits(qf)
+            k[...] = f32_to_f16_bits(kf)
+        return
     if q.dtype == np.float32:
         lib().ora_qknorm_rope_rows_style(_p(q), _p(k), rows, n_q, n_kv, head_dim, _p(qw), _p(kw), _p(rope_flat), half, eps, style)
     else:

@@ -555,6 +555,13 @@ ORA_API void ora_qknorm_rope_rows(float *q, float *k, size_t rows, size_t n_q, s
     ora_qknorm_rope_rows_style(q, k, rows, n_q, n_kv, head_dim, qw, kw, rope_flat, half, eps, 0);
 }
 
+/* add_bias_rows, crates/allpaka-model/src/model/loader.rs:519-523: every row of bias_len elements gets
+ * ops::add_assign_slice(row, bias); a trailing partial row is left alone (chunks_exact_mut). */
+ORA_API void ora_add_bias_rows(float *rows, size_t len, const float *bias, size_t bias_len) {
+    for (size_t r = 0; r + bias_len <= len && bias_len; r += bias_len)
+        for (size_t i = 0; i < bias_len; i++) rows[r + i] += bias[i];
+}
+
 /* ------------------------------------------------------------- activation */
 
 /* crates/allpaka-backend/src/ops/activation.rs:19-22 */

@@ -79,6 +79,20 @@ static void sandwich_norm_matches_the_three_ops() {  // decode.rs:581-584, :771-
     for (size_t i = 0; i < h.size(); i++) CHECK(h[i] == want[i]);
     CHECK(throws<Panic>([] { std::vector<float> a(64), d(64), pw(32), h(64), w(64); ops::postnorm_add_assign_then_rmsnorm_into(a, d, pw, h, w, 0.0f); }));
 }
+static void add_bias_rows_biases_every_whole_row() {  // loader.rs:519-523
+    std::vector<float> x = {1, 2, 3, 4, 5, 6, 7, 8}, b = {10, 20, 30};
+    ops::add_bias_rows(x, b);
+    const std::vector<float> want = {11, 22, 33, 14, 25, 36, 7, 8};
+    CHECK(x == want);
+    std::vector<float> big(300 * 1024), bias(1024);
+    for (size_t i = 0; i < big.size(); i++) big[i] = std::sin(0.01f * i);
+    for (size_t i = 0; i < bias.size(); i++) bias[i] = 0.001f * i - 0.5f;
+    std::vector<float> sum(big);
+    for (size_t i = 0; i < big.size(); i++) sum[i] = big[i] + bias[i % 1024];
+    ops::add_bias_rows(big, bias);
+    CHECK(big == sum);
+    CHECK(throws<Panic>([] { std::vector<float> x(4), b; ops::add_bias_rows(x, b); }));
+}
 static void swiglu_is_silu_of_gate_times_up() {  // :172-185, silu fixed points :163-170
     std::vector<float> gate, up;
     for (int i = -25; i < 26; i++) gate.push_back(i * 0.7f);
@@ -367,6 +381,7 @@ int main() {
         {"rmsnorm_rows_into_rejects_a_short_destination", rmsnorm_rows_into_rejects_a_short_destination},
         {"add_assign_then_norm_matches_the_two_ops", add_assign_then_norm_matches_the_two_ops},
         {"sandwich_norm_matches_the_three_ops", sandwich_norm_matches_the_three_ops},
+        {"add_bias_rows_biases_every_whole_row", add_bias_rows_biases_every_whole_row},
         {"swiglu_is_silu_of_gate_times_up", swiglu_is_silu_of_gate_times_up},
         {"geglu_tanh_is_the_tanh_gelu_of_gate_times_up", geglu_tanh_is_the_tanh_gelu_of_gate_times_up},
         {"softmax_sums_to_one_and_survives_huge_logits", softmax_sums_to_one_and_survives_huge_logits},

@@ -637,6 +637,108 @@ def test_kv_store_position_past_capacity_is_flagged_not_faulted(be, ora):
     assert host(kc)[1].any() and host(kc)[3].any() and not host(kc)[[0, 2]].any()
 
 
+# ------------------------------------- projection biases, and the whole q/k/v step as one call
+@pytest.mark.parametrize("rows,n", [(1, 1024), (6, 5120), (300, 4096), (5, 1001), (64, 24), (3, 7)])
+@pytest.mark.parametrize("f16", [False, True])
+def test_add_bias_rows(be, ora, rows, n, f16):
+    """add_bias_rows (loader.rs:519-523): f32 bit-exact; fp16 rows widened, biased in f32 and rounded once."""
+    s = synth()
+    g = s.rng(3, rows * 31 + n)
+    x, b = s.normal_f32(g, (rows, n)), s.normal_f32(g, n, 0.0, 0.5)
+    want = x.copy()
+    if f16:
+        xb = s.to_f16_bits(x)
+        want = ora.f16_bits_to_f32(xb)
+        ora.add_bias_rows(want, b)
+        want = ora.f32_to_f16_bits(want)
+        x = xb
+    else:
+        ora.add_bias_rows(want, b)
+    t = dev(x)
+    be.add_bias_rows(t, dev(b))
+    assert np.array_equal(host(t), want)
+
+
+@pytest.mark.parametrize("rows,n_q,n_kv,hd,rot,style", [
+    (1, 28, 4, 128, 128, 0),    # Qwen2.5-7B decode: biases, no QK-norm, NeoX
+    (6, 28, 4, 128, 128, 0), (300, 40, 8, 128, 128, 0), (2048, 12, 2, 128, 128, 0),
+    (33, 32, 2, 128, 64, 0),    # GLM style: biases and partial rotary
+    (40, 32, 2, 128, 64, 1), (9, 8, 2, 256, 256, 1), (65, 12, 2, 64, 64, 0), (5, 3, 0, 128, 128, 0), (5, 0, 3, 64, 64, 1),
+    (7, 5, 1, 80, 32, 0), (4, 3, 3, 96, 96, 1), (3, 2, 1, 128, 0, 0),   # the element-wise kernel
+])
+@pytest.mark.parametrize("f16", [False, True])
+@pytest.mark.parametrize("normed", [False, True])
+@pytest.mark.parametrize("store", [False, True])
+def test_attn_prologue_rows(be, ora, rows, n_q, n_kv, hd, rot, style, f16, normed, store):
+    """attention.rs:125-165 + kv.rs:682-697 as one call: add_bias_rows on q, k, v; per-head norm (optional) and the
+    row's rotation; k and v narrowed into the cache rows -- against the oracle's ops in the reference's order."""
+    import allpaka_amd as apk
+
+    s = synth()
+    g = s.rng(3, rows * 577 + n_q * 5 + hd + rot + style)
+    q, k, v = s.normal_f32(g, (rows, n_q * hd)), s.normal_f32(g, (rows, n_kv * hd)), s.normal_f32(g, (rows, n_kv * hd))
+    qb, kb, vb = s.normal_f32(g, n_q * hd, 0.0, 0.5), s.normal_f32(g, n_kv * hd, 0.0, 0.5), s.normal_f32(g, n_kv * hd, 0.0, 0.5)
+    qw, kw = (s.normal_f32(g, hd, 1.0, 0.05), s.normal_f32(g, hd, 1.0, 0.05)) if normed else (None, None)
+    if f16:
+        q, k, v = s.to_f16_bits(q), s.to_f16_bits(k), s.to_f16_bits(v)
+    cap = max(rows + 9, 40)
+    positions = g.permutation(cap)[:rows].astype(np.uint32)
+    ropes = ora.rope_table([int(p) for p in positions], ora.rope_inv_freq(rot, 1e6)) if rot else np.zeros((rows, 0, 2), np.float32)
+    # the oracle, in the reference's order
+    wq, wk = q.copy(), k.copy()
+    ora.qknorm_rope_rows(wq, wk, n_q, n_kv, hd, qw, kw, ropes, 1e-6, style=style, q_bias=qb if n_q else None, k_bias=kb if n_kv else None)
+    wv = ora.f16_bits_to_f32(v) if f16 else v.copy()
+    if n_kv:
+        ora.add_bias_rows(wv, vb)
+    if f16:
+        wv = ora.f32_to_f16_bits(wv)
+    wkc, wvc = np.zeros((cap, n_kv * hd), np.uint16), np.zeros((cap, n_kv * hd), np.uint16)
+    ora.kv_store_rows(wk, wv, positions, wkc, wvc)
+    tq, tk, tv = dev(q), dev(k), dev(v)
+    kc = torch.zeros((cap, n_kv * hd), dtype=torch.float16, device="cuda")
+    vc = torch.zeros_like(kc)
+    rt = dev(ropes) if rot else torch.zeros((rows, 0, 2), device="cuda")
+    kw_args = dict(q_bias=dev(qb) if n_q else None, k_bias=dev(kb) if n_kv else None, v_bias=dev(vb) if n_kv else None,
+                   q_norm=None if qw is None else dev(qw), k_norm=None if kw is None else dev(kw), adjacent_pairs=bool(style), rot_dim=rot)
+    if store:
+        kw_args.update(cache_pos=dev(positions), k_cache=kc, v_cache=vc)
+    es = 2 if f16 else 4
+    tiled = hd in (64, 128, 256) and rot > 0 and (rot % (16 // es) == 0 if style else (rot // 2) % (16 // es) == 0)
+    if store and (not tiled or n_kv == 0):  # the cache store rides on the tiled kernels' k items only
+        with pytest.raises(apk.Declined):
+            be.attn_prologue_rows(tq, tk, tv, n_q, n_kv, hd, 1e-6, rt, **kw_args)
+        assert np.array_equal(host(tv), v) and np.array_equal(host(tq), q)  # declined before anything ran
+        return
+    be.attn_prologue_rows(tq, tk, tv, n_q, n_kv, hd, 1e-6, rt, **kw_args)
+    gk = host(tk)
+    for got, want in ((host(tq), wq), (gk, wk)):
+        if f16:
+            assert f16_ulp_diff(got, want) <= TOL_F16_ULP
+            assert got.size == 0 or np.mean(got == want) > 0.99  # one rounding of the same f32 chain: equal nearly everywhere
+        elif not normed:
+            assert np.array_equal(got, want)  # bias and rotation only: the same f32 operations
+        else:
+            assert rel_err_f32(got, want) <= TOL_F32 and close_idiom(got, want)
+    assert np.array_equal(host(tv), wv)  # v + v_bias: one f32 add, rounded once
+    if store:
+        assert np.array_equal(host(vc), wvc)
+        mine_k, mine_v = np.zeros_like(wkc), np.zeros_like(wvc)
+        ora.kv_store_rows(gk, wv, positions, mine_k, mine_v)
+        assert np.array_equal(host(kc), mine_k)
+        assert f16_ulp_diff(host(kc), wkc) <= (TOL_F16_ULP if f16 else 1)
+
+
+def test_attn_prologue_rows_without_biases_is_the_plain_op(be, ora):
+    """No biases: the same kernels as apk_qknorm_rope_kv_store / _neox (two passes per q wave in fp16 included)."""
+    rows, n_q, n_kv, hd = 600, 64, 8, 128
+    positions = [int(p) for p in np.arange(rows)]
+    q, k, qw, kw, inv, ropes = _qk_case(ora, 3, rows, n_q, n_kv, hd, True, positions)
+    t1q, t1k, t2q, t2k = dev(q), dev(k), dev(q), dev(k)
+    be.qknorm_rope_neox(t1q, t1k, dev(qw), dev(kw), dev(ropes), n_q, n_kv, hd, 1e-6)
+    be.attn_prologue_rows(t2q, t2k, None, n_q, n_kv, hd, 1e-6, dev(ropes), q_norm=dev(qw), k_norm=dev(kw))
+    assert np.array_equal(host(t1q), host(t2q)) and np.array_equal(host(t1k), host(t2k))
+
+
 # ------------------------------------------- single-launch layer prologue
 @pytest.mark.parametrize("rows,n,n_q,n_kv,hd,f16", [
     (64, 5120, 64, 8, 128, True), (1, 5120, 64, 8, 128, True), (6, 5120, 64, 8, 128, True),

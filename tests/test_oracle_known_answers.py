@@ -761,3 +761,21 @@ def test_moe_combine_is_fma_in_hit_order_then_residual_then_norm(ora):
     x3 = x.copy()
     ora.moe_combine_add_rmsnorm(x3, flat, tok_off, hit_row, hit_w, None, None, 1e-6)
     assert np.array_equal(x3, x2)
+
+
+def test_add_bias_rows_known_answer(ora):
+    """add_bias_rows (loader.rs:519-523): bias[i] goes to column i of every whole row; what is left of a partial last
+    row (chunks_exact_mut) is untouched.  Values chosen so a row/column mix-up or a shifted index shows."""
+    x = np.array([1, 2, 3, 4, 5, 6, 7, 8], np.float32)  # two rows of 3, then 2 stray elements
+    ora.add_bias_rows(x, np.array([10, 20, 30], np.float32))
+    assert x.tolist() == [11, 22, 33, 14, 25, 36, 7, 8]
+    y = np.array([[0.5, -0.5]], np.float32)
+    ora.add_bias_rows(y, np.array([2.0 ** -25, 1.0], np.float32))  # one rounded f32 add per element
+    assert y.tolist() == [[0.5, 0.5]]
+    # in front of the per-head norm + rotation: q_bias / k_bias shift the rows the op then sees
+    q = np.array([[3.0, -1.0, 0.0, 2.0]], np.float32)
+    k = np.zeros((1, 0), np.float32)
+    rope = np.array([[[0.0, 1.0], [1.0, 0.0]]], np.float32)  # pair 0: identity; pair 1: quarter turn
+    ora.qknorm_rope_rows(q, k, 1, 0, 4, None, None, rope, 0.0, q_bias=np.array([1.0, 1.0, 1.0, 1.0], np.float32))
+    # biased row (4, 0, 1, 3): NeoX pairs (0, 2) and (1, 3); (a, b) -> (a cos - b sin, a sin + b cos)
+    assert q.tolist() == [[4.0, -3.0, 1.0, 0.0]]
