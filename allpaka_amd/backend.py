@@ -384,6 +384,20 @@ class Backend:
             return table, tok, tok_off, hit_row, hit_w
         return table[: int(n_used.item())], tok, tok_off, hit_row, hit_w
 
+    def moe_shared_hits(self, tok_off, hit_row, hit_w, total_rows):
+        """The shared expert's hit per token (prefill.rs:621-635): (total_rows + token, 1.0) after the routed hits.
+        Returns the lengthened (tok_off, hit_row, hit_w)."""
+        rows = tok_off.numel() - 1
+        n = hit_row.numel() + rows
+        dev = self.device
+        to = torch.empty(rows + 1, dtype=torch.int32, device=dev)
+        hr = torch.empty(n, dtype=torch.int32, device=dev)
+        hw = torch.empty(n, dtype=torch.float32, device=dev)
+        self._enter()
+        check(self.L.apk_moe_shared_hits(self.h, _ptr(tok_off), _ptr(hit_row), _ptr(hit_w), rows, total_rows, _ptr(to), _ptr(hr), _ptr(hw)))
+        self._leave()
+        return to, hr, hw
+
     def route_group(self, logits, k, n_expert=None, gating=Gating.Softmax, norm=True, scale=1.0, bias=None):
         """route_rows then moe_permute with the same results; one launch for a decode-sized batch
         (the router and the grouping of Ffn::moe_batch, moe.rs:204-271, :298-309).

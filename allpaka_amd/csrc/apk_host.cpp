@@ -68,7 +68,7 @@ std::vector<std::string> all_kernel_names() {
                                   "apk_moe_permute", "apk_gather_rows", "apk_scatter_rows_t1", "apk_scatter_rows_t2", "apk_argmax_rows", "apk_add_rmsnorm_ragged_f32", "apk_add_rmsnorm_ragged_f16", "apk_copy",
                                   "apk_qknorm_rope_generic_f32", "apk_qknorm_rope_generic_f16", "apk_route_topk_wide", "apk_route_topk_e64", "apk_route_topk_e128", "apk_route_group_small_e64", "apk_route_group_small_e128",
                                   "apk_route_group_small_e256", "apk_route_group_small_e1024", "apk_add_assign_f32", "apk_add_assign_f16", "apk_softmax_rows", "apk_moe_count", "apk_moe_rank",
-                                  "apk_add_bias_rows_f32", "apk_add_bias_rows_f16"};
+                                  "apk_add_bias_rows_f32", "apk_add_bias_rows_f16", "apk_moe_shared_hits"};
     for (const char* t : {"f32", "f16"}) {
         for (const char* f : {"q5k", "q6k", "q2k", "q3k", "q5_0", "f16", "f32", "bf16"}) v.push_back(std::string("apk_embed_") + f + "_" + t);
         for (int c : kAddnormTiles) v.push_back(std::string("apk_add_rmsnorm_") + t + "_c" + std::to_string(c));
@@ -1290,6 +1290,21 @@ int apk_scatter_rows(apk_ctx* c, const void* src, const uint32_t* hit_row, size_
     uint32_t k32 = (uint32_t)k, total32 = (uint32_t)total_rows;
     void* args[] = {&src, &hit_row, &k32, &total32, &row_vecs, &dst, &c->fault_dev, &p.items, &p.slices_per_row};
     return launch(c, p.kernel, p.grid, p.block, 0, args);
+}
+
+int apk_moe_shared_hits(apk_ctx* c, const uint32_t* tok_off, const uint32_t* hit_row, const float* hit_w, size_t rows,
+                        size_t total_rows, uint32_t* tok_off_out, uint32_t* hit_row_out, float* hit_w_out) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_moe_shared_hits: ctx is NULL");
+    CallScope s(c);
+    if (!tok_off || !tok_off_out || (rows && (!hit_row_out || !hit_w_out)) || (total_rows && (!hit_row || !hit_w)))
+        return fail(APK_DECLINE_NULL, "apk_moe_shared_hits: NULL tensor");
+    if (rows >= 0x7fffffffu || total_rows + rows > 0xffffffffu) return fail(APK_DECLINE_SHAPE, "apk_moe_shared_hits: too large");
+    if (tok_off_out == tok_off || hit_row_out == hit_row || hit_w_out == hit_w)
+        return fail(APK_DECLINE_SHAPE, "apk_moe_shared_hits: the lengthened lists need arrays of their own");
+    if (int rc = set_device(c)) return rc;
+    uint32_t rows32 = (uint32_t)rows, total32 = (uint32_t)total_rows;
+    void* args[] = {&tok_off, &hit_row, &hit_w, &rows32, &total32, &tok_off_out, &hit_row_out, &hit_w_out};
+    return launch(c, "apk_moe_shared_hits", (unsigned)((rows + 1 + 255) / 256), 256, 0, args);
 }
 
 int apk_moe_combine_add_rmsnorm(apk_ctx* c, void* x, const void* flat, const uint32_t* tok_off, const uint32_t* hit_row,

@@ -447,3 +447,24 @@ extern "C" __global__ __launch_bounds__(256) void apk_copy(const u32x4* src, u32
     const uint64_t c = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (c < nvec) __builtin_nontemporal_store(__builtin_nontemporal_load(src + c), dst + c);
 }
+
+// The shared expert of GLM-style MoE layers in the per-token hit lists (model/prefill.rs:621-635, flattened :658-675):
+// every token gets one more hit, after its routed ones, of weight 1 at flat row total_rows + token -- the shared FFN's
+// rows sit right after the experts' rows.  Any CSR in, the lengthened CSR out (tok_off_out[t] = tok_off[t] + t).
+extern "C" __global__ __launch_bounds__(256) void apk_moe_shared_hits(const uint32_t* tok_off, const uint32_t* hit_row,
+                                                                     const float* hit_w, uint32_t rows, uint32_t total_rows,
+                                                                     uint32_t* tok_off_out, uint32_t* hit_row_out,
+                                                                     float* hit_w_out) {
+    const uint32_t t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t > rows) return;
+    const uint32_t h0 = tok_off[t];
+    tok_off_out[t] = h0 + t;
+    if (t == rows) return;
+    const uint32_t h1 = tok_off[t + 1];
+    for (uint32_t i = h0; i < h1; i++) {
+        hit_row_out[i + t] = hit_row[i];
+        hit_w_out[i + t] = hit_w[i];
+    }
+    hit_row_out[h1 + t] = total_rows + t;
+    hit_w_out[h1 + t] = 1.0f;
+}

@@ -340,6 +340,16 @@ int apk_route_group(apk_ctx* ctx, const float* logits, const float* bias, size_t
                     int norm, float scale, int sigmoid, uint32_t* ids, float* w, uint32_t* table, uint32_t* n_used,
                     uint32_t* tok, uint32_t* tok_off, uint32_t* hit_row, float* hit_w);
 
+/* The shared expert of GLM-style MoE layers in the per-token hit lists: every token gets one more hit, after
+ * its routed ones, of weight 1.0 at flat row total_rows + token (the shared FFN's rows sit right after the
+ * experts' rows).  Replaces model/prefill.rs:621-635 (h.push((total_rows + i, 1.0))) and the flattening
+ * :658-675.  tok_off: u32[rows+1], hit_row / hit_w: [tok_off[rows]] as apk_moe_permute writes them (any CSR
+ * will do); the outputs hold tok_off[rows] + rows hits and must be arrays of their own.  apk_moe_combine_add_rmsnorm
+ * then takes the lengthened lists with total_rows + rows flat rows; apk_gather_rows / apk_scatter_rows keep
+ * the routed lists. */
+int apk_moe_shared_hits(apk_ctx* ctx, const uint32_t* tok_off, const uint32_t* hit_row, const float* hit_w, size_t rows,
+                        size_t total_rows, uint32_t* tok_off_out, uint32_t* hit_row_out, float* hit_w_out);
+
 /* dst[r,:] = src[tok[r],:] -- the gathered expert activations (model/moe.rs:348-352).
  * src: [src_rows][cols], dst: [total_rows][cols] of dtype; cols*sizeof(dtype) must
  * be a multiple of 16. */

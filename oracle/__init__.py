@@ -58,6 +58,8 @@ def lib():
         L.ora_add_assign_slice.argtypes = [vp, sz, vp, sz]
         L.ora_add_bias_rows.argtypes = [vp, sz, vp, sz]
         L.ora_add_bias_rows.restype = None
+        L.ora_moe_shared_hits.argtypes = [vp, vp, vp, sz, sz, vp, vp, vp]
+        L.ora_moe_shared_hits.restype = None
         L.ora_add_assign_par.argtypes = [vp, sz, vp, sz, sz]
         L.ora_add_scaled_slice.argtypes = [vp, sz, vp, sz, f32]
         L.ora_rope_inv_freq.argtypes = [sz, f32, vp]
@@ -417,6 +419,15 @@ def moe_group(ids, w, n_expert):
     hit_w = np.zeros(rows * k, np.float32)
     n_used = lib().ora_moe_group(_p(ids), _p(w), rows, k, n_expert, _p(table), _p(tok), _p(tok_off), _p(hit_row), _p(hit_w))
     return table[:n_used].copy(), tok, tok_off, hit_row, hit_w
+
+
+def moe_shared_hits(tok_off, hit_row, hit_w, total_rows):
+    """prefill.rs:621-635, :658-675: one more hit per token, (total_rows + token, 1.0), after its routed ones."""
+    rows = tok_off.size - 1
+    n = int(tok_off[-1]) + rows
+    to, hr, hw = np.zeros(rows + 1, np.uint32), np.zeros(n, np.uint32), np.zeros(n, np.float32)
+    lib().ora_moe_shared_hits(_p(tok_off), _p(hit_row), _p(hit_w), rows, total_rows, _p(to), _p(hr), _p(hw))
+    return to, hr, hw
 
 
 def gather_rows(src, tok):

@@ -757,6 +757,25 @@ ORA_API size_t ora_moe_group(const uint32_t *ids, const float *w, size_t rows, s
     return n_used;
 }
 
+/* The shared expert's hit, crates/allpaka-model/src/model/prefill.rs:621-635: after the routed hits of token i,
+ * h.push((total_rows + i, 1.0)); then the flattening of :658-675 (hits in list order, tok_off = running length). */
+ORA_API void ora_moe_shared_hits(const uint32_t *tok_off, const uint32_t *hit_row, const float *hit_w, size_t rows,
+                                 size_t total_rows, uint32_t *tok_off_out, uint32_t *hit_row_out, float *hit_w_out) {
+    size_t n = 0;
+    tok_off_out[0] = 0;
+    for (size_t i = 0; i < rows; i++) {
+        for (uint32_t h = tok_off[i]; h < tok_off[i + 1]; h++) {
+            hit_row_out[n] = hit_row[h];
+            hit_w_out[n] = hit_w[h];
+            n++;
+        }
+        hit_row_out[n] = (uint32_t)(total_rows + i);
+        hit_w_out[n] = 1.0f;
+        n++;
+        tok_off_out[i + 1] = (uint32_t)n;
+    }
+}
+
 /* Gathered activations in tok order, moe.rs:348-352: dst[r,:] = src[tok[r],:]. */
 ORA_API void ora_gather_rows(const float *src, const uint32_t *tok, size_t total_rows, size_t cols, float *dst) {
     for (size_t r = 0; r < total_rows; r++) memcpy(dst + r * cols, src + (size_t)tok[r] * cols, cols * sizeof(float));

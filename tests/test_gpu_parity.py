@@ -1133,6 +1133,42 @@ def test_moe_combine_add_rmsnorm(be, ora, rows, k, n_expert, n, f16):
     assert torch.equal(tx2, tx)
 
 
+@pytest.mark.parametrize("rows,k,n_expert,n,f16", [(1024, 8, 128, 2048, False), (1, 8, 128, 2048, True), (33, 4, 16, 512, True),
+                                                    (300, 6, 64, 1024, False), (7, 1, 4, 256, False)])
+def test_moe_shared_expert_hits(be, ora, rows, k, n_expert, n, f16):
+    """GLM-style layers: the shared expert's rows follow the routed experts' rows and every token takes one more hit of
+    weight 1 there (prefill.rs:621-635).  Device grouping -> lengthened lists -> combine, against the oracle's."""
+    s = synth()
+    g = s.rng(4, rows * 11 + n + k)
+    logits = s.normal_f32(g, (rows, n_expert))
+    ids, w = ora.route_rows(logits, k, threads=4)
+    table, tok, tok_off, hit_row, hit_w = ora.moe_group(ids, w, n_expert)
+    wto, whr, whw = ora.moe_shared_hits(tok_off, hit_row, hit_w, rows * k)
+    got = be.moe_permute(dev(ids), dev(w), n_expert)
+    gto, ghr, ghw = be.moe_shared_hits(got[2], got[3], got[4], rows * k)
+    assert np.array_equal(host(gto), wto) and np.array_equal(host(ghr), whr) and np.array_equal(host(ghw), whw)
+    assert whr.reshape(rows, k + 1)[:, k].tolist() == list(range(rows * k, rows * k + rows)) and (whw.reshape(rows, k + 1)[:, k] == 1).all()
+    flat = s.normal_f32(g, (rows * k + rows, n))  # the routed experts' down rows, then the shared expert's
+    x = s.normal_f32(g, (rows, n))
+    gamma = s.normal_f32(g, n, 1.0, 0.05)
+    if f16:
+        flat, x = s.to_f16_bits(flat), s.to_f16_bits(x)
+    wx, wh = x.copy(), np.zeros_like(x)
+    ora.moe_combine_add_rmsnorm(wx, flat, wto, whr, whw, wh, gamma, 1e-6)
+    tx, th = dev(x), torch.zeros_like(dev(x))
+    be.moe_combine_add_rmsnorm(tx, dev(flat), gto, ghr, ghw, th, dev(gamma), 1e-6)
+    assert np.array_equal(host(tx), wx)
+    if f16:
+        assert f16_ulp_diff(host(th), wh) <= TOL_F16_ULP
+    else:
+        assert rel_err_f32(host(th), wh) <= TOL_F32 and close_idiom(host(th), wh)
+    import allpaka_amd as apk
+
+    with pytest.raises(apk.Declined):  # the lengthened lists need arrays of their own
+        apk.lib.check(be.L.apk_moe_shared_hits(be.h, got[2].data_ptr(), got[3].data_ptr(), got[4].data_ptr(), rows, rows * k,
+                                               got[2].data_ptr(), ghr.data_ptr(), ghw.data_ptr()))
+
+
 @pytest.mark.parametrize("rows,n", [(1, 151936), (64, 151936), (3, 1000), (5, 7), (2, 16384), (300, 4096)])
 def test_argmax_rows(be, ora, rows, n):
     g = synth().rng(5, rows + n)

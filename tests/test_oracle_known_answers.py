@@ -779,3 +779,18 @@ def test_add_bias_rows_known_answer(ora):
     ora.qknorm_rope_rows(q, k, 1, 0, 4, None, None, rope, 0.0, q_bias=np.array([1.0, 1.0, 1.0, 1.0], np.float32))
     # biased row (4, 0, 1, 3): NeoX pairs (0, 2) and (1, 3); (a, b) -> (a cos - b sin, a sin + b cos)
     assert q.tolist() == [[4.0, -3.0, 1.0, 0.0]]
+
+
+def test_moe_shared_hits_known_answer(ora):
+    """prefill.rs:621-635: after its routed hits every token gets (total_rows + token, 1.0); :658-675: lists flattened
+    in order, tok_off the running length.  Two tokens, two picks each, by hand."""
+    tok_off = np.array([0, 2, 4], np.uint32)
+    hit_row = np.array([0, 2, 1, 3], np.uint32)
+    hit_w = np.array([0.75, 0.25, 0.5, 0.5], np.float32)
+    to, hr, hw = ora.moe_shared_hits(tok_off, hit_row, hit_w, 4)
+    assert to.tolist() == [0, 3, 6]
+    assert hr.tolist() == [0, 2, 4, 1, 3, 5]
+    assert hw.tolist() == [0.75, 0.25, 1.0, 0.5, 0.5, 1.0]
+    # uneven lists (a dense layer's identity CSR has one hit per token; a token with none keeps only the shared one)
+    to, hr, hw = ora.moe_shared_hits(np.array([0, 0, 3], np.uint32), np.array([5, 6, 7], np.uint32), np.array([1, 2, 3], np.float32), 8)
+    assert to.tolist() == [0, 1, 5] and hr.tolist() == [8, 5, 6, 7, 9] and hw.tolist() == [1.0, 1.0, 2.0, 3.0, 1.0]
