@@ -626,6 +626,7 @@ int apk_timer_begin(apk_ctx* c) {
     if (!c) return fail(APK_DECLINE_NULL, "apk_timer_begin: ctx is NULL");
     std::lock_guard<std::mutex> lock(c->mu);
     NOT_WHILE_CAPTURING(c, "apk_timer_begin");
+    if (int rc = set_device(c)) return rc;
     HIP_TRY(hipEventRecord(c->ev0, c->stream));
     return APK_OK;
 }
@@ -633,6 +634,7 @@ int apk_timer_end(apk_ctx* c, float* ms_out) {
     if (!c || !ms_out) return fail(APK_DECLINE_NULL, "apk_timer_end: NULL argument");
     std::lock_guard<std::mutex> lock(c->mu);
     NOT_WHILE_CAPTURING(c, "apk_timer_end");
+    if (int rc = set_device(c)) return rc;
     HIP_TRY(hipEventRecord(c->ev1, c->stream));
     uint64_t t0 = now_ns();
     HIP_TRY(hipEventSynchronize(c->ev1));
@@ -851,6 +853,11 @@ int apk_postnorm_add_rmsnorm_rows(apk_ctx* c, void* x, void* delta, const float*
     if (p.variant != ADDNORM_TILED) {
         // rows outside the tiled kernels (not whole 16-byte tiles, longer than they hold, short rows in bulk):
         // the reference's own two steps, the delta normalised in place first
+        // (the one decline the second step could raise after the first has run is checked first)
+        apk_plan p2;
+        if (int rc = plan_add_rmsnorm(n, rows, dtype, &p2)) return rc;
+        if (p2.variant != ADDNORM_RAGGED && (!aligned16(x) || !aligned16(h) || !aligned16(gamma) || !aligned16(delta) || !aligned16(post_gamma)))
+            return fail(APK_DECLINE_SHAPE, "apk_postnorm_add_rmsnorm_rows: tensors must be 16-byte aligned");
         if (int rc = apk_add_rmsnorm_rows(c, delta, nullptr, delta, post_gamma, n, rows, eps, dtype)) return rc;
         return apk_add_rmsnorm_rows(c, x, delta, h, gamma, n, rows, eps, dtype);
     }
@@ -1296,7 +1303,7 @@ int apk_moe_shared_hits(apk_ctx* c, const uint32_t* tok_off, const uint32_t* hit
                         size_t total_rows, uint32_t* tok_off_out, uint32_t* hit_row_out, float* hit_w_out) {
     if (!c) return fail(APK_DECLINE_NULL, "apk_moe_shared_hits: ctx is NULL");
     CallScope s(c);
-    if (!tok_off || !tok_off_out || (rows && (!hit_row_out || !hit_w_out)) || (total_rows && (!hit_row || !hit_w)))
+    if (!tok_off || !tok_off_out || (rows && (!hit_row_out || !hit_w_out || !hit_row || !hit_w)))
         return fail(APK_DECLINE_NULL, "apk_moe_shared_hits: NULL tensor");
     if (rows >= 0x7fffffffu || total_rows + rows > 0xffffffffu) return fail(APK_DECLINE_SHAPE, "apk_moe_shared_hits: too large");
     if (tok_off_out == tok_off || hit_row_out == hit_row || hit_w_out == hit_w)

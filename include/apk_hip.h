@@ -430,7 +430,8 @@ int apk_attn_prologue_rows(apk_ctx* ctx, const apk_attn_prologue* args);
 /* Launch plans (no context, no GPU; see apk_plan): what apk_add_rmsnorm_rows, apk_postnorm_add_rmsnorm_rows, apk_qknorm_rope_neox /
  * _norm (adjacent_pairs != 0) / _kv_store (with_kv_store != 0), apk_scatter_rows and apk_embed_rows /
  * apk_dequant_rows launch for these sizes.  Return APK_OK with plan filled (kernel "" and grid 0 when
- * the call would be a no-op), or the decline the entry itself would return for the sizes.  They have no
+ * the call would be a no-op), or the decline the entry itself would return for the sizes.  (apk_plan_attn_prologue_rows:
+ * the launch over q and k; a v_bias without the cache store is one more launch, of the plain bias kernel.)  They have no
  * counterpart in the reference: its hosts size their dispatches inline (e.g. gpu/cuda/runtime/gemm.rs:218-233). */
 int apk_plan_add_rmsnorm_rows(size_t n, size_t rows, int dtype, apk_plan* plan);
 int apk_plan_postnorm_add_rmsnorm_rows(size_t n, size_t rows, int dtype, apk_plan* plan);

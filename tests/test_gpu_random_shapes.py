@@ -101,6 +101,97 @@ def test_add_rmsnorm_random_batches(be, ora, case):
 
 
 @pytest.mark.parametrize("case", range(CASES))
+def test_postnorm_add_rmsnorm_random(be, ora, case):
+    """The sandwich norm and the next norm in one call, over drawn row counts and lengths (tiled kernels, ragged and
+    short rows): against the oracle's two norms and the add between them."""
+    g = np.random.default_rng(1700 + case)
+    f16 = bool(case & 1)
+    if case % 4 == 3:  # batches in the thousands
+        n = int(g.integers(8, 500)) * 8
+        rows = int(g.integers(1000, min(6000, 6_000_000 // n) + 1))
+    else:
+        rows = int(g.integers(1, 70))
+        n = int(g.integers(1, 1300)) * 8 if case % 3 else int(g.integers(1, 9000))
+    x, d = act(g, (rows, n), f16), act(g, (rows, n), f16)
+    pg, gamma = S().normal_f32(g, n, 1.0, 0.05), S().normal_f32(g, n, 1.0, 0.05)
+    nd = np.zeros_like(d)
+    ora.add_rmsnorm_rows(d.copy(), None, nd, pg, 1e-6)
+    wx, wh = x.copy(), np.zeros_like(x)
+    ora.add_rmsnorm_rows(wx, nd, wh, gamma, 1e-6)
+    tx, th = dev(x), torch.zeros_like(dev(x))
+    be.postnorm_add_rmsnorm_rows(tx, dev(d), dev(pg), th, dev(gamma), 1e-6)
+    what = (rows, n, f16)
+    if f16:
+        # the sum can cancel: held to 2 ulp, or to one ulp of its larger operand where the two-step path's
+        # normalised delta is an ulp off
+        fv = lambda a: a.view(np.float16).astype(np.float64)  # noqa: E731
+        key = lambda b: np.where(b.astype(np.int32) & 0x8000, 0x8000 - b.astype(np.int32), b.astype(np.int32))  # noqa: E731
+        slack = 2.0 ** -10 * np.maximum(np.abs(fv(x)), np.abs(fv(nd)))
+        gx = host(tx)
+        assert np.all((np.abs(key(gx) - key(wx)) <= TOL_F16_ULP) | (np.abs(fv(gx) - fv(wx)) <= slack)), what
+        assert np.mean(gx == wx) > 0.99, what
+        assert np.mean(np.abs(key(host(th)) - key(wh)) <= TOL_F16_ULP) > 0.999, what
+    else:
+        check_float(host(tx), wx, False, what)
+        check_float(host(th), wh, False, what)
+
+
+@pytest.mark.parametrize("case", range(CASES))
+def test_attn_prologue_random(be, ora, case):
+    """Projection biases (any subset), per-head norms (any subset), either pairing, drawn head geometry, with and
+    without the K/V cache store, against the oracle's ops in the reference's order (attention.rs:125-165, kv.rs:682-697)."""
+    g = np.random.default_rng(2600 + case)
+    f16 = bool(case & 1)
+    rows = int(g.integers(1, 60)) if case % 6 else int(g.integers(1500, 2600))
+    n_q, n_kv = int(g.integers(1, 40)), int(g.integers(1, 9))
+    hd = int(g.choice([64, 128, 256]))
+    if hd == 256 or rows > 1000:
+        n_q = min(n_q, 12)
+    style = int(g.integers(0, 2))
+    es = 2 if f16 else 4
+    tile = 16 // es if style else 2 * (16 // es)  # rotary widths the tiled kernels take
+    rot = hd if case % 3 else int(g.integers(1, hd // tile + 1)) * tile
+    store = case % 4 != 3
+    q, k, v = act(g, (rows, n_q * hd), f16), act(g, (rows, n_kv * hd), f16), act(g, (rows, n_kv * hd), f16)
+    qb = S().normal_f32(g, n_q * hd, 0.0, 0.5) if case % 5 else None
+    kb = S().normal_f32(g, n_kv * hd, 0.0, 0.5) if case % 7 else None
+    vb = S().normal_f32(g, n_kv * hd, 0.0, 0.5) if case % 2 or case % 3 else None
+    qw = S().normal_f32(g, hd, 1.0, 0.05) if case % 4 < 2 else None
+    kw = S().normal_f32(g, hd, 1.0, 0.05) if case % 4 in (0, 3) else None
+    cap = rows + 11
+    positions = g.permutation(cap)[:rows].astype(np.uint32)
+    ropes = ora.rope_table([int(p) for p in positions], ora.rope_inv_freq(rot, 1e6))
+    wq, wk = q.copy(), k.copy()
+    ora.qknorm_rope_rows(wq, wk, n_q, n_kv, hd, qw, kw, ropes, 1e-6, style=style, q_bias=qb, k_bias=kb)
+    wv = v
+    if vb is not None:
+        wv = ora.f16_bits_to_f32(v) if f16 else v.copy()
+        ora.add_bias_rows(wv, vb)
+        wv = ora.f32_to_f16_bits(wv) if f16 else wv
+    wkc, wvc = np.zeros((cap, n_kv * hd), np.uint16), np.zeros((cap, n_kv * hd), np.uint16)
+    ora.kv_store_rows(wk, wv, positions, wkc, wvc)
+    tq, tk, tv = dev(q), dev(k), dev(v)
+    kc = torch.zeros((cap, n_kv * hd), dtype=torch.float16, device="cuda")
+    vc = torch.zeros_like(kc)
+    d = lambda a: None if a is None else dev(a)  # noqa: E731
+    kwargs = dict(q_bias=d(qb), k_bias=d(kb), v_bias=d(vb), q_norm=d(qw), k_norm=d(kw), adjacent_pairs=bool(style), rot_dim=rot)
+    if store:
+        kwargs.update(cache_pos=dev(positions), k_cache=kc, v_cache=vc)
+    be.attn_prologue_rows(tq, tk, tv, n_q, n_kv, hd, 1e-6, dev(ropes), **kwargs)
+    what = (rows, n_q, n_kv, hd, rot, style, f16, store, qb is not None, kb is not None, vb is not None)
+    gk = host(tk)
+    check_float(host(tq), wq, f16, what)
+    check_float(gk, wk, f16, what)
+    assert np.array_equal(host(tv), wv), what
+    if store:
+        assert np.array_equal(host(vc), wvc), what
+        mine_k, mine_v = np.zeros_like(wkc), np.zeros_like(wvc)
+        ora.kv_store_rows(gk, wv, positions, mine_k, mine_v)
+        assert np.array_equal(host(kc), mine_k), what
+        assert f16_ulp_diff(host(kc), wkc) <= (TOL_F16_ULP if f16 else 1), what
+
+
+@pytest.mark.parametrize("case", range(CASES))
 def test_qknorm_rope_random(be, ora, case):
     g = np.random.default_rng(2000 + case)
     f16 = bool(case & 1)
