@@ -106,3 +106,31 @@ def test_rope_inv_freq_is_the_reference_powf_series():
         assert np.array_equal(inv.view(np.uint32), ora.rope_inv_freq(d, base).view(np.uint32))
         assert inv[0] == 1.0 and np.all(np.diff(inv) < 0)
     assert L.apk_rope_inv_freq(0, 1e4, None) == 0 and L.apk_rope_inv_freq(8, 1e4, None) == 3
+
+
+def test_header_is_plain_c_and_the_ctypes_structs_have_its_layout(tmp_path):
+    """include/apk_hip.h is what a C, Rust or cgo binding reads: it must compile as C11 on its own, and the two
+    structs that cross the boundary (apk_plan, apk_attn_prologue) must have the layout the ctypes mirror assumes."""
+    import shutil
+
+    lib, _ = _lib()
+    cc = shutil.which("gcc") or shutil.which("cc")
+    assert cc, "no C compiler"
+    inc = os.path.join(ROOT, "include")
+    subprocess.check_call([cc, "-std=c11", "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", "-x", "c",
+                           os.path.join(inc, "apk_hip.h")])
+    fields = {"apk_plan": [f[0] for f in lib.Plan._fields_], "apk_attn_prologue": [f[0] for f in lib.AttnPrologue._fields_]}
+    src = ['#include <stddef.h>', '#include <stdio.h>', '#include "apk_hip.h"', "int main(void) {"]
+    for st, names in fields.items():
+        src.append(f'    printf("{st} %zu\\n", sizeof({st}));')
+        for f in names:
+            src.append(f'    printf("{st}.{f} %zu\\n", offsetof({st}, {f}));')
+    src += ["    return 0;", "}"]
+    cfile, exe = tmp_path / "layout.c", tmp_path / "layout"
+    cfile.write_text("\n".join(src))
+    subprocess.check_call([cc, "-std=c11", f"-I{inc}", "-o", str(exe), str(cfile)])
+    got = dict(line.rsplit(" ", 1) for line in subprocess.check_output([str(exe)], text=True).splitlines())
+    for st, cls in (("apk_plan", lib.Plan), ("apk_attn_prologue", lib.AttnPrologue)):
+        assert int(got[st]) == C.sizeof(cls), st
+        for f in fields[st]:
+            assert int(got[f"{st}.{f}"]) == getattr(cls, f).offset, (st, f)
