@@ -271,6 +271,15 @@ class Backend:
         if not self._recording and self.take_faults() & _l.FAULT_CACHE_RANGE:
             raise AssertionError("position past capacity")
 
+    def cast(self, src, dtype):
+        """allpaka_dtype::f32_to_f16 / f16_to_f32 over a tensor (dtype/src/lib.rs:129-184), bit for bit."""
+        assert src.dtype in (torch.float32, torch.float16) and dtype in (torch.float32, torch.float16) and dtype != src.dtype
+        dst = torch.empty(src.shape, dtype=dtype, device=self.device)
+        self._enter()
+        check(self.L.apk_cast(self.h, _ptr(src), _dt(src), _ptr(dst), _dt(dst), src.numel()))
+        self._leave()
+        return dst
+
     def add_bias_rows(self, x, bias):
         """add_bias_rows (model/loader.rs:519-523): x[r][i] += bias[i] over rows of bias.numel() elements."""
         n = bias.numel()

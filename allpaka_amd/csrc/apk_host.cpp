@@ -68,7 +68,7 @@ std::vector<std::string> all_kernel_names() {
                                   "apk_moe_permute", "apk_gather_rows", "apk_scatter_rows_t1", "apk_scatter_rows_t2", "apk_argmax_rows", "apk_add_rmsnorm_ragged_f32", "apk_add_rmsnorm_ragged_f16", "apk_copy",
                                   "apk_qknorm_rope_generic_f32", "apk_qknorm_rope_generic_f16", "apk_route_topk_wide", "apk_route_topk_e64", "apk_route_topk_e128", "apk_route_group_small_e64", "apk_route_group_small_e128",
                                   "apk_route_group_small_e256", "apk_route_group_small_e1024", "apk_add_assign_f32", "apk_add_assign_f16", "apk_softmax_rows", "apk_moe_count", "apk_moe_rank",
-                                  "apk_add_bias_rows_f32", "apk_add_bias_rows_f16", "apk_moe_shared_hits"};
+                                  "apk_add_bias_rows_f32", "apk_add_bias_rows_f16", "apk_moe_shared_hits", "apk_cast_f32_f16", "apk_cast_f16_f32"};
     for (const char* t : {"f32", "f16"}) {
         for (const char* f : {"q5k", "q6k", "q2k", "q3k", "q5_0", "f16", "f32", "bf16"}) v.push_back(std::string("apk_embed_") + f + "_" + t);
         for (int c : kAddnormTiles) v.push_back(std::string("apk_add_rmsnorm_") + t + "_c" + std::to_string(c));
@@ -794,6 +794,23 @@ int apk_add_assign(apk_ctx* c, void* a, const void* b, size_t n, int dtype) {
     void* args[] = {&a, &b, &n64};
     return launch_keyed(c, OP_ADD_ASSIGN, (uint32_t)dtype,
                         [&] { return std::string(dtype == APK_F32 ? "apk_add_assign_f32" : "apk_add_assign_f16"); }, (unsigned)grid, 256, 0, args);
+}
+
+int apk_cast(apk_ctx* c, const void* src, int src_dtype, void* dst, int dst_dtype, size_t n) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_cast: ctx is NULL");
+    CallScope s(c);
+    if (!elem_size(src_dtype) || !elem_size(dst_dtype) || src_dtype == dst_dtype)
+        return fail(APK_DECLINE_UNSUPPORTED, "apk_cast: from dtype %d to dtype %d", src_dtype, dst_dtype);
+    if (n == 0) return APK_OK;
+    if (!src || !dst) return fail(APK_DECLINE_NULL, "apk_cast: NULL tensor");
+    if (!aligned16(src) || !aligned16(dst)) return fail(APK_DECLINE_SHAPE, "apk_cast: tensors must be 16-byte aligned");
+    if (int rc = set_device(c)) return rc;
+    uint64_t grid = (n / 8 + 255) / 256;
+    if (grid == 0) grid = 1;
+    if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_cast: n too large");
+    uint64_t n64 = n;
+    void* args[] = {&src, &dst, &n64};
+    return launch(c, src_dtype == APK_F32 ? "apk_cast_f32_f16" : "apk_cast_f16_f32", (unsigned)grid, 256, 0, args);
 }
 
 int apk_softmax_rows(apk_ctx* c, float* x, size_t rows, size_t n) {

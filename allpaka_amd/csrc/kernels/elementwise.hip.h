@@ -134,6 +134,52 @@ extern "C" __global__ __launch_bounds__(256) void apk_add_bias_rows_f16(f16_t* x
     add_bias_rows_body<f16_t>(x, bias, rows, n);
 }
 
+// Activation type conversion between the reference's f32 and the fp16 storage form (allpaka_dtype::f32_to_f16 /
+// f16_to_f32 over slices, crates/allpaka-dtype/src/lib.rs:129-184; the reference's CUDA cast_f32_to_f16 /
+// cast_f16_to_f32, gpu/cuda/kernels.rs:448, :3625).  The hardware conversions are the reference's for every finite
+// value, infinities and subnormals (round to nearest even; overflow to infinity); NaNs are patched to the reference's
+// bits: narrowing gives the canonical quiet NaN sign | 0x7e00, widening keeps the payload (frac << 13) and does not
+// quiet a signalling NaN.  8 elements per lane, a scalar tail.
+DEV uint16_t narrow_ref(float x) {
+    const uint32_t b = __builtin_bit_cast(uint32_t, x);
+    if ((b & 0x7fffffffu) > 0x7f800000u) return (uint16_t)(((b >> 16) & 0x8000u) | 0x7e00u);
+    return __builtin_bit_cast(uint16_t, (f16_t)x);
+}
+DEV float widen_ref(uint16_t h) {
+    if ((h & 0x7c00u) == 0x7c00u && (h & 0x3ffu))
+        return __builtin_bit_cast(float, ((uint32_t)(h & 0x8000u) << 16) | 0x7f800000u | ((uint32_t)(h & 0x3ffu) << 13));
+    return (float)__builtin_bit_cast(f16_t, h);
+}
+extern "C" __global__ __launch_bounds__(256) void apk_cast_f32_f16(const float* src, uint16_t* dst, uint64_t n) {
+    const uint64_t nvec = n / 8, c = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c < nvec) {
+        const f32x4 a = __builtin_nontemporal_load((const f32x4*)src + 2 * c), b = __builtin_nontemporal_load((const f32x4*)src + 2 * c + 1);
+        u32x4 o;
+        o[0] = narrow_ref(a.x) | (uint32_t)narrow_ref(a.y) << 16;
+        o[1] = narrow_ref(a.z) | (uint32_t)narrow_ref(a.w) << 16;
+        o[2] = narrow_ref(b.x) | (uint32_t)narrow_ref(b.y) << 16;
+        o[3] = narrow_ref(b.z) | (uint32_t)narrow_ref(b.w) << 16;
+        __builtin_nontemporal_store(o, (u32x4*)dst + c);
+    }
+    if (blockIdx.x == gridDim.x - 1)
+        for (uint64_t i = nvec * 8 + threadIdx.x; i < n; i += blockDim.x) dst[i] = narrow_ref(src[i]);
+}
+extern "C" __global__ __launch_bounds__(256) void apk_cast_f16_f32(const uint16_t* src, float* dst, uint64_t n) {
+    const uint64_t nvec = n / 8, c = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c < nvec) {
+        const u32x4 t = __builtin_nontemporal_load((const u32x4*)src + c);
+        f32x4 a, b;
+        a.x = widen_ref((uint16_t)t[0]); a.y = widen_ref((uint16_t)(t[0] >> 16));
+        a.z = widen_ref((uint16_t)t[1]); a.w = widen_ref((uint16_t)(t[1] >> 16));
+        b.x = widen_ref((uint16_t)t[2]); b.y = widen_ref((uint16_t)(t[2] >> 16));
+        b.z = widen_ref((uint16_t)t[3]); b.w = widen_ref((uint16_t)(t[3] >> 16));
+        __builtin_nontemporal_store(a, (f32x4*)dst + 2 * c);
+        __builtin_nontemporal_store(b, (f32x4*)dst + 2 * c + 1);
+    }
+    if (blockIdx.x == gridDim.x - 1)
+        for (uint64_t i = nvec * 8 + threadIdx.x; i < n; i += blockDim.x) dst[i] = widen_ref(src[i]);
+}
+
 // Softmax over rows in place (ops::softmax, activation.rs:5-16): max, exp(v - max), sum,
 // times 1/sum.  A wave per row, any row length; the sum runs in lane order, not index order.
 extern "C" __global__ __launch_bounds__(256) void apk_softmax_rows(float* x, int rows, int n) {

@@ -88,6 +88,7 @@ SYMBOLS = {
     "apk_plan_scatter_rows": (_i, [_sz, _sz, _sz, _i, _plan]),
     "apk_plan_attn_prologue_rows": (_i, [C.POINTER(AttnPrologue), _plan]),
     "apk_add_bias_rows": (_i, [_vp, _vp, _vp, _sz, _sz, _i]),
+    "apk_cast": (_i, [_vp, _vp, _i, _vp, _i, _sz]),
     "apk_moe_shared_hits": (_i, [_vp, _vp, _vp, _vp, _sz, _sz, _vp, _vp, _vp]),
     "apk_attn_prologue_rows": (_i, [_vp, C.POINTER(AttnPrologue)]),
     "apk_plan_embed_rows": (_i, [_i, _sz, _sz, _i, _plan]),

@@ -391,6 +391,13 @@ int apk_argmax_rows(apk_ctx* ctx, const float* logits, size_t rows, size_t n, ui
  * figures of the other kernels are calibrated against. */
 int apk_copy(apk_ctx* ctx, const void* src, void* dst, size_t bytes);
 
+/* dst[i] = src[i] converted between the reference's f32 activations and the fp16 storage form: APK_F32 ->
+ * APK_F16 is allpaka_dtype::f32_to_f16 (crates/allpaka-dtype/src/lib.rs:151-184: round to nearest even,
+ * overflow to infinity, subnormals kept, NaN -> sign | 0x7e00), APK_F16 -> APK_F32 is f16_to_f32 (:129-146:
+ * exact, NaN payloads kept); bit for bit, for every input.  The reference's CUDA cast_f32_to_f16 /
+ * cast_f16_to_f32 (gpu/cuda/kernels.rs:448, :3625).  Any n; src and dst distinct, 16-byte aligned. */
+int apk_cast(apk_ctx* ctx, const void* src, int src_dtype, void* dst, int dst_dtype, size_t n);
+
 /* x[r][i] += bias[i] over rows of length n (add_bias_rows, crates/allpaka-model/src/model/loader.rs:519-523:
  * ops::add_assign_slice(row, bias) per row).  x: [rows][n] of dtype, in place; bias: f32[n]. */
 int apk_add_bias_rows(apk_ctx* ctx, void* x, const float* bias, size_t rows, size_t n, int dtype);

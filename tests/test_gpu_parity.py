@@ -637,6 +637,41 @@ def test_kv_store_position_past_capacity_is_flagged_not_faulted(be, ora):
     assert host(kc)[1].any() and host(kc)[3].any() and not host(kc)[[0, 2]].any()
 
 
+# ------------------------------------------------ f32 <-> fp16 activation conversion
+def test_cast_is_the_reference_conversion_for_every_pattern(be, ora):
+    """allpaka_dtype::f16_to_f32 over all 65 536 half patterns (NaN payloads kept, signalling NaNs not quieted), and
+    f32_to_f16 (lib.rs:151-184) over every half value's f32 image, its f32 neighbours, every midpoint between
+    consecutive halves (the ties) and their neighbours, the overflow threshold, f32 subnormals, infinities, NaNs of
+    every kind, and two million random bit patterns -- bit for bit."""
+    halves = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    wide = host(be.cast(dev(halves), torch.float32)).view(np.uint32)
+    assert np.array_equal(wide, ora.f16_bits_to_f32(halves).view(np.uint32))
+    finite = halves[(halves & 0x7c00) != 0x7c00]
+    img = ora.f16_bits_to_f32(finite).view(np.uint32).astype(np.int64)
+    nxt = ora.f16_bits_to_f32(((finite & 0x7fff) + 1).astype(np.uint16) | (finite & 0x8000)).view(np.uint32).astype(np.int64)
+    mid = (img + nxt) // 2  # adjacent normal halves of one sign: the f32 halfway between them
+    sub = (np.arange(0, 2049, dtype=np.float64) * 2.0 ** -25).astype(np.float32)  # halfway between adjacent subnormal halves
+    sub = np.concatenate([sub, -sub]).view(np.uint32).astype(np.int64)
+    cases = [img + d for d in (-1, 0, 1)] + [mid + d for d in (-1, 0, 1)] + [sub + d for d in (-1, 0, 1)]
+    g = np.random.default_rng(77)
+    special = np.array([0x7f800000, 0xff800000, 0x7fc00000, 0xffc00000, 0x7f800001, 0xff800001, 0x7fffffff, 0x7fa00000, 0x00000001,
+                        0x80000001, 0x007fffff, 0x00800000, 0x33000000, 0x33000001, 0x32ffffff, 0x477fe000, 0x477fefff, 0x477ff000,
+                        0x477ff001, 0x7f7fffff, 0xff7fffff, 0, 0x80000000], dtype=np.int64)
+    bits = np.concatenate(cases + [special, g.integers(0, 2 ** 32, size=2_000_003, dtype=np.int64)])
+    bits = np.clip(bits, 0, 2 ** 32 - 1).astype(np.uint32)
+    x = bits.view(np.float32)
+    got = host(be.cast(torch.from_numpy(x.copy()).cuda(), torch.float16))
+    assert np.array_equal(got, ora.f32_to_f16_bits(x))
+    # a length that is not whole tiles, and the declines
+    odd = x[:1003].copy()
+    assert np.array_equal(host(be.cast(torch.from_numpy(odd).cuda(), torch.float16)), ora.f32_to_f16_bits(odd))
+    import allpaka_amd as apk
+
+    t = torch.zeros(16, device="cuda")
+    with pytest.raises(apk.Declined):
+        apk.lib.check(be.L.apk_cast(be.h, t.data_ptr(), 0, t.data_ptr(), 0, 16))
+
+
 # ------------------------------------- projection biases, and the whole q/k/v step as one call
 @pytest.mark.parametrize("rows,n", [(1, 1024), (6, 5120), (300, 4096), (5, 1001), (64, 24), (3, 7)])
 @pytest.mark.parametrize("f16", [False, True])
