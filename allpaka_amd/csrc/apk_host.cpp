@@ -76,18 +76,14 @@ std::vector<std::string> all_kernel_names() {
         for (int l : {4, 8, 16, 32}) v.push_back(std::string("apk_add_rmsnorm_small_") + t + "_l" + std::to_string(l));
         for (int c : {1, 2, 4}) v.push_back(std::string("apk_combine_add_rmsnorm_") + t + "_c" + std::to_string(c));
         for (int hd : kQkHeadDims) v.push_back(std::string("apk_layer_prologue_") + t + "_hd" + std::to_string(hd));
-        for (int hd : kQkHeadDims)  // with the projection biases (two passes per q wave exist in fp16 only)
-            for (int it : kQkIters)
-                for (const char* style : {"", "pairs_"})
-                    for (const char* kv : {"", "kv_"})
-                        if (it == 1 || t[1] == '1')
-                            v.push_back(std::string("apk_qknorm_rope_") + style + kv + "bias_" + t + "_hd" + std::to_string(hd) + "_i" + std::to_string(it));
-        for (int hd : kQkHeadDims)
-            for (int it : kQkIters) {
-                for (const char* style : {"", "pairs_"})
-                    for (const char* kv : {"", "kv_"})
-                        v.push_back(std::string("apk_qknorm_rope_") + style + kv + t + "_hd" + std::to_string(hd) + "_i" + std::to_string(it));
-            }
+        for (const char* pfx : {"apk_qknorm_rope_", "apk_rope_"})  // with a norm weight for q and / or k; with none
+            for (int hd : kQkHeadDims)
+                for (int it : kQkIters)
+                    for (const char* style : {"", "pairs_"})
+                        for (const char* kv : {"", "kv_"})
+                            for (const char* bias : {"", "bias_"})
+                                if (it == 1 || t[1] == '1')  // two passes per q wave exist in fp16 only
+                                    v.push_back(std::string(pfx) + style + kv + bias + t + "_hd" + std::to_string(hd) + "_i" + std::to_string(it));
     }
     return v;
 }
@@ -203,9 +199,10 @@ void plan_name(apk_plan* p, const std::string& k) { snprintf(p->kernel, sizeof p
 
 enum { QK_TILED = 0, QK_GENERIC = 1 };
 // style: 0 = NeoX pairs (i, i + rot_dim/2), 1 = adjacent pairs (2i, 2i+1); with_kv: the K/V cache store fused in
-// with_bias: the kernels that also add the projection biases
+// with_bias: the kernels that also add the projection biases; with_norm = false: no norm weight for q or for k
+// (the kernels without statistics)
 int plan_qknorm_rope(size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim, int style, int dtype, bool with_kv,
-                     apk_plan* p, bool with_bias = false) {
+                     apk_plan* p, bool with_bias = false, bool with_norm = true) {
     plan_reset(p);
     const int es = elem_size(dtype);
     if (!es) return fail(APK_DECLINE_UNSUPPORTED, "apk_qknorm_rope: dtype %d", dtype);
@@ -250,7 +247,7 @@ int plan_qknorm_rope(size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size
     const uint64_t grid = (waves * 64 + block - 1) / block;
     if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope: too large");
     p->variant = QK_TILED;
-    plan_name(p, std::string("apk_qknorm_rope_") + (style ? "pairs_" : "") + (with_kv ? "kv_" : "") + (with_bias ? "bias_" : "") + t + "_hd" +
+    plan_name(p, std::string(with_norm ? "apk_qknorm_rope_" : "apk_rope_") + (style ? "pairs_" : "") + (with_kv ? "kv_" : "") + (with_bias ? "bias_" : "") + t + "_hd" +
                      std::to_string(head_dim) + "_i" + std::to_string(iter));
     p->grid = (unsigned)grid;
     p->block = block;
@@ -909,7 +906,8 @@ static int qknorm_rope_common(apk_ctx* c, void* q, void* k, const float* qw, con
                               const KvStore* kv, int style = 0, bool validate_only = false, const QkvBias* bias = nullptr) {
     apk_plan p;
     if (bias && !bias->q && !bias->k && !bias->v) bias = nullptr;
-    if (int rc = plan_qknorm_rope(rows, n_q, n_kv, head_dim, rot_dim, style, dtype, kv != nullptr, &p, bias != nullptr)) return rc;
+    const bool with_norm = qw || kw;
+    if (int rc = plan_qknorm_rope(rows, n_q, n_kv, head_dim, rot_dim, style, dtype, kv != nullptr, &p, bias != nullptr, with_norm)) return rc;
     if (rows == 0 || n_q + n_kv == 0) return APK_OK;
     if ((n_q && !q) || (n_kv && !k) || (!rope && rot_dim)) return fail(APK_DECLINE_NULL, "apk_qknorm_rope: NULL tensor");
     if ((q && !aligned16(q)) || (k && !aligned16(k)) || !aligned16(rope) || (qw && !aligned16(qw)) || (kw && !aligned16(kw)))
@@ -936,7 +934,7 @@ static int qknorm_rope_common(apk_ctx* c, void* q, void* k, const float* qw, con
         return launch(c, p.kernel, p.grid, p.block, 0, gargs);
     }
     auto which = [&] { return std::string(p.kernel); };
-    const uint32_t variant = (uint32_t)(bias != nullptr) << 21 | (uint32_t)style << 20 | (uint32_t)dtype << 16 | (uint32_t)head_dim << 4 | p.tiles_per_lane;
+    const uint32_t variant = (uint32_t)with_norm << 22 | (uint32_t)(bias != nullptr) << 21 | (uint32_t)style << 20 | (uint32_t)dtype << 16 | (uint32_t)head_dim << 4 | p.tiles_per_lane;
     if (kv && bias) {
         uint32_t cap32 = (uint32_t)kv->capacity;
         void* kargs[] = {&q, &k, (void*)&kv->v, &qw, &kw, &rope, (void*)&kv->cache_pos, (void*)&kv->k_cache, (void*)&kv->v_cache,
@@ -1422,7 +1420,8 @@ int apk_plan_attn_prologue_rows(const apk_attn_prologue* a, apk_plan* plan) {
     if (!plan || !a) return fail(APK_DECLINE_NULL, "apk_plan_attn_prologue_rows: NULL argument");
     const bool store = a->k_cache || a->v_cache || a->cache_pos;
     const bool bias = a->q_bias || a->k_bias || (store && a->v_bias);
-    return plan_qknorm_rope(a->rows, a->n_q, a->n_kv, a->head_dim, a->rot_dim, a->adjacent_pairs ? 1 : 0, a->dtype, store, plan, bias);
+    return plan_qknorm_rope(a->rows, a->n_q, a->n_kv, a->head_dim, a->rot_dim, a->adjacent_pairs ? 1 : 0, a->dtype, store, plan, bias,
+                            a->q_norm || a->k_norm);
 }
 
 int apk_plan_scatter_rows(size_t rows, size_t k, size_t cols, int dtype, apk_plan* plan) {

@@ -36,7 +36,9 @@
 // v right in front of this loop; loader.rs:519-523) are added as the tiles are widened: bias [nheads*HD] f32 for the
 // item's tensor (NULL: none); with the cache store, vbias is added to the row's v, which is written back (vout)
 // as well as narrowed into the cache.
-template <typename T, int HD, int ITER, bool KV = false, bool PAIRS = false, bool BIAS = false>
+// NORM = false: neither tensor has a norm weight (the Llama / Qwen2 families: biases or not, then the rotation):
+// no statistics, no weight tiles -- the launch then runs at the speed of a plain copy of the same bytes.
+template <typename T, int HD, int ITER, bool KV = false, bool PAIRS = false, bool BIAS = false, bool NORM = true>
 DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, float eps, int l, int sub, int rot,
                  f16_t* kc = nullptr, const T* vrow = nullptr, f16_t* vc = nullptr, const float* bias = nullptr,
                  const float* vbias = nullptr, T* vout = nullptr) {
@@ -73,12 +75,14 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
         io<float>::load(trow + sc_a + i, sc + i);
         io<float>::load(trow + sc_b + i, sc + EPL + i);
     }
-    const float* wp = w ? w : trow;
-    const int w_a = w ? off_a : 0, w_b = w ? off_b : 0;
+    if constexpr (NORM) {
+        const float* wp = w ? w : trow;
+        const int w_a = w ? off_a : 0, w_b = w ? off_b : 0;
 #pragma unroll
-    for (int i = 0; i < EPL; i += 4) {
-        io<float>::load(wp + w_a + i, wa + i);
-        io<float>::load(wp + w_b + i, wb + i);
+        for (int i = 0; i < EPL; i += 4) {
+            io<float>::load(wp + w_a + i, wa + i);
+            io<float>::load(wp + w_b + i, wb + i);
+        }
     }
     typename io<T>::raw_t araw[ITER], braw[ITER], varaw[ITER], vbraw[ITER];
     float ba[BIAS ? ITER : 1][EPL], bb[BIAS ? ITER : 1][EPL], bva[BIAS && KV ? ITER : 1][EPL], bvb[BIAS && KV ? ITER : 1][EPL];
@@ -116,7 +120,7 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
         }
     }
     __builtin_amdgcn_sched_barrier(0);  // every load above; all uses below
-    const bool normed = w != nullptr;  // uniform for the wave
+    const bool normed = NORM && w != nullptr;  // uniform for the wave
 #pragma unroll
     for (int it = 0; it < ITER; it++) {
         float a[EPL], b[EPL], oa[EPL], ob[EPL];
@@ -131,14 +135,17 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
                 }
             }
         }
-        acc_t ss = 0;
+        typename headstat<T>::scale_t scale{};
+        if constexpr (NORM) {
+            acc_t ss = 0;
 #pragma unroll
-        for (int i = 0; i < EPL; i++) {
-            ss = headstat<T>::sq(ss, a[i]);
-            ss = headstat<T>::sq(ss, b[i]);
+            for (int i = 0; i < EPL; i++) {
+                ss = headstat<T>::sq(ss, a[i]);
+                ss = headstat<T>::sq(ss, b[i]);
+            }
+            ss = group_sum<LPH>(ss);
+            scale = headstat<T>::rscale(ss, HD, eps);
         }
-        ss = group_sum<LPH>(ss);
-        const typename headstat<T>::scale_t scale = headstat<T>::rscale(ss, HD, eps);
         if constexpr (PAIRS) {
 #pragma unroll
             for (int i = 0; i < EPL; i++) {
@@ -202,7 +209,7 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
     }
 }
 
-template <typename T, int HD, int ITERQ, bool KV = false, bool PAIRS = false, bool BIAS = false>
+template <typename T, int HD, int ITERQ, bool KV = false, bool PAIRS = false, bool BIAS = false, bool NORM = true>
 DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv,
                           float eps, int rot, uint32_t vblock, T* v = nullptr, const uint32_t* cache_pos = nullptr,
                           f16_t* k_cache = nullptr, f16_t* v_cache = nullptr, uint32_t capacity = 0,
@@ -218,7 +225,7 @@ DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const fl
     if (wid >= nq_items + (uint64_t)rows * gk) return;  // whole wave
     if (wid < nq_items) {
         const uint64_t row = wid / gq;
-        qk_item<T, HD, ITERQ, false, PAIRS, BIAS>(q + row * (uint64_t)n_q * HD, n_q, (int)(wid % gq), qw, rope + row * (uint64_t)rot, eps, l, sub,
+        qk_item<T, HD, ITERQ, false, PAIRS, BIAS, NORM>(q + row * (uint64_t)n_q * HD, n_q, (int)(wid % gq), qw, rope + row * (uint64_t)rot, eps, l, sub,
                                                   rot, nullptr, nullptr, nullptr, qb);
     } else {
         const uint64_t w2 = wid - nq_items, row = w2 / gk;
@@ -227,76 +234,61 @@ DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const fl
             const uint32_t pos = cache_pos[row];
             const bool ok = pos < capacity;
             if (!ok && lane == 0 && w2 % gk == 0) atomicOr(fault, APK_FAULT_CACHE_RANGE);
-            qk_item<T, HD, 1, true, PAIRS, BIAS>(k + row * kv_dim, n_kv, (int)(w2 % gk), kw, rope + row * (uint64_t)rot, eps, l, sub, rot,
+            qk_item<T, HD, 1, true, PAIRS, BIAS, NORM>(k + row * kv_dim, n_kv, (int)(w2 % gk), kw, rope + row * (uint64_t)rot, eps, l, sub, rot,
                                                  ok ? k_cache + pos * kv_dim : nullptr, v + row * kv_dim,
                                                  ok ? v_cache + pos * kv_dim : nullptr, kb, vb, v + row * kv_dim);
         } else {
-            qk_item<T, HD, 1, false, PAIRS, BIAS>(k + row * kv_dim, n_kv, (int)(w2 % gk), kw, rope + row * (uint64_t)rot, eps, l, sub, rot,
+            qk_item<T, HD, 1, false, PAIRS, BIAS, NORM>(k + row * kv_dim, n_kv, (int)(w2 % gk), kw, rope + row * (uint64_t)rot, eps, l, sub, rot,
                                                   nullptr, nullptr, nullptr, kb);
         }
     }
 }
 // At most 128 VGPRs (at least 4 waves per SIMD).
 #define APK_QK_OCC __attribute__((amdgpu_waves_per_eu(4)))
-#define APK_QKROPE(T, TN, HD, ITER)                                                                          \
-    extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void apk_qknorm_rope_##TN##_hd##HD##_i##ITER(   \
+// One kernel per (norm or not, pairing, cache store, biases, type, head size, passes per q wave).  PFX: apk_qknorm_rope
+// (a norm weight for q and / or k) or apk_rope (none for either); PN: pairs_ or nothing.  The argument lists are the
+// same with and without norm weights (qw, kw are then NULL and unused).
+#define APK_QK_PLAIN(PFX, NORM, T, TN, HD, ITER, PAIRS, PN)                                                        \
+    extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void PFX##_##PN##TN##_hd##HD##_i##ITER(               \
         T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv, float eps, int rot) { \
-        qknorm_rope_body<T, HD, ITER>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x);                  \
-    }                                                                                                        \
-    extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void apk_qknorm_rope_pairs_##TN##_hd##HD##_i##ITER( \
-        T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv, float eps, int rot) { \
-        qknorm_rope_body<T, HD, ITER, false, true>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x);     \
+        qknorm_rope_body<T, HD, ITER, false, PAIRS, false, NORM>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x); \
     }
-#define APK_QKROPE_ALL(T, TN)                                                                                          \
-    APK_QKROPE(T, TN, 64, 1) APK_QKROPE(T, TN, 64, 2) APK_QKROPE(T, TN, 128, 1) APK_QKROPE(T, TN, 128, 2)              \
-    APK_QKROPE(T, TN, 256, 1) APK_QKROPE(T, TN, 256, 2)
-APK_QKROPE_ALL(float, f32)
-APK_QKROPE_ALL(f16_t, f16)
-
 // The same with the K/V cache store fused in: rotated k and the row's v narrowed to fp16
 // at cache row cache_pos[row] (one launch instead of QK-norm+RoPE, then two narrowing copies).
-#define APK_QKROPE_KV(T, TN, HD, ITER)                                                                            \
-    extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void apk_qknorm_rope_kv_##TN##_hd##HD##_i##ITER(     \
-        T* q, T* k, const T* v, const float* qw, const float* kw, const float* rope, const uint32_t* cache_pos,  \
+#define APK_QK_KV(PFX, NORM, T, TN, HD, ITER, PAIRS, PN)                                                           \
+    extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void PFX##_##PN##kv_##TN##_hd##HD##_i##ITER(          \
+        T* q, T* k, const T* v, const float* qw, const float* kw, const float* rope, const uint32_t* cache_pos,   \
         f16_t* k_cache, f16_t* v_cache, uint32_t capacity, int rows, int n_q, int n_kv, float eps, uint32_t* fault, int rot) { \
-        qknorm_rope_body<T, HD, ITER, true>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x, (T*)v, cache_pos, \
-                                            k_cache, v_cache, capacity, fault);                                   \
-    }                                                                                                             \
-    extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void apk_qknorm_rope_pairs_kv_##TN##_hd##HD##_i##ITER( \
-        T* q, T* k, const T* v, const float* qw, const float* kw, const float* rope, const uint32_t* cache_pos,  \
-        f16_t* k_cache, f16_t* v_cache, uint32_t capacity, int rows, int n_q, int n_kv, float eps, uint32_t* fault, int rot) { \
-        qknorm_rope_body<T, HD, ITER, true, true>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x, (T*)v, cache_pos, \
-                                                  k_cache, v_cache, capacity, fault);                             \
+        qknorm_rope_body<T, HD, ITER, true, PAIRS, false, NORM>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x, (T*)v, \
+                                                                cache_pos, k_cache, v_cache, capacity, fault);    \
     }
-#define APK_QKROPE_KV_ALL(T, TN)                                                                                       \
-    APK_QKROPE_KV(T, TN, 64, 1) APK_QKROPE_KV(T, TN, 64, 2) APK_QKROPE_KV(T, TN, 128, 1) APK_QKROPE_KV(T, TN, 128, 2)  \
-    APK_QKROPE_KV(T, TN, 256, 1) APK_QKROPE_KV(T, TN, 256, 2)
-APK_QKROPE_KV_ALL(float, f32)
-APK_QKROPE_KV_ALL(f16_t, f16)
-
-// With the projection biases (two passes per q wave in fp16 only, as without them).  Without the
-// cache store v is not touched here; with it, v + v_bias is written back to v and narrowed into the cache.
-#define APK_QKROPE_BIAS(T, TN, HD, ITER, PAIRS, PN)                                                               \
-    extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void apk_qknorm_rope_##PN##bias_##TN##_hd##HD##_i##ITER( \
+// With the projection biases.  Without the cache store v is not touched here; with it, v + v_bias is written back
+// to v and narrowed into the cache.
+#define APK_QK_BIAS(PFX, NORM, T, TN, HD, ITER, PAIRS, PN)                                                         \
+    extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void PFX##_##PN##bias_##TN##_hd##HD##_i##ITER(        \
         T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv, float eps, int rot, \
         const float* qb, const float* kb) {                                                                       \
-        qknorm_rope_body<T, HD, ITER, false, PAIRS, true>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x, nullptr, nullptr, \
-                                                          nullptr, nullptr, 0, nullptr, qb, kb, nullptr);         \
+        qknorm_rope_body<T, HD, ITER, false, PAIRS, true, NORM>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x, nullptr, \
+                                                                nullptr, nullptr, nullptr, 0, nullptr, qb, kb, nullptr); \
     }                                                                                                             \
-    extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void apk_qknorm_rope_##PN##kv_bias_##TN##_hd##HD##_i##ITER( \
+    extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void PFX##_##PN##kv_bias_##TN##_hd##HD##_i##ITER(     \
         T* q, T* k, T* v, const float* qw, const float* kw, const float* rope, const uint32_t* cache_pos,         \
         f16_t* k_cache, f16_t* v_cache, uint32_t capacity, int rows, int n_q, int n_kv, float eps, uint32_t* fault, int rot, \
         const float* qb, const float* kb, const float* vb) {                                                      \
-        qknorm_rope_body<T, HD, ITER, true, PAIRS, true>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x, v, cache_pos, \
-                                                         k_cache, v_cache, capacity, fault, qb, kb, vb);          \
+        qknorm_rope_body<T, HD, ITER, true, PAIRS, true, NORM>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x, v, \
+                                                               cache_pos, k_cache, v_cache, capacity, fault, qb, kb, vb); \
     }
-#define APK_QKROPE_BIAS_ALL(T, TN, ITER)                                                                           \
-    APK_QKROPE_BIAS(T, TN, 64, ITER, false, ) APK_QKROPE_BIAS(T, TN, 128, ITER, false, ) APK_QKROPE_BIAS(T, TN, 256, ITER, false, ) \
-    APK_QKROPE_BIAS(T, TN, 64, ITER, true, pairs_) APK_QKROPE_BIAS(T, TN, 128, ITER, true, pairs_) APK_QKROPE_BIAS(T, TN, 256, ITER, true, pairs_)
-APK_QKROPE_BIAS_ALL(float, f32, 1)
-APK_QKROPE_BIAS_ALL(f16_t, f16, 1)
-APK_QKROPE_BIAS_ALL(f16_t, f16, 2)
-
+#define APK_QK_FAMILY(PFX, NORM, T, TN, HD, ITER)                                                                  \
+    APK_QK_PLAIN(PFX, NORM, T, TN, HD, ITER, false, ) APK_QK_PLAIN(PFX, NORM, T, TN, HD, ITER, true, pairs_)       \
+    APK_QK_KV(PFX, NORM, T, TN, HD, ITER, false, ) APK_QK_KV(PFX, NORM, T, TN, HD, ITER, true, pairs_)             \
+    APK_QK_BIAS(PFX, NORM, T, TN, HD, ITER, false, ) APK_QK_BIAS(PFX, NORM, T, TN, HD, ITER, true, pairs_)
+// two passes per q wave in fp16 only (measured: f32 is fastest with one)
+#define APK_QK_SIZES(PFX, NORM)                                                                                    \
+    APK_QK_FAMILY(PFX, NORM, float, f32, 64, 1) APK_QK_FAMILY(PFX, NORM, float, f32, 128, 1) APK_QK_FAMILY(PFX, NORM, float, f32, 256, 1) \
+    APK_QK_FAMILY(PFX, NORM, f16_t, f16, 64, 1) APK_QK_FAMILY(PFX, NORM, f16_t, f16, 128, 1) APK_QK_FAMILY(PFX, NORM, f16_t, f16, 256, 1) \
+    APK_QK_FAMILY(PFX, NORM, f16_t, f16, 64, 2) APK_QK_FAMILY(PFX, NORM, f16_t, f16, 128, 2) APK_QK_FAMILY(PFX, NORM, f16_t, f16, 256, 2)
+APK_QK_SIZES(apk_qknorm_rope, true)
+APK_QK_SIZES(apk_rope, false)
 // Any other head geometry: head_dim not 64/128/256, a rotary table that covers only the
 // leading rot_half pairs of a head (partial rotary: channels >= 2*rot_half are normalised
 // and pass through, rope.rs:52-81), or the adjacent-pair style (RopeStyle::Norm, pairs

@@ -140,7 +140,7 @@ def test_add_rmsnorm_plans_cover_every_row_once(L, kernels, bounds, post):
     assert fn(1024, 4, F32, None) == 3
 
 
-def plan_attn(L, rows, n_q, n_kv, hd, rot, style, dtype, kv, bias):
+def plan_attn(L, rows, n_q, n_kv, hd, rot, style, dtype, kv, bias, norm=True):
     """The struct form of the same plan: biases and the cache store are asked for by non-NULL pointers."""
     import allpaka_amd.lib as lib
 
@@ -151,21 +151,24 @@ def plan_attn(L, rows, n_q, n_kv, hd, rot, style, dtype, kv, bias):
         a.capacity = 1
     if bias:
         a.q_bias = a.k_bias = 16
+    if norm:
+        a.k_norm = 16
     p = lib.Plan()
     return L.apk_plan_attn_prologue_rows(C.byref(a), C.byref(p)), p
 
 
-@pytest.mark.parametrize("bias", [False, True])
-def test_qknorm_rope_plans_cover_every_head(L, kernels, bounds, bias):
-    """bias: the kernels that add the projection biases on the way."""
+@pytest.mark.parametrize("bias,norm", [(False, True), (True, True), (False, False), (True, False)])
+def test_qknorm_rope_plans_cover_every_head(L, kernels, bounds, bias, norm):
+    """bias: the kernels that add the projection biases on the way; norm = False: no norm weight for q or k, the
+    kernels without statistics."""
     for dtype, es in ((F32, 4), (F16, 2)):
         for hd, rot, style in ((64, 64, 0), (128, 128, 0), (256, 256, 0), (128, 64, 0), (96, 96, 0), (128, 128, 1), (80, 0, 0), (2, 2, 1),
                                (128, 64, 1), (256, 64, 0), (128, 8, 0), (128, 8, 1), (128, 0, 0), (64, 36, 1), (64, 48, 0)):
             for n_q, n_kv in ((64, 8), (32, 8), (16, 8), (40, 8), (28, 4), (8, 1), (1, 0), (0, 3), (12, 2), (96, 8), (5, 5)):
                 for rows in (1, 6, 64, 255, 512, 2048, 2061, 8192, 100000):
                     for kv in (0, 1):
-                        rc, p = plan_attn(L, rows, n_q, n_kv, hd, rot, style, dtype, kv, bias)
-                        if not bias:  # the struct form and the flat form are one plan
+                        rc, p = plan_attn(L, rows, n_q, n_kv, hd, rot, style, dtype, kv, bias, norm)
+                        if not bias and norm:  # the struct form and the flat form are one plan
                             rc2, p2 = plan(L.apk_plan_qknorm_rope, rows, n_q, n_kv, hd, rot, style, dtype, kv)
                             assert (rc2, bytes(p2)) == (rc, bytes(p))
                         epl = 16 // es  # elements of a lane's 16-byte tile
@@ -182,7 +185,7 @@ def test_qknorm_rope_plans_cover_every_head(L, kernels, bounds, bias):
                         if not tiled:
                             assert "generic" in name and waves_launched >= rows * (n_q + n_kv) > waves_launched - 4
                             continue
-                        assert name == (f"apk_qknorm_rope_{'pairs_' if style else ''}{'kv_' if kv else ''}{'bias_' if bias else ''}"
+                        assert name == (f"apk_{'qknorm_rope' if norm else 'rope'}_{'pairs_' if style else ''}{'kv_' if kv else ''}{'bias_' if bias else ''}"
                                         f"{'f32' if dtype == F32 else 'f16'}_hd{hd}_i{p.tiles_per_lane}")
                         lph = hd // 2 // (16 // es)  # lanes per head
                         hpw = 64 // lph
