@@ -116,6 +116,55 @@ def build():
     lg[3, :] = 0.0
     out["argmax.logits"] = lg
     out["argmax.pick"] = np.array([ora.argmax_last(r) for r in lg], np.uint32)
+
+    # (added after the arrays above: the generator's stream up to here, and with it every array above, is unchanged)
+    # GeGLU with the tanh GELU
+    gate, up = s.normal_f32(g, 2003, 0.0, 2.5), s.normal_f32(g, 2003)
+    out["geglu.gate"], out["geglu.up"] = gate, up
+    w = gate.copy()
+    ora.geglu_tanh(w, up)
+    out["geglu.f32"] = w
+    w = f16(gate)
+    ora.geglu_tanh(w, f16(up))
+    out["geglu.f16"] = w
+
+    # sandwich norm + next norm: x += rmsnorm(delta) * post_gamma; h = rmsnorm(x) * gamma
+    x, d = s.normal_f32(g, (3, 2304)), s.normal_f32(g, (3, 2304), 0.0, 3.0)
+    pg, gamma = s.normal_f32(g, 2304, 1.0, 0.05), s.normal_f32(g, 2304, 1.0, 0.05)
+    out["postnorm.x"], out["postnorm.d"], out["postnorm.pg"], out["postnorm.gamma"] = x, d, pg, gamma
+    for tag, xx, dd in (("f32", x, d), ("f16", f16(x), f16(d))):
+        nd = np.zeros_like(dd)
+        ora.add_rmsnorm_rows(dd.copy(), None, nd, pg, 1e-6)
+        wx, wh = xx.copy(), np.zeros_like(xx)
+        ora.add_rmsnorm_rows(wx, nd, wh, gamma, 1e-6)
+        out[f"postnorm.{tag}.x"], out[f"postnorm.{tag}.h"] = wx, wh
+
+    # q/k/v biases, no QK-norm, NeoX rotation, K/V cache store (28 + 4 heads of 128, three rows)
+    rows, nq, nkv, hd = 3, 28, 4, 128
+    q, k, v = s.normal_f32(g, (rows, nq * hd)), s.normal_f32(g, (rows, nkv * hd)), s.normal_f32(g, (rows, nkv * hd))
+    qb, kb, vb = s.normal_f32(g, nq * hd, 0.0, 0.5), s.normal_f32(g, nkv * hd, 0.0, 0.5), s.normal_f32(g, nkv * hd, 0.0, 0.5)
+    pos = np.array([5, 0, 9], np.uint32)
+    ropes = ora.rope_table([int(p) for p in pos], ora.rope_inv_freq(hd, 1e6))
+    out["bias.q"], out["bias.k"], out["bias.v"], out["bias.qb"], out["bias.kb"], out["bias.vb"] = q, k, v, qb, kb, vb
+    out["bias.pos"], out["bias.ropes"] = pos, ropes
+    for tag, conv, back in (("f32", lambda a: a.copy(), lambda a: a), ("f16", f16, None)):
+        wq, wk = conv(q), conv(k)
+        ora.qknorm_rope_rows(wq, wk, nq, nkv, hd, None, None, ropes, 1e-6, q_bias=qb, k_bias=kb)
+        if tag == "f32":
+            wv = v.copy()
+            ora.add_bias_rows(wv, vb)
+        else:
+            wv = ora.f16_bits_to_f32(f16(v))
+            ora.add_bias_rows(wv, vb)
+            wv = ora.f32_to_f16_bits(wv)
+        kc, vc = np.zeros((12, nkv * hd), np.uint16), np.zeros((12, nkv * hd), np.uint16)
+        ora.kv_store_rows(wk, wv, pos, kc, vc)
+        out[f"bias.{tag}.q"], out[f"bias.{tag}.k"], out[f"bias.{tag}.v"] = wq, wk, wv
+        out[f"bias.{tag}.kc"], out[f"bias.{tag}.vc"] = kc, vc
+
+    # the shared expert's hit in the lists of the grouping above
+    to, hr, hw = ora.moe_shared_hits(tok_off, hit_row, hit_w, 40 * 8)
+    out["moe.shared.tok_off"], out["moe.shared.hit_row"], out["moe.shared.hit_w"] = to, hr, hw
     return out
 
 

@@ -27,7 +27,7 @@ def same(a, b):
 
 # ----------------------------------------------------------------------- CPU
 def test_fixture_file_is_complete(gold):
-    assert len(gold) == 123
+    assert len(gold) == 156
     for name in FORMATS:
         assert f"embed.{name}.f16" in gold
     assert gold["moe.ids"].shape == (40, 8) and gold["argmax.pick"].shape == (5,)
@@ -66,6 +66,22 @@ def test_oracle_reproduces_the_frozen_outputs(gold, ora):
     assert same(wx, g["moe.combine.x"]) and same(wh, g["moe.combine.h"])
     assert same(np.array([ora.argmax_last(r) for r in g["argmax.logits"]], np.uint32), g["argmax.pick"])
     assert list(g["argmax.pick"][[1, 3]]) == [500, 599]  # ties: the last maximum
+    w = g["geglu.gate"].copy()
+    ora.geglu_tanh(w, g["geglu.up"])
+    assert same(w, g["geglu.f32"])
+    f16 = lambda a: a.astype(np.float16).view(np.uint16)  # noqa: E731
+    for tag, conv in (("f32", lambda a: a.copy()), ("f16", f16)):
+        xx, dd = conv(g["postnorm.x"]), conv(g["postnorm.d"])
+        nd = np.zeros_like(dd)
+        ora.add_rmsnorm_rows(dd.copy(), None, nd, g["postnorm.pg"], 1e-6)
+        wx, wh = xx.copy(), np.zeros_like(xx)
+        ora.add_rmsnorm_rows(wx, nd, wh, g["postnorm.gamma"], 1e-6)
+        assert same(wx, g[f"postnorm.{tag}.x"]) and same(wh, g[f"postnorm.{tag}.h"]), tag
+        wq, wk = conv(g["bias.q"]), conv(g["bias.k"])
+        ora.qknorm_rope_rows(wq, wk, 28, 4, 128, None, None, g["bias.ropes"], 1e-6, q_bias=g["bias.qb"], k_bias=g["bias.kb"])
+        assert same(wq, g[f"bias.{tag}.q"]) and same(wk, g[f"bias.{tag}.k"]), tag
+    to, hr, hw = ora.moe_shared_hits(g["moe.tok_off"], g["moe.hit_row"], g["moe.hit_w"], 320)
+    assert same(to, g["moe.shared.tok_off"]) and same(hr, g["moe.shared.hit_row"]) and same(hw, g["moe.shared.hit_w"])
 
 
 # ----------------------------------------------------------------------- GPU
@@ -165,3 +181,35 @@ def test_device_moe_chain_and_argmax_match_the_frozen_outputs(gold, be):
     assert same(host(tx), g["moe.combine.x"])
     assert rel_err_f32(host(th), g["moe.combine.h"]) <= 1e-5
     assert same(host(be.argmax_rows(dev(g["argmax.logits"]))), g["argmax.pick"])
+
+
+@pytest.mark.gpu
+def test_device_gemma_and_bias_steps_match_the_frozen_outputs(gold, be):
+    g = gold
+    f16 = lambda a: a.astype(np.float16).view(np.uint16)  # noqa: E731
+    tg = dev(g["geglu.gate"])
+    be.geglu_tanh(tg, dev(g["geglu.up"]))
+    assert close_idiom(host(tg), g["geglu.f32"])
+    for tag, conv in (("f32", lambda a: a), ("f16", f16)):
+        tx, th = dev(conv(g["postnorm.x"])), torch.zeros_like(dev(conv(g["postnorm.x"])))
+        be.postnorm_add_rmsnorm_rows(tx, dev(conv(g["postnorm.d"])), dev(g["postnorm.pg"]), th, dev(g["postnorm.gamma"]), 1e-6)
+        if tag == "f16":
+            assert same(host(tx), g["postnorm.f16.x"])
+            assert f16_ulp_diff(host(th), g["postnorm.f16.h"]) <= 2
+        else:
+            for got, key in ((tx, "postnorm.f32.x"), (th, "postnorm.f32.h")):
+                assert rel_err_f32(host(got), g[key]) <= 1e-5 and close_idiom(host(got), g[key]), key
+        tq, tk, tv = dev(conv(g["bias.q"])), dev(conv(g["bias.k"])), dev(conv(g["bias.v"]))
+        kc = torch.zeros((12, 4 * 128), dtype=torch.float16, device="cuda")
+        vc = torch.zeros_like(kc)
+        be.attn_prologue_rows(tq, tk, tv, 28, 4, 128, 1e-6, dev(g["bias.ropes"]), q_bias=dev(g["bias.qb"]), k_bias=dev(g["bias.kb"]),
+                              v_bias=dev(g["bias.vb"]), cache_pos=dev(g["bias.pos"]), k_cache=kc, v_cache=vc)
+        if tag == "f32":  # one add, then the reference's four products and two sums: bit for bit
+            assert same(host(tq), g["bias.f32.q"]) and same(host(tk), g["bias.f32.k"])
+        else:
+            assert f16_ulp_diff(host(tq), g["bias.f16.q"]) <= 2 and f16_ulp_diff(host(tk), g["bias.f16.k"]) <= 2
+        assert same(host(tv), g[f"bias.{tag}.v"]) and same(host(vc), g[f"bias.{tag}.vc"])
+        assert f16_ulp_diff(host(kc), g[f"bias.{tag}.kc"]) <= (2 if tag == "f16" else 1)
+    got = be.moe_shared_hits(dev(g["moe.tok_off"]), dev(g["moe.hit_row"]), dev(g["moe.hit_w"]), 320)
+    for a, name in zip(got, ["tok_off", "hit_row", "hit_w"]):
+        assert same(host(a), g[f"moe.shared.{name}"]), name
