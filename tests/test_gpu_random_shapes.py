@@ -7,6 +7,8 @@ beaten path (a last partial tile, a workgroup tail, a wave that owns no head) is
 too.  Same bars: bit-exact for integer / byte / index work and pure data movement,
 1e-5 relative for f32, 2 ulp for fp16.
 """
+import os
+
 import numpy as np
 import pytest
 
@@ -18,7 +20,7 @@ torch = pytest.importorskip("torch")
 
 TOL_F32 = 1e-5
 TOL_F16_ULP = 2
-CASES = 24
+CASES = int(os.environ.get("APK_RANDOM_CASES", "24"))  # more cases for an occasional wider run
 
 
 @pytest.fixture(scope="module")
