@@ -790,13 +790,14 @@ int apk_add_assign(apk_ctx* c, void* a, const void* b, size_t n, int dtype) {
     if (!aligned16(a) || !aligned16(b)) return fail(APK_DECLINE_SHAPE, "apk_add_assign: tensors must be 16-byte aligned");
     if (int rc = set_device(c)) return rc;
     const uint64_t nvec = n / (16 / es);
-    uint64_t grid = (nvec + 255) / 256;
+    const unsigned block = stream_block(nvec);
+    uint64_t grid = (nvec + block - 1) / block;
     if (grid == 0) grid = 1;
     if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_add_assign: n too large");
     uint64_t n64 = n;
     void* args[] = {&a, &b, &n64};
     return launch_keyed(c, OP_ADD_ASSIGN, (uint32_t)dtype,
-                        [&] { return std::string(dtype == APK_F32 ? "apk_add_assign_f32" : "apk_add_assign_f16"); }, (unsigned)grid, 256, 0, args);
+                        [&] { return std::string(dtype == APK_F32 ? "apk_add_assign_f32" : "apk_add_assign_f16"); }, (unsigned)grid, block, 0, args);
 }
 
 int apk_cast(apk_ctx* c, const void* src, int src_dtype, void* dst, int dst_dtype, size_t n) {
@@ -1458,10 +1459,11 @@ int apk_copy(apk_ctx* c, const void* src, void* dst, size_t bytes) {
     if (bytes % 16 || !aligned16(src) || !aligned16(dst)) return fail(APK_DECLINE_SHAPE, "apk_copy: whole 16-byte tiles only");
     if (int rc = set_device(c)) return rc;
     uint64_t nvec = bytes / 16;
-    const uint64_t grid = (nvec + 255) / 256;
+    const unsigned block = stream_block(nvec);
+    const uint64_t grid = (nvec + block - 1) / block;
     if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_copy: too large");
     void* args[] = {&src, &dst, &nvec};
-    return launch(c, "apk_copy", (unsigned)grid, 256, 0, args);
+    return launch(c, "apk_copy", (unsigned)grid, block, 0, args);
 }
 
 }  // extern "C"

@@ -31,7 +31,7 @@ COLD_BYTES = 640e6  # every op rotates through at least this many distinct bytes
 
 # FETCH_SIZE / WRITE_SIZE of the dominant kernel (rocprofv3 --pmc, KiB per dispatch,
 # scaled by the same counters on apk_copy of a known size); see profiles/.
-TRAFFIC_BYTES_PER_LAUNCH = 314481433
+TRAFFIC_BYTES_PER_LAUNCH = 314546888
 
 
 def main():
