@@ -809,12 +809,13 @@ int apk_cast(apk_ctx* c, const void* src, int src_dtype, void* dst, int dst_dtyp
     if (!src || !dst) return fail(APK_DECLINE_NULL, "apk_cast: NULL tensor");
     if (!aligned16(src) || !aligned16(dst)) return fail(APK_DECLINE_SHAPE, "apk_cast: tensors must be 16-byte aligned");
     if (int rc = set_device(c)) return rc;
-    uint64_t grid = (n / 8 + 255) / 256;
+    const unsigned block = stream_block(n / 8);
+    uint64_t grid = (n / 4 + 2 * block - 1) / (2 * block);  // four elements per lane and step, two steps
     if (grid == 0) grid = 1;
     if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_cast: n too large");
     uint64_t n64 = n;
     void* args[] = {&src, &dst, &n64};
-    return launch(c, src_dtype == APK_F32 ? "apk_cast_f32_f16" : "apk_cast_f16_f32", (unsigned)grid, 256, 0, args);
+    return launch(c, src_dtype == APK_F32 ? "apk_cast_f32_f16" : "apk_cast_f16_f32", (unsigned)grid, block, 0, args);
 }
 
 int apk_softmax_rows(apk_ctx* c, float* x, size_t rows, size_t n) {
@@ -1007,12 +1008,13 @@ static int add_bias_rows_locked(apk_ctx* c, void* x, const float* bias, size_t r
     if (int rc = set_device(c)) return rc;
     const size_t vec = 16 / es;
     const uint64_t lanes = n % vec == 0 ? (uint64_t)rows * (n / vec) : (uint64_t)rows * n;
-    const uint64_t grid = (lanes + 255) / 256;
+    const unsigned block = stream_block(lanes);
+    const uint64_t grid = (lanes + block - 1) / block;
     if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_add_bias_rows: too large");
     uint64_t rows64 = rows;
     uint32_t n32 = (uint32_t)n;
     void* args[] = {&x, &bias, &rows64, &n32};
-    return launch(c, dtype == APK_F32 ? "apk_add_bias_rows_f32" : "apk_add_bias_rows_f16", (unsigned)grid, 256, 0, args);
+    return launch(c, dtype == APK_F32 ? "apk_add_bias_rows_f32" : "apk_add_bias_rows_f16", (unsigned)grid, block, 0, args);
 }
 
 int apk_add_bias_rows(apk_ctx* c, void* x, const float* bias, size_t rows, size_t n, int dtype) {
