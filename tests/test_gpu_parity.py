@@ -1238,6 +1238,51 @@ def test_permute_declines_and_faults(be):
     assert be.take_faults() & 4 and np.all(host(out)[[0, 1, 3]] == 1.0)
 
 
+def test_family_step_entries_decline_and_leave_their_tensors_alone(be):
+    """NULL arguments, unsupported types, misaligned tensors and impossible geometry are declined (a positive status
+    with a message) by the entries of the Gemma / Qwen2 / GLM steps, before anything is launched."""
+    import ctypes as C
+
+    import allpaka_amd.lib as lib
+
+    L, h = be.L, be.h
+    t = torch.ones(1024, device="cuda")
+    before = t.clone()
+    ptr = t.data_ptr()
+
+    def declined(rc, code):
+        assert rc == code, (rc, L.apk_last_error())
+        assert L.apk_last_error()  # a message is left for the caller
+
+    declined(L.apk_cast(h, ptr, 0, ptr + 2048, 7, 16), 1)            # unknown type
+    declined(L.apk_cast(h, None, 0, ptr, 1, 16), 3)                  # NULL
+    declined(L.apk_cast(h, ptr + 4, 0, ptr + 2048, 1, 16), 2)        # misaligned
+    declined(L.apk_add_bias_rows(h, ptr, None, 2, 64, 0), 3)
+    declined(L.apk_add_bias_rows(h, ptr, ptr + 2048, 2, 64, 5), 1)
+    declined(L.apk_add_bias_rows(h, ptr + 4, ptr + 2048, 2, 64, 0), 2)
+    assert L.apk_add_bias_rows(h, None, None, 0, 64, 0) == 0          # no rows: nothing to do
+    declined(L.apk_postnorm_add_rmsnorm_rows(h, ptr, ptr, ptr + 2048, ptr + 1024, ptr + 2048, 64, 2, 1e-6, 0), 2)  # x aliases delta
+    declined(L.apk_postnorm_add_rmsnorm_rows(h, ptr, ptr + 512, None, ptr + 1024, ptr + 2048, 64, 2, 1e-6, 0), 3)
+    declined(L.apk_moe_shared_hits(h, None, ptr, ptr, 2, 4, ptr + 1024, ptr + 2048, ptr + 3072), 3)
+    declined(L.apk_attn_prologue_rows(h, None), 3)
+    a = lib.AttnPrologue()
+    a.q, a.k, a.rope = ptr, ptr + 2048, ptr
+    a.rows, a.n_q, a.n_kv, a.head_dim, a.rot_dim, a.eps, a.dtype = 1, 2, 1, 128, 128, 1e-6, 0
+    a.q_bias = ptr + 4                                                # misaligned bias
+    declined(L.apk_attn_prologue_rows(h, C.byref(a)), 2)
+    a.q_bias = None
+    a.rot_dim = 130                                                   # wider than the head
+    declined(L.apk_attn_prologue_rows(h, C.byref(a)), 2)
+    a.rot_dim, a.dtype = 128, 9
+    declined(L.apk_attn_prologue_rows(h, C.byref(a)), 1)
+    a.dtype, a.k_cache = 0, ptr                                       # a cache store without v / positions
+    declined(L.apk_attn_prologue_rows(h, C.byref(a)), 3)
+    a.k_cache, a.head_dim, a.rot_dim, a.v_bias = None, 96, 96, ptr    # v_bias without v (and no store)
+    declined(L.apk_attn_prologue_rows(h, C.byref(a)), 3)
+    be.sync()
+    assert torch.equal(t, before)
+
+
 @pytest.mark.parametrize("rows,k,cols,f16", [(600, 8, 3600, False), (600, 8, 3600, True), (3, 2, 8200, False), (4099, 1, 520, True),
                                              (9, 64, 4, False)])
 def test_scatter_rows_is_the_permutation(be, rows, k, cols, f16):
