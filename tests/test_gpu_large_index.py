@@ -48,6 +48,33 @@ def test_streams_past_four_gigabytes(be, ora):
     for (a, m), (g0, u0) in zip(windows, before):
         want = ora.f32_to_f16_bits(ora.f16_bits_to_f32(g0) + ora.f16_bits_to_f32(u0))
         assert np.array_equal(bits(gate[a:a + m]), want), a
+    # GeGLU over the same tensors
+    before = [(bits(gate[a:a + m]).copy(), bits(up[a:a + m]).copy()) for a, m in windows]
+    be.geglu_tanh(gate, up)
+    for (a, m), (g0, u0) in zip(windows, before):
+        want = g0.copy()
+        ora.geglu_tanh(want, u0)
+        ok = (np.abs(ora.f16_bits_to_f32(bits(gate[a:a + m])) - ora.f16_bits_to_f32(want)) <= 1e-3 * (1 + np.abs(ora.f16_bits_to_f32(want))))
+        assert ok.all(), a
+    # a per-row bias over rows of 16 384 (131 080 rows: past 2^32 bytes), in place, bit for bit
+    width = 16384
+    nrows = n // width
+    bias = torch.randn(width, generator=gen, device="cuda")
+    before = [bits(gate[a:a + m]).copy() for a, m in windows[:3]]
+    be.add_bias_rows(gate[: nrows * width], bias)
+    hb = bias.cpu().numpy()
+    for (a, m), g0 in zip(windows[:3], before):
+        w = ora.f16_bits_to_f32(g0)
+        w += hb[(np.arange(a, a + m)) % width]
+        assert np.array_equal(bits(gate[a:a + m]), ora.f32_to_f16_bits(w)), a
+    # fp16 -> f32 of the first 2^30 + 2^20 elements (a 4 GiB + 4 MiB result) and back
+    m32 = (1 << 30) + (1 << 20)
+    wide = be.cast(up[:m32], torch.float32)
+    for a in (0, (1 << 29) - 2048, (1 << 30) - 2048, m32 - 4096):
+        assert np.array_equal(wide[a:a + 4096].cpu().numpy().view(np.uint32), ora.f16_bits_to_f32(bits(up[a:a + 4096])).view(np.uint32)), a
+    back = be.cast(wide, torch.float16)
+    assert torch.equal(back, up[:m32])
+    del wide, back
     # rows x n beyond 2^32 bytes: residual add + RMSNorm over 131 080 rows of 16 384 (the same memory, reshaped)
     rows, width = 131080, 16384
     x = gate[: rows * width].view(rows, width)
