@@ -387,3 +387,54 @@ def test_recorded_router_and_grouping_follow_the_logits_of_every_replay(be, ora)
         for name, a, b in zip(["table", "tok", "tok_off", "hit_row", "hit_w"], outs, want):
             assert np.array_equal(host(a)[: b.shape[0]].view(np.uint32), b.view(np.uint32)), (step, name)
     rec.graph.destroy()
+
+
+def test_recorded_family_steps_replay_on_the_data_of_the_day(be, ora):
+    """The q/k/v step with biases and the cache store, the sandwich norm and GeGLU inside one recording (three nodes,
+    four with the separate v-bias launch of the storeless form): every replay works on what is in the buffers then,
+    and equals the unrecorded calls bit for bit."""
+    from allpaka_amd import synth as s
+
+    rows, n_q, n_kv, hd, n = 5, 12, 2, 128, 2304
+    g = s.rng(6, 1)
+    qb, kb, vb = (dev(s.normal_f32(g, m * hd, 0.0, 0.5)) for m in (n_q, n_kv, n_kv))
+    pg, gamma = dev(s.normal_f32(g, n, 1.0, 0.05)), dev(s.normal_f32(g, n, 1.0, 0.05))
+    pos = torch.tensor([3, 0, 7, 1, 5], dtype=torch.int32, device="cuda")
+    ropes = dev(ora.rope_table([3, 0, 7, 1, 5], ora.rope_inv_freq(hd, 1e6)))
+    f16 = torch.float16
+    q, k, v = (torch.zeros((rows, m * hd), dtype=f16, device="cuda") for m in (n_q, n_kv, n_kv))
+    x, d, h = (torch.zeros((rows, n), dtype=f16, device="cuda") for _ in range(3))
+    gate, up = torch.zeros(4000, dtype=f16, device="cuda"), torch.zeros(4000, dtype=f16, device="cuda")
+    kc = torch.zeros((8, n_kv * hd), dtype=f16, device="cuda")
+    vc = torch.zeros_like(kc)
+
+    def step():
+        be.attn_prologue_rows(q, k, v, n_q, n_kv, hd, 1e-6, ropes, q_bias=qb, k_bias=kb, v_bias=vb, cache_pos=pos, k_cache=kc, v_cache=vc)
+        be.postnorm_add_rmsnorm_rows(x, d, pg, h, gamma, 1e-6)
+        be.geglu_tanh(gate, up)
+
+    with be.record() as rec:
+        step()
+    assert rec.graph.nodes == 3
+    bufs = (q, k, v, x, d, gate, up)
+    for it in range(3):
+        gen = torch.Generator(device="cuda").manual_seed(50 + it)
+        fresh = [torch.randn(b.shape, generator=gen, device="cuda").to(f16) for b in bufs]
+        for b, f in zip(bufs, fresh):
+            b.copy_(f)
+        for t in (kc, vc, h):
+            t.zero_()
+        be.swiglu(torch.ones(64, device="cuda"), torch.ones(64, device="cuda"))  # unrecorded work in between
+        rec.graph.launch()
+        be.sync()
+        got = [t.clone() for t in (q, k, v, x, h, gate, kc, vc)]
+        for b, f in zip(bufs, fresh):
+            b.copy_(f)
+        for t in (kc, vc, h):
+            t.zero_()
+        step()
+        be.sync()
+        for name, a, b in zip("q k v x h gate kc vc".split(), got, (q, k, v, x, h, gate, kc, vc)):
+            assert torch.equal(a, b), (it, name)
+        assert be.take_faults() == 0
+    rec.graph.destroy()
