@@ -59,7 +59,7 @@ struct Mapping {
 // missing symbol fails there and not at the first launch.
 const int kAddnormTiles[] = {1, 2, 3, 4, 5, 6, 8, 10, 12, 16, 20};  // 16-byte tiles per lane
 const int kAddnormBound[] = {1024, 1024, 512, 512, 256, 256, 256, 256, 256, 256, 256};  // launch bound of each
-const int kQkIters[] = {1, 2};
+const int kQkIters[] = {1};
 const int kQkHeadDims[] = {64, 128, 256};
 
 std::vector<std::string> all_kernel_names() {
@@ -82,8 +82,7 @@ std::vector<std::string> all_kernel_names() {
                     for (const char* style : {"", "pairs_"})
                         for (const char* kv : {"", "kv_"})
                             for (const char* bias : {"", "bias_"})
-                                if (it == 1 || t[1] == '1')  // two passes per q wave exist in fp16 only
-                                    v.push_back(std::string(pfx) + style + kv + bias + t + "_hd" + std::to_string(hd) + "_i" + std::to_string(it));
+                                v.push_back(std::string(pfx) + style + kv + bias + t + "_hd" + std::to_string(hd) + "_i" + std::to_string(it));
     }
     return v;
 }
@@ -239,19 +238,18 @@ int plan_qknorm_rope(size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size
         p->rows_per_block = 4;
         return APK_OK;
     }
-    // A wave owns (row, q or k, group of HPW*ITER heads), HPW = heads per wave pass; k waves
-    // take one pass.  Measured over 1024..8192 rows: fp16 is fastest with two passes per q wave
-    // (16 heads, 4 KB), f32 with one (4 heads, 2 KB); more passes per wave gain nothing where
-    // the batch happens to be a whole number of resident rounds and lose up to 15 % elsewhere.
-    // Small batches (under 6 waves per CU) take one pass: more waves.
+    // A wave owns (row, q or k, group of HPW heads), HPW = heads per wave pass: one pass per wave.  Measured over
+    // 1024..8192 rows: longer waves (two or four passes) hold more registers per resident byte and lose 2-8 % once
+    // the arithmetic of a pass shows next to the stream; short waves also fill in evenly when a batch is not a whole
+    // number of resident rounds.  fp16 kernels keep their constants in LDS and run as workgroups of two waves
+    // (8 resident waves per SIMD); f32 kernels keep them in registers, four waves to a workgroup.
     const size_t epl = 16 / es, lph = head_dim / 2 / epl, hpw = 64 / lph;
     const size_t gk = (n_kv + hpw - 1) / hpw;
-    unsigned iter = 1;
-    if (dtype == APK_F16 && n_q > hpw && rows * ((n_q + 2 * hpw - 1) / (2 * hpw) + gk) >= 1536) iter = 2;
+    const unsigned iter = 1;
     const uint64_t waves = (uint64_t)rows * ((n_q + hpw * iter - 1) / (hpw * iter) + gk);
-    const unsigned block = 256;  // (64 and 128 measure the same: the waves of a workgroup share nothing)
+    const unsigned block = dtype == APK_F16 ? 128 : 256;
     const uint64_t grid = (waves * 64 + block - 1) / block;
-    if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope: too large");
+    if (grid > 0x7fffffffu || waves > 0xffffffffu) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope: too large");  // the kernels index waves in 32 bits
     p->variant = QK_TILED;
     plan_name(p, std::string(with_norm ? "apk_qknorm_rope_" : "apk_rope_") + (style ? "pairs_" : "") + (with_kv ? "kv_" : "") + (with_bias ? "bias_" : "") + t + "_hd" +
                      std::to_string(head_dim) + "_i" + std::to_string(iter));

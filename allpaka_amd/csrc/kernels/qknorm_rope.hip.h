@@ -38,19 +38,47 @@
 // as well as narrowed into the cache.
 // NORM = false: neither tensor has a norm weight (the Llama / Qwen2 families: biases or not, then the rotation):
 // no statistics, no weight tiles -- the launch then runs at the speed of a plain copy of the same bytes.
-template <typename T, int HD, int ITER, bool KV = false, bool PAIRS = false, bool BIAS = false, bool NORM = true>
+// The per-head statistics of this op, for both activation types: the reference's own operations
+// (norm.rs:115-187) -- the sum of squares in f64, scale = 1/sqrt(mean + eps) in f64, (x as f64 * scale) as f32 -- so
+// that an fp16 result is the reference's f32 result rounded once (a rotated output a*cos - b*sin can nearly cancel,
+// and an f32-level difference in the normalised inputs is then many ulps of the fp16 result).  f32 rows take the
+// IEEE square root and division; fp16 rows take two f64 Newton steps from the hardware rsq (1e-16 of
+// sqrt-then-divide, a third of the instructions), which no fp16 result can show.
+template <typename T> struct rotstat : stat<float> {};
+template <> struct rotstat<f16_t> : stat<float> {
+    DEV double rscale(double ss, int n, float eps) {
+        const double v = ss / (double)n + (double)eps;  // n a power of two known at compile time: a multiplication
+        double y = (double)__builtin_amdgcn_rsqf((float)v);
+        y = y * __builtin_fma(-0.5 * v, y * y, 1.5);
+        return y * __builtin_fma(-0.5 * v, y * y, 1.5);
+    }
+};
+
+// LDSC = true: the wave copies the row's [sin, cos] entries (rot floats) and its tensor's norm weight (HD floats)
+// into 2*HD floats of LDS of its own (lmem) and reads the lane's entries back pass by pass, right where they are
+// used, instead of holding them in 2-4 registers per element from the first load on.  With fp16 tiles that is the
+// difference between 84 and 63 registers, i.e. between 5 and 8 resident waves per SIMD, and this kernel's speed
+// follows its resident waves (the arithmetic of a pass is not free next to the stream).  Nothing is shared between
+// waves: no barrier, only the wave's own LDS counter.
+template <typename T, int HD, int ITER, bool KV = false, bool PAIRS = false, bool BIAS = false, bool NORM = true, bool LDSC = false, bool FULL = false>
 DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, float eps, int l, int sub, int rot,
                  f16_t* kc = nullptr, const T* vrow = nullptr, f16_t* vc = nullptr, const float* bias = nullptr,
-                 const float* vbias = nullptr, T* vout = nullptr) {
+                 const float* vbias = nullptr, T* vout = nullptr, float* lmem = nullptr) {
     constexpr int EPL = io<T>::VEC;   // elements per lane per half
     constexpr int HALF = HD / 2;
     constexpr int LPH = HALF / EPL;   // lanes per head
     constexpr int HPW = 64 / LPH;     // heads per wave pass
-    typedef typename headstat<T>::acc_t acc_t;
     // the lane's two tiles inside a head, whether each rotates, and where its [sin, cos] floats start
     int off_a, off_b, sc_a, sc_b;
     bool rot_a, rot_b;
-    if constexpr (PAIRS) {
+    if constexpr (FULL) {  // rot == HD, known at compile time: every tile rotates, no selects below
+        rot_a = rot_b = true;
+        off_a = EPL * l;
+        off_b = HALF + EPL * l;
+        sc_a = PAIRS ? off_a : 2 * EPL * l;
+        sc_b = PAIRS ? off_b : sc_a + EPL;
+        rot = HD;
+    } else if constexpr (PAIRS) {
         off_a = EPL * l;
         off_b = HALF + EPL * l;
         rot_a = off_a < rot;
@@ -67,21 +95,30 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
     }
     // Loads return in issue order, so the small cached ones go first and the first pass
     // can start as soon as its own two tiles arrive.  No branch, no conversion here: a
-    // lane of a pass beyond the last head re-reads the last head and stores nothing; a
-    // missing norm weight is read from the [sin, cos] tile instead and never used.
+    // lane of a pass beyond the last head re-reads the last head and stores nothing.
     float sc[2 * EPL], wa[EPL], wb[EPL];
+    constexpr int NST = (HD + 127) / 128;  // 8-byte pieces per lane of a staged array
+    f32x2 st_sc[LDSC ? NST : 1], st_w[LDSC ? NST : 1];
+    if constexpr (LDSC) {
+        const int lane = sub * LPH + l;
 #pragma unroll
-    for (int i = 0; i < EPL; i += 4) {  // a tile that does not rotate reads the row's first entries and ignores them
-        io<float>::load(trow + sc_a + i, sc + i);
-        io<float>::load(trow + sc_b + i, sc + EPL + i);
-    }
-    if constexpr (NORM) {
-        const float* wp = w ? w : trow;
-        const int w_a = w ? off_a : 0, w_b = w ? off_b : 0;
+        for (int j = 0; j < NST; j++) {  // a piece past the end re-reads the last one and is not written
+            const int i = 2 * lane + 128 * j;
+            st_sc[j] = *(const f32x2*)(trow + min(i, rot - 2));
+            if constexpr (NORM) st_w[j] = *(const f32x2*)(w + min(i, HD - 2));
+        }
+    } else {
 #pragma unroll
-        for (int i = 0; i < EPL; i += 4) {
-            io<float>::load(wp + w_a + i, wa + i);
-            io<float>::load(wp + w_b + i, wb + i);
+        for (int i = 0; i < EPL; i += 4) {  // a tile that does not rotate reads the row's first entries and ignores them
+            io<float>::load(trow + sc_a + i, sc + i);
+            io<float>::load(trow + sc_b + i, sc + EPL + i);
+        }
+        if constexpr (NORM) {
+#pragma unroll
+            for (int i = 0; i < EPL; i += 4) {
+                io<float>::load(w + off_a + i, wa + i);
+                io<float>::load(w + off_b + i, wb + i);
+            }
         }
     }
     typename io<T>::raw_t araw[ITER], braw[ITER], varaw[ITER], vbraw[ITER];
@@ -120,7 +157,18 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
         }
     }
     __builtin_amdgcn_sched_barrier(0);  // every load above; all uses below
-    const bool normed = NORM && w != nullptr;  // uniform for the wave
+    if constexpr (LDSC) {
+        const int lane = sub * LPH + l;
+#pragma unroll
+        for (int j = 0; j < NST; j++) {
+            const int i = 2 * lane + 128 * j;
+            if (i < rot) *(f32x2*)(lmem + i) = st_sc[j];
+            if constexpr (NORM) {
+                if (i < HD) *(f32x2*)(lmem + HD + i) = st_w[j];
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
 #pragma unroll
     for (int it = 0; it < ITER; it++) {
         float a[EPL], b[EPL], oa[EPL], ob[EPL];
@@ -135,51 +183,65 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
                 }
             }
         }
-        typename headstat<T>::scale_t scale{};
+        double scale = 0;
         if constexpr (NORM) {
-            acc_t ss = 0;
+            double ss = 0;
 #pragma unroll
             for (int i = 0; i < EPL; i++) {
-                ss = headstat<T>::sq(ss, a[i]);
-                ss = headstat<T>::sq(ss, b[i]);
+                ss = rotstat<T>::sq(ss, a[i]);
+                ss = rotstat<T>::sq(ss, b[i]);
             }
             ss = group_sum<LPH>(ss);
-            scale = headstat<T>::rscale(ss, HD, eps);
+            scale = rotstat<T>::rscale(ss, HD, eps);
+        }
+        if constexpr (LDSC) {  // the lane's entries, back from the wave's LDS (a tile that does not rotate reads the first entries)
+#pragma unroll
+            for (int i = 0; i < EPL; i += 4) {
+                io<float>::load(lmem + sc_a + i, sc + i);
+                io<float>::load(lmem + sc_b + i, sc + EPL + i);
+            }
+            if constexpr (NORM) {
+#pragma unroll
+                for (int i = 0; i < EPL; i += 4) {
+                    io<float>::load(lmem + HD + off_a + i, wa + i);
+                    io<float>::load(lmem + HD + off_b + i, wb + i);
+                }
+            }
         }
         if constexpr (PAIRS) {
 #pragma unroll
             for (int i = 0; i < EPL; i++) {
-                if (normed) {
-                    a[i] = headstat<T>::apply(a[i], scale, wa[i]);
-                    b[i] = headstat<T>::apply(b[i], scale, wb[i]);
+                if constexpr (NORM) {
+                    a[i] = rotstat<T>::apply(a[i], scale, wa[i]);
+                    b[i] = rotstat<T>::apply(b[i], scale, wb[i]);
                 }
             }
 #pragma unroll
             for (int m = 0; m < EPL / 2; m++) {  // sc[0 .. EPL): the pairs of tile a, sc[EPL .. 2 EPL): of tile b
                 const float sa = sc[2 * m], ca = sc[2 * m + 1], sb = sc[EPL + 2 * m], cb = sc[EPL + 2 * m + 1];
-                oa[2 * m] = rot_a ? a[2 * m] * ca - a[2 * m + 1] * sa : a[2 * m];
-                oa[2 * m + 1] = rot_a ? a[2 * m] * sa + a[2 * m + 1] * ca : a[2 * m + 1];
-                ob[2 * m] = rot_b ? b[2 * m] * cb - b[2 * m + 1] * sb : b[2 * m];
-                ob[2 * m + 1] = rot_b ? b[2 * m] * sb + b[2 * m + 1] * cb : b[2 * m + 1];
+                oa[2 * m] = FULL || rot_a ? a[2 * m] * ca - a[2 * m + 1] * sa : a[2 * m];
+                oa[2 * m + 1] = FULL || rot_a ? a[2 * m] * sa + a[2 * m + 1] * ca : a[2 * m + 1];
+                ob[2 * m] = FULL || rot_b ? b[2 * m] * cb - b[2 * m + 1] * sb : b[2 * m];
+                ob[2 * m + 1] = FULL || rot_b ? b[2 * m] * sb + b[2 * m + 1] * cb : b[2 * m + 1];
             }
         } else {
 #pragma unroll
             for (int i = 0; i < EPL; i++) {
                 float x = a[i], y = b[i];
-                if (normed) {
-                    x = headstat<T>::apply(x, scale, wa[i]);
-                    y = headstat<T>::apply(y, scale, wb[i]);
+                if constexpr (NORM) {
+                    x = rotstat<T>::apply(x, scale, wa[i]);
+                    y = rotstat<T>::apply(y, scale, wb[i]);
                 }
                 const float s = sc[2 * i], c = sc[2 * i + 1];
-                oa[i] = rot_a ? x * c - y * s : x;  // not contracted: the reference's four products and two sums
-                ob[i] = rot_a ? x * s + y * c : y;
+                oa[i] = FULL || rot_a ? x * c - y * s : x;  // not contracted: the reference's four products and two sums
+                ob[i] = FULL || rot_a ? x * s + y * c : y;
             }
         }
         const bool live = hh_first + it * HPW < nheads;
         const int off = head_off(it);
         if (live) {
-            io<T>::store_nt(base + off + off_a, oa);
-            io<T>::store_nt(base + off + off_b, ob);
+            io<T>::store_wt(base + off + off_a, oa);
+            io<T>::store_wt(base + off + off_b, ob);
         }
         if constexpr (KV) {
             if (live) {
@@ -193,8 +255,8 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
                             va[i] += bva[it][i];
                             vb[i] += bvb[it][i];
                         }
-                        io<T>::store_nt(vout + off + off_a, va);
-                        io<T>::store_nt(vout + off + off_b, vb);
+                        io<T>::store_wt(vout + off + off_a, va);
+                        io<T>::store_wt(vout + off + off_b, vb);
                     }
                 }
                 if (kc != nullptr) {  // kc == nullptr: cache position out of range, the row's cache store is skipped
@@ -209,84 +271,106 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
     }
 }
 
-template <typename T, int HD, int ITERQ, bool KV = false, bool PAIRS = false, bool BIAS = false, bool NORM = true>
+// BLOCK: the workgroup size the host launches (the wave's LDS slot is its index in the workgroup).
+template <typename T, int HD, int ITERQ, bool KV = false, bool PAIRS = false, bool BIAS = false, bool NORM = true, bool LDSC = false, int BLOCK = 256>
 DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv,
                           float eps, int rot, uint32_t vblock, T* v = nullptr, const uint32_t* cache_pos = nullptr,
                           f16_t* k_cache = nullptr, f16_t* v_cache = nullptr, uint32_t capacity = 0,
                           uint32_t* fault = nullptr, const float* qb = nullptr, const float* kb = nullptr,
                           const float* vb = nullptr) {
     constexpr int LPH = HD / 2 / io<T>::VEC, HPW = 64 / LPH;
+    __shared__ __attribute__((aligned(16))) float lds_consts[LDSC ? BLOCK / 64 : 1][LDSC ? 2 * HD : 4];
+    float* lmem = LDSC ? lds_consts[threadIdx.x >> 6] : nullptr;
     const int lane = threadIdx.x & 63;
     const int l = lane % LPH, sub = lane / LPH;
-    const int gq = (n_q + HPW * ITERQ - 1) / (HPW * ITERQ), gk = (n_kv + HPW - 1) / HPW;
-    // all q items first (the longer ones, up to two passes), then the k items, one pass each
-    const uint64_t wid = ((uint64_t)vblock * blockDim.x + threadIdx.x) >> 6;
-    const uint64_t nq_items = (uint64_t)rows * gq;
-    if (wid >= nq_items + (uint64_t)rows * gk) return;  // whole wave
+    const uint32_t gq = (n_q + HPW * ITERQ - 1) / (HPW * ITERQ), gk = (n_kv + HPW - 1) / HPW;
+    // all q items first (the longer ones when ITERQ > 1), then the k items, one pass each.  The wave's index is a
+    // scalar (the host keeps the number of waves below 2^32): the row and group come from scalar arithmetic.
+    const uint32_t wid = __builtin_amdgcn_readfirstlane(vblock * (blockDim.x >> 6) + (threadIdx.x >> 6));
+    const uint32_t nq_items = (uint32_t)rows * gq;
+    if (wid >= nq_items + (uint32_t)rows * gk) return;  // whole wave
+    // Two facts of the launch choose among four instances of the item: whether this tensor has a norm weight (a model
+    // may norm q and not k) and whether the whole head rotates (no per-lane selects then).  Uniform branches.
+    const bool full = rot == HD;
     if (wid < nq_items) {
-        const uint64_t row = wid / gq;
-        qk_item<T, HD, ITERQ, false, PAIRS, BIAS, NORM>(q + row * (uint64_t)n_q * HD, n_q, (int)(wid % gq), qw, rope + row * (uint64_t)rot, eps, l, sub,
-                                                  rot, nullptr, nullptr, nullptr, qb);
+        const uint32_t row = wid / gq;
+        T* base = q + (uint64_t)row * n_q * HD;
+        const float* trow = rope + (uint64_t)row * rot;
+        const int g = (int)(wid - row * gq);
+#define APK_QK_Q(N, F) qk_item<T, HD, ITERQ, false, PAIRS, BIAS, N, LDSC, F>(base, n_q, g, qw, trow, eps, l, sub, rot, nullptr, nullptr, nullptr, qb, nullptr, nullptr, lmem)
+        if (NORM && qw) { if (full) APK_QK_Q(NORM, true); else APK_QK_Q(NORM, false); }
+        else { if (full) APK_QK_Q(false, true); else APK_QK_Q(false, false); }
+#undef APK_QK_Q
     } else {
-        const uint64_t w2 = wid - nq_items, row = w2 / gk;
+        const uint32_t w2 = wid - nq_items, row = w2 / gk;
+        const int g = (int)(w2 - row * gk);
         const uint64_t kv_dim = (uint64_t)n_kv * HD;
+        T* base = k + row * kv_dim;
+        const float* trow = rope + (uint64_t)row * rot;
+        f16_t *kc = nullptr, *vc = nullptr;
+        T* vrow = nullptr;
         if constexpr (KV) {
             const uint32_t pos = cache_pos[row];
             const bool ok = pos < capacity;
-            if (!ok && lane == 0 && w2 % gk == 0) atomicOr(fault, APK_FAULT_CACHE_RANGE);
-            qk_item<T, HD, 1, true, PAIRS, BIAS, NORM>(k + row * kv_dim, n_kv, (int)(w2 % gk), kw, rope + row * (uint64_t)rot, eps, l, sub, rot,
-                                                 ok ? k_cache + pos * kv_dim : nullptr, v + row * kv_dim,
-                                                 ok ? v_cache + pos * kv_dim : nullptr, kb, vb, v + row * kv_dim);
-        } else {
-            qk_item<T, HD, 1, false, PAIRS, BIAS, NORM>(k + row * kv_dim, n_kv, (int)(w2 % gk), kw, rope + row * (uint64_t)rot, eps, l, sub, rot,
-                                                  nullptr, nullptr, nullptr, kb);
+            if (!ok && lane == 0 && g == 0) atomicOr(fault, APK_FAULT_CACHE_RANGE);
+            kc = ok ? k_cache + pos * kv_dim : nullptr;  // nullptr: the row's cache store is skipped
+            vc = ok ? v_cache + pos * kv_dim : nullptr;
+            vrow = v + row * kv_dim;
         }
+#define APK_QK_K(N, F) qk_item<T, HD, 1, KV, PAIRS, BIAS, N, LDSC, F>(base, n_kv, g, kw, trow, eps, l, sub, rot, kc, vrow, vc, kb, vb, vrow, lmem)
+        if (NORM && kw) { if (full) APK_QK_K(NORM, true); else APK_QK_K(NORM, false); }
+        else { if (full) APK_QK_K(false, true); else APK_QK_K(false, false); }
+#undef APK_QK_K
     }
 }
-// At most 128 VGPRs (at least 4 waves per SIMD).
-#define APK_QK_OCC __attribute__((amdgpu_waves_per_eu(4)))
-// One kernel per (norm or not, pairing, cache store, biases, type, head size, passes per q wave).  PFX: apk_qknorm_rope
+// fp16 tiles: one pass per wave, constants in LDS, workgroups of two waves, up to 64 registers (8 waves per SIMD);
+// f32 tiles: one pass per wave, constants in registers, workgroups of four waves.
+template <typename T> struct qk_shape { static constexpr bool LDSC = false; static constexpr int BLOCK = 256; };
+template <> struct qk_shape<f16_t> { static constexpr bool LDSC = true; static constexpr int BLOCK = 128; };
+// Resident waves per SIMD the compiler is to allow for (W16 for the fp16 kernels: the register ceiling that the
+// variant meets without spilling -- 80 plain or with biases, 96 with the cache store, 128 with both; f32: 128).
+#define APK_QK_OCC(T, W16) __launch_bounds__(qk_shape<T>::BLOCK) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 2 ? W16 : 4)))
+// One kernel per (norm or not, pairing, cache store, biases, type, head size).  PFX: apk_qknorm_rope
 // (a norm weight for q and / or k) or apk_rope (none for either); PN: pairs_ or nothing.  The argument lists are the
 // same with and without norm weights (qw, kw are then NULL and unused).
 #define APK_QK_PLAIN(PFX, NORM, T, TN, HD, ITER, PAIRS, PN)                                                        \
-    extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void PFX##_##PN##TN##_hd##HD##_i##ITER(               \
+    extern "C" __global__ APK_QK_OCC(T, 6) void PFX##_##PN##TN##_hd##HD##_i##ITER(                                    \
         T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv, float eps, int rot) { \
-        qknorm_rope_body<T, HD, ITER, false, PAIRS, false, NORM>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x); \
+        qknorm_rope_body<T, HD, ITER, false, PAIRS, false, NORM, qk_shape<T>::LDSC, qk_shape<T>::BLOCK>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x); \
     }
 // The same with the K/V cache store fused in: rotated k and the row's v narrowed to fp16
 // at cache row cache_pos[row] (one launch instead of QK-norm+RoPE, then two narrowing copies).
 #define APK_QK_KV(PFX, NORM, T, TN, HD, ITER, PAIRS, PN)                                                           \
-    extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void PFX##_##PN##kv_##TN##_hd##HD##_i##ITER(          \
+    extern "C" __global__ APK_QK_OCC(T, 5) void PFX##_##PN##kv_##TN##_hd##HD##_i##ITER(                               \
         T* q, T* k, const T* v, const float* qw, const float* kw, const float* rope, const uint32_t* cache_pos,   \
         f16_t* k_cache, f16_t* v_cache, uint32_t capacity, int rows, int n_q, int n_kv, float eps, uint32_t* fault, int rot) { \
-        qknorm_rope_body<T, HD, ITER, true, PAIRS, false, NORM>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x, (T*)v, \
+        qknorm_rope_body<T, HD, ITER, true, PAIRS, false, NORM, qk_shape<T>::LDSC, qk_shape<T>::BLOCK>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x, (T*)v, \
                                                                 cache_pos, k_cache, v_cache, capacity, fault);    \
     }
 // With the projection biases.  Without the cache store v is not touched here; with it, v + v_bias is written back
 // to v and narrowed into the cache.
 #define APK_QK_BIAS(PFX, NORM, T, TN, HD, ITER, PAIRS, PN)                                                         \
-    extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void PFX##_##PN##bias_##TN##_hd##HD##_i##ITER(        \
+    extern "C" __global__ APK_QK_OCC(T, 6) void PFX##_##PN##bias_##TN##_hd##HD##_i##ITER(                             \
         T* q, T* k, const float* qw, const float* kw, const float* rope, int rows, int n_q, int n_kv, float eps, int rot, \
         const float* qb, const float* kb) {                                                                       \
-        qknorm_rope_body<T, HD, ITER, false, PAIRS, true, NORM>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x, nullptr, \
+        qknorm_rope_body<T, HD, ITER, false, PAIRS, true, NORM, qk_shape<T>::LDSC, qk_shape<T>::BLOCK>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x, nullptr, \
                                                                 nullptr, nullptr, nullptr, 0, nullptr, qb, kb, nullptr); \
     }                                                                                                             \
-    extern "C" __global__ __launch_bounds__(256) APK_QK_OCC void PFX##_##PN##kv_bias_##TN##_hd##HD##_i##ITER(     \
+    extern "C" __global__ APK_QK_OCC(T, 4) void PFX##_##PN##kv_bias_##TN##_hd##HD##_i##ITER(                          \
         T* q, T* k, T* v, const float* qw, const float* kw, const float* rope, const uint32_t* cache_pos,         \
         f16_t* k_cache, f16_t* v_cache, uint32_t capacity, int rows, int n_q, int n_kv, float eps, uint32_t* fault, int rot, \
         const float* qb, const float* kb, const float* vb) {                                                      \
-        qknorm_rope_body<T, HD, ITER, true, PAIRS, true, NORM>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x, v, \
+        qknorm_rope_body<T, HD, ITER, true, PAIRS, true, NORM, qk_shape<T>::LDSC, qk_shape<T>::BLOCK>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x, v, \
                                                                cache_pos, k_cache, v_cache, capacity, fault, qb, kb, vb); \
     }
 #define APK_QK_FAMILY(PFX, NORM, T, TN, HD, ITER)                                                                  \
     APK_QK_PLAIN(PFX, NORM, T, TN, HD, ITER, false, ) APK_QK_PLAIN(PFX, NORM, T, TN, HD, ITER, true, pairs_)       \
     APK_QK_KV(PFX, NORM, T, TN, HD, ITER, false, ) APK_QK_KV(PFX, NORM, T, TN, HD, ITER, true, pairs_)             \
     APK_QK_BIAS(PFX, NORM, T, TN, HD, ITER, false, ) APK_QK_BIAS(PFX, NORM, T, TN, HD, ITER, true, pairs_)
-// two passes per q wave in fp16 only (measured: f32 is fastest with one)
+// one pass per wave for both types (measured)
 #define APK_QK_SIZES(PFX, NORM)                                                                                    \
     APK_QK_FAMILY(PFX, NORM, float, f32, 64, 1) APK_QK_FAMILY(PFX, NORM, float, f32, 128, 1) APK_QK_FAMILY(PFX, NORM, float, f32, 256, 1) \
-    APK_QK_FAMILY(PFX, NORM, f16_t, f16, 64, 1) APK_QK_FAMILY(PFX, NORM, f16_t, f16, 128, 1) APK_QK_FAMILY(PFX, NORM, f16_t, f16, 256, 1) \
-    APK_QK_FAMILY(PFX, NORM, f16_t, f16, 64, 2) APK_QK_FAMILY(PFX, NORM, f16_t, f16, 128, 2) APK_QK_FAMILY(PFX, NORM, f16_t, f16, 256, 2)
+    APK_QK_FAMILY(PFX, NORM, f16_t, f16, 64, 1) APK_QK_FAMILY(PFX, NORM, f16_t, f16, 128, 1) APK_QK_FAMILY(PFX, NORM, f16_t, f16, 256, 1)
 APK_QK_SIZES(apk_qknorm_rope, true)
 APK_QK_SIZES(apk_rope, false)
 // Any other head geometry: head_dim not 64/128/256, a rotary table that covers only the
