@@ -246,7 +246,9 @@ int plan_qknorm_rope(size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size
     const size_t epl = 16 / es, lph = head_dim / 2 / epl, hpw = 64 / lph;
     const size_t gk = (n_kv + hpw - 1) / hpw;
     const unsigned iter = 1;
-    const uint64_t waves = (uint64_t)rows * ((n_q + hpw * iter - 1) / (hpw * iter) + gk);
+    // with the cache store, the v rows are narrowed by waves of their own (as many as the k waves)
+    const size_t waves_per_row = (n_q + hpw * iter - 1) / (hpw * iter) + gk + (with_kv ? gk : 0);
+    const uint64_t waves = (uint64_t)rows * waves_per_row;
     const unsigned block = dtype == APK_F16 ? 128 : 256;
     const uint64_t grid = (waves * 64 + block - 1) / block;
     if (grid > 0x7fffffffu || waves > 0xffffffffu) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope: too large");  // the kernels index waves in 32 bits
@@ -257,7 +259,7 @@ int plan_qknorm_rope(size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size
     p->block = block;
     p->tiles_per_lane = iter;
     p->lanes_per_row = (unsigned)lph;
-    p->waves_per_row = (unsigned)((n_q + hpw * iter - 1) / (hpw * iter) + gk);
+    p->waves_per_row = (unsigned)waves_per_row;
     p->items = (unsigned)(waves > 0xffffffffu ? 0xffffffffu : waves);
     return APK_OK;
 }

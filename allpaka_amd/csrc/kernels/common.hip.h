@@ -19,18 +19,23 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 DEV float h2f(uint32_t bits16) { return (float)__builtin_bit_cast(f16_t, (uint16_t)bits16); }
 
 // ----------------------------------------------------------- 16-byte tile IO
-// Streaming stores: non-temporal and written through at device scope (the sc1 bit).  A plain or nt-only store leaves
-// its line dirty in the XCD's L2, and the dirty lines of a launch are written back when the kernel ends, after the
-// last wave: for an in-place stream of 75 MB that tail is 1 us of 14 (measured with a one-tile-per-lane copy:
-// 13.9 us with nt stores, 12.9 us with sc1 nt).  The compiler has no builtin for the bit, so the instruction is
-// written out; the s_nop covers the two wait states this part needs between a store of more than 8 bytes and
-// a VALU write to its data registers, which the compiler cannot insert for an instruction it does not see.
-DEV void st_stream16(void* p, u32x4 v) {
-    asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
-}
-DEV void st_stream8(void* p, u32x2 v) {
-    asm volatile("global_store_dwordx2 %0, %1, off sc1 nt" ::"v"(p), "v"(v) : "memory");
-}
+// Two kinds of streaming store.  nt_store: non-temporal (the compiler's builtin).  wt_store: non-temporal and written
+// through at device scope (the sc1 bit).  An nt-only store leaves its line dirty in the XCD's L2, and what a launch
+// left dirty is written back when the kernel ends, after its last wave; a written-through store has nothing left to
+// write back but completes later, and a wave holds its registers until its stores complete.  Measured per kernel:
+// short waves at full occupancy gain (one-tile-per-lane copy of 75 MB in place: 13.9 -> 12.9 us; SwiGLU on
+// [8192 x 768] f32: 14.0 -> 13.65; QK-norm + RoPE: 13.8 -> 13.5), long waves at low occupancy lose (add + RMSNorm with
+// a wave per row: 14.4 -> 16.4; the embedding gathers 5.3 -> 5.7), so each kernel family names the kind it takes.
+// The compiler has no builtin for the bit, so the instruction is written out; the s_nop covers the two wait
+// states this part needs between a store of more than 8 bytes and a VALU write to its data registers, which the
+// compiler cannot insert for an instruction it does not see.  No kernel reads back what it stores this way, so the
+// statement needs no memory clobber (the stored value depends on every load it must follow).
+DEV void wt_store(u32x4 v, void* p) { asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 1" ::"v"(p), "v"(v)); }
+DEV void wt_store(f32x4 v, void* p) { wt_store(__builtin_bit_cast(u32x4, v), p); }
+DEV void wt_store(u32x2 v, void* p) { asm volatile("global_store_dwordx2 %0, %1, off sc1 nt" ::"v"(p), "v"(v)); }
+DEV void nt_store(u32x4 v, void* p) { __builtin_nontemporal_store(v, (u32x4*)p); }
+DEV void nt_store(f32x4 v, void* p) { __builtin_nontemporal_store(v, (f32x4*)p); }
+DEV void nt_store(u32x2 v, void* p) { __builtin_nontemporal_store(v, (u32x2*)p); }
 template <typename T> struct io;
 template <> struct io<float> {
     static constexpr int VEC = 4;
@@ -52,11 +57,11 @@ template <> struct io<float> {
     }
     DEV void store_nt(float* p, const float* v) {
         f32x4 t = {v[0], v[1], v[2], v[3]};
-        __builtin_nontemporal_store(t, (f32x4*)p);
+        nt_store(t, p);
     }
-    DEV void store_wt(float* p, const float* v) {  // streaming store, written through (see st_stream16)
+    DEV void store_wt(float* p, const float* v) {
         f32x4 t = {v[0], v[1], v[2], v[3]};
-        st_stream16(p, __builtin_bit_cast(u32x4, t));
+        wt_store(t, p);
     }
 };
 template <> struct io<f16_t> {
@@ -84,8 +89,8 @@ template <> struct io<f16_t> {
     DEV void load(const f16_t* p, float* v) { unpack(*(const u32x4*)p, v); }
     DEV void load_nt(const f16_t* p, float* v) { unpack(__builtin_nontemporal_load((const u32x4*)p), v); }
     DEV void store(f16_t* p, const float* v) { *(u32x4*)p = pack(v); }
-    DEV void store_nt(f16_t* p, const float* v) { __builtin_nontemporal_store(pack(v), (u32x4*)p); }
-    DEV void store_wt(f16_t* p, const float* v) { st_stream16(p, pack(v)); }
+    DEV void store_nt(f16_t* p, const float* v) { nt_store(pack(v), p); }
+    DEV void store_wt(f16_t* p, const float* v) { wt_store(pack(v), p); }
 };
 
 // ------------------------------------------------------- wave reductions (DPP)
@@ -157,7 +162,7 @@ template <> __device__ __forceinline__ void store_f16_tile<float>(f16_t* p, cons
     f32x2 lo = {v[0], v[1]}, hi = {v[2], v[3]};
     u32x2 t = {__builtin_bit_cast(uint32_t, __builtin_convertvector(lo, f16x2)),
                __builtin_bit_cast(uint32_t, __builtin_convertvector(hi, f16x2))};
-    st_stream8(p, t);
+    wt_store(t, p);
 }
 
 

@@ -59,7 +59,7 @@ template <typename T, int UNR, bool GELU = false> DEV void swiglu_body(T* gate, 
         if (c < nvec) {
 #pragma unroll
             for (int i = 0; i < VEC; i++) g[j][i] = gate_mul<T, GELU>(g[j][i], u[j][i]);
-            io<T>::store_nt(gate + c * VEC, g[j]);
+            io<T>::store_wt(gate + c * VEC, g[j]);
         }
     }
     // ragged tail (n not a multiple of the 16-byte tile): last block, scalar
@@ -94,7 +94,7 @@ template <typename T> DEV void add_assign_body(T* a, const T* b, uint64_t n) {
         io<T>::load_nt(b + c * VEC, y);
 #pragma unroll
         for (int i = 0; i < VEC; i++) x[i] += y[i];
-        io<T>::store_nt(a + c * VEC, x);
+        io<T>::store_wt(a + c * VEC, x);
     }
     if (blockIdx.x == gridDim.x - 1)
         for (uint64_t i = nvec * VEC + threadIdx.x; i < n; i += blockDim.x) a[i] = (T)((float)a[i] + (float)b[i]);
@@ -121,7 +121,7 @@ template <typename T> DEV void add_bias_rows_body(T* x, const float* bias, uint6
         for (int q = 0; q < VEC; q += 4) io<float>::load(bias + col + q, b + q);
 #pragma unroll
         for (int i = 0; i < VEC; i++) v[i] += b[i];
-        io<T>::store_nt(x + c * VEC, v);
+        io<T>::store_wt(x + c * VEC, v);
     } else {
         if (c >= rows * n) return;
         x[c] = (T)((float)x[c] + bias[c % n]);
@@ -159,11 +159,11 @@ extern "C" __global__ __launch_bounds__(256) void apk_cast_f32_f16(const float* 
     if (c1 < nq) b = __builtin_nontemporal_load((const f32x4*)src + c1);
     if (c0 < nq) {
         const u32x2 o = {narrow_ref(a.x) | (uint32_t)narrow_ref(a.y) << 16, narrow_ref(a.z) | (uint32_t)narrow_ref(a.w) << 16};
-        __builtin_nontemporal_store(o, (u32x2*)dst + c0);
+        wt_store(o, (u32x2*)dst + c0);
     }
     if (c1 < nq) {
         const u32x2 o = {narrow_ref(b.x) | (uint32_t)narrow_ref(b.y) << 16, narrow_ref(b.z) | (uint32_t)narrow_ref(b.w) << 16};
-        __builtin_nontemporal_store(o, (u32x2*)dst + c1);
+        wt_store(o, (u32x2*)dst + c1);
     }
     if (blockIdx.x == gridDim.x - 1)
         for (uint64_t i = nq * 4 + threadIdx.x; i < n; i += blockDim.x) dst[i] = narrow_ref(src[i]);
@@ -175,11 +175,11 @@ extern "C" __global__ __launch_bounds__(256) void apk_cast_f16_f32(const uint16_
     if (c1 < nq) b = __builtin_nontemporal_load((const u32x2*)src + c1);
     if (c0 < nq) {
         const f32x4 o = {widen_ref((uint16_t)a.x), widen_ref((uint16_t)(a.x >> 16)), widen_ref((uint16_t)a.y), widen_ref((uint16_t)(a.y >> 16))};
-        __builtin_nontemporal_store(o, (f32x4*)dst + c0);
+        wt_store(o, (f32x4*)dst + c0);
     }
     if (c1 < nq) {
         const f32x4 o = {widen_ref((uint16_t)b.x), widen_ref((uint16_t)(b.x >> 16)), widen_ref((uint16_t)b.y), widen_ref((uint16_t)(b.y >> 16))};
-        __builtin_nontemporal_store(o, (f32x4*)dst + c1);
+        wt_store(o, (f32x4*)dst + c1);
     }
     if (blockIdx.x == gridDim.x - 1)
         for (uint64_t i = nq * 4 + threadIdx.x; i < n; i += blockDim.x) dst[i] = widen_ref(src[i]);

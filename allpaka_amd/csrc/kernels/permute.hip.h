@@ -392,7 +392,7 @@ extern "C" __global__ __launch_bounds__(256) void apk_gather_rows(const u32x4* s
         m &= m - 1;
         const u32x4* sp = src + (uint64_t)__shfl(t, j, 64) * row_vecs;
         u32x4* dp = dst + (uint64_t)(r0 + (uint32_t)j) * row_vecs;
-        for (int c = threadIdx.x; c < row_vecs; c += blockDim.x) __builtin_nontemporal_store(sp[c], dp + c);
+        for (int c = threadIdx.x; c < row_vecs; c += blockDim.x) nt_store(sp[c], dp + c);
     }
 }
 
@@ -429,7 +429,7 @@ DEV void scatter_rows_body(const u32x4* src, const uint32_t* hit_row, uint32_t k
     u32x4* dp = dst + (uint64_t)r * row_vecs;
 #pragma unroll
     for (int i = 0; i < TPT; i++)
-        if (c[i] < row_vecs) __builtin_nontemporal_store(a[i], dp + c[i]);
+        if (c[i] < row_vecs) nt_store(a[i], dp + c[i]);
 }
 extern "C" __global__ __launch_bounds__(256) void apk_scatter_rows_t1(const u32x4* src, const uint32_t* hit_row, uint32_t k,
                                                                      uint32_t total_rows, int row_vecs, u32x4* dst,
@@ -445,7 +445,7 @@ extern "C" __global__ __launch_bounds__(256) void apk_scatter_rows_t2(const u32x
 // Reference stream for bandwidth calibration: dst = src, one 16-byte tile per lane.
 extern "C" __global__ __launch_bounds__(256) void apk_copy(const u32x4* src, u32x4* dst, uint64_t nvec) {
     const uint64_t c = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (c < nvec) __builtin_nontemporal_store(__builtin_nontemporal_load(src + c), dst + c);
+    if (c < nvec) wt_store(__builtin_nontemporal_load(src + c), dst + c);
 }
 
 // The shared expert of GLM-style MoE layers in the per-token hit lists (model/prefill.rs:621-635, flattened :658-675):

@@ -62,8 +62,7 @@ template <> struct rotstat<f16_t> : stat<float> {
 // waves: no barrier, only the wave's own LDS counter.
 template <typename T, int HD, int ITER, bool KV = false, bool PAIRS = false, bool BIAS = false, bool NORM = true, bool LDSC = false, bool FULL = false>
 DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, float eps, int l, int sub, int rot,
-                 f16_t* kc = nullptr, const T* vrow = nullptr, f16_t* vc = nullptr, const float* bias = nullptr,
-                 const float* vbias = nullptr, T* vout = nullptr, float* lmem = nullptr) {
+                 f16_t* kc = nullptr, const float* bias = nullptr, float* lmem = nullptr) {
     constexpr int EPL = io<T>::VEC;   // elements per lane per half
     constexpr int HALF = HD / 2;
     constexpr int LPH = HALF / EPL;   // lanes per head
@@ -121,8 +120,8 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
             }
         }
     }
-    typename io<T>::raw_t araw[ITER], braw[ITER], varaw[ITER], vbraw[ITER];
-    float ba[BIAS ? ITER : 1][EPL], bb[BIAS ? ITER : 1][EPL], bva[BIAS && KV ? ITER : 1][EPL], bvb[BIAS && KV ? ITER : 1][EPL];
+    typename io<T>::raw_t araw[ITER], braw[ITER];
+    float ba[BIAS ? ITER : 1][EPL], bb[BIAS ? ITER : 1][EPL];
     // head of pass `it` and its element offset: recomputed where needed (a few integer
     // operations) rather than kept in registers across the loads
     const int hh_first = g * ITER * HPW + sub;
@@ -139,22 +138,9 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
                     io<float>::load(bias + off + off_b + i, bb[it] + i);
                 }
             }
-            if constexpr (KV) {
-                if (vbias) {
-#pragma unroll
-                    for (int i = 0; i < EPL; i += 4) {
-                        io<float>::load(vbias + off + off_a + i, bva[it] + i);
-                        io<float>::load(vbias + off + off_b + i, bvb[it] + i);
-                    }
-                }
-            }
         }
         araw[it] = io<T>::ldraw_nt(base + off + off_a);
         braw[it] = io<T>::ldraw_nt(base + off + off_b);
-        if constexpr (KV) {
-            varaw[it] = io<T>::ldraw_nt(vrow + off + off_a);
-            vbraw[it] = io<T>::ldraw_nt(vrow + off + off_b);
-        }
     }
     __builtin_amdgcn_sched_barrier(0);  // every load above; all uses below
     if constexpr (LDSC) {
@@ -244,30 +230,51 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
             io<T>::store_wt(base + off + off_b, ob);
         }
         if constexpr (KV) {
-            if (live) {
-                float va[EPL], vb[EPL];
-                io<T>::widen(varaw[it], va);
-                io<T>::widen(vbraw[it], vb);
-                if constexpr (BIAS) {
-                    if (vbias) {
-#pragma unroll
-                        for (int i = 0; i < EPL; i++) {
-                            va[i] += bva[it][i];
-                            vb[i] += bvb[it][i];
-                        }
-                        io<T>::store_wt(vout + off + off_a, va);
-                        io<T>::store_wt(vout + off + off_b, vb);
-                    }
-                }
-                if (kc != nullptr) {  // kc == nullptr: cache position out of range, the row's cache store is skipped
-                    store_f16_tile<T>(kc + off + off_a, oa);
-                    store_f16_tile<T>(kc + off + off_b, ob);
-                    store_f16_tile<T>(vc + off + off_a, va);
-                    store_f16_tile<T>(vc + off + off_b, vb);
-                }
+            if (live && kc != nullptr) {  // kc == nullptr: cache position out of range, the row's cache store is skipped
+                store_f16_tile<T>(kc + off + off_a, oa);
+                store_f16_tile<T>(kc + off + off_b, ob);
             }
         }
         __builtin_amdgcn_sched_barrier(0);  // pass by pass: pass it+1 waits only for its own tiles
+    }
+}
+
+// The v half of the cache store, waves of its own (a pure stream: short, few registers, so the k waves stay as light
+// as the q waves): a wave narrows HPW heads of the row's v into the cache row vc (two 16-byte tiles per lane, each
+// instruction a contiguous run); with a bias, v + v_bias is written back to v as well.
+template <typename T, int HD, bool BIAS>
+DEV void v_item(T* vrow, int nheads, int g, f16_t* vc, const float* vbias, int lane) {
+    constexpr int EPL = io<T>::VEC, HPW = 64 / (HD / 2 / EPL);
+    const int total = nheads * HD, start = g * HPW * HD;
+    typename io<T>::raw_t raw[2];
+    float bv[BIAS ? 2 : 1][EPL];
+    int off[2];
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        off[j] = start + (lane + 64 * j) * EPL;
+        const int oc = min(off[j], total - EPL);  // a lane past the last head re-reads the last tile and stores nothing
+        if constexpr (BIAS) {
+            if (vbias) {
+#pragma unroll
+                for (int i = 0; i < EPL; i += 4) io<float>::load(vbias + oc + i, bv[j] + i);
+            }
+        }
+        raw[j] = io<T>::ldraw_nt(vrow + oc);
+    }
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        float v[EPL];
+        io<T>::widen(raw[j], v);
+        if (off[j] < total) {
+            if constexpr (BIAS) {
+                if (vbias) {
+#pragma unroll
+                    for (int i = 0; i < EPL; i++) v[i] += bv[j][i];
+                    io<T>::store_wt(vrow + off[j], v);
+                }
+            }
+            if (vc != nullptr) store_f16_tile<T>(vc + off[j], v);
+        }
     }
 }
 
@@ -284,43 +291,46 @@ DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const fl
     const int lane = threadIdx.x & 63;
     const int l = lane % LPH, sub = lane / LPH;
     const uint32_t gq = (n_q + HPW * ITERQ - 1) / (HPW * ITERQ), gk = (n_kv + HPW - 1) / HPW;
-    // all q items first (the longer ones when ITERQ > 1), then the k items, one pass each.  The wave's index is a
-    // scalar (the host keeps the number of waves below 2^32): the row and group come from scalar arithmetic.
+    // The k items first, then (with the cache store) the v items, then the q items.  The wave's index is a scalar
+    // (the host keeps the number of waves below 2^32): the row and group come from scalar arithmetic.
     const uint32_t wid = __builtin_amdgcn_readfirstlane(vblock * (blockDim.x >> 6) + (threadIdx.x >> 6));
-    const uint32_t nq_items = (uint32_t)rows * gq;
-    if (wid >= nq_items + (uint32_t)rows * gk) return;  // whole wave
+    const uint32_t nq_items = (uint32_t)rows * gq, nk_items = (uint32_t)rows * gk, nv_items = KV ? nk_items : 0;
+    if (wid >= nq_items + nk_items + nv_items) return;  // whole wave
     // Two facts of the launch choose among four instances of the item: whether this tensor has a norm weight (a model
     // may norm q and not k) and whether the whole head rotates (no per-lane selects then).  Uniform branches.
     const bool full = rot == HD;
-    if (wid < nq_items) {
-        const uint32_t row = wid / gq;
+    const uint64_t kv_dim = (uint64_t)n_kv * HD;
+    if (wid >= nk_items + nv_items) {
+        const uint32_t w1 = wid - nk_items - nv_items, row = w1 / gq;
         T* base = q + (uint64_t)row * n_q * HD;
         const float* trow = rope + (uint64_t)row * rot;
-        const int g = (int)(wid - row * gq);
-#define APK_QK_Q(N, F) qk_item<T, HD, ITERQ, false, PAIRS, BIAS, N, LDSC, F>(base, n_q, g, qw, trow, eps, l, sub, rot, nullptr, nullptr, nullptr, qb, nullptr, nullptr, lmem)
+        const int g = (int)(w1 - row * gq);
+#define APK_QK_Q(N, F) qk_item<T, HD, ITERQ, false, PAIRS, BIAS, N, LDSC, F>(base, n_q, g, qw, trow, eps, l, sub, rot, nullptr, qb, lmem)
         if (NORM && qw) { if (full) APK_QK_Q(NORM, true); else APK_QK_Q(NORM, false); }
         else { if (full) APK_QK_Q(false, true); else APK_QK_Q(false, false); }
 #undef APK_QK_Q
-    } else {
-        const uint32_t w2 = wid - nq_items, row = w2 / gk;
-        const int g = (int)(w2 - row * gk);
-        const uint64_t kv_dim = (uint64_t)n_kv * HD;
+    } else if (wid < nk_items) {
+        const uint32_t row = wid / gk;
+        const int g = (int)(wid - row * gk);
         T* base = k + row * kv_dim;
         const float* trow = rope + (uint64_t)row * rot;
-        f16_t *kc = nullptr, *vc = nullptr;
-        T* vrow = nullptr;
+        f16_t* kc = nullptr;
         if constexpr (KV) {
             const uint32_t pos = cache_pos[row];
             const bool ok = pos < capacity;
             if (!ok && lane == 0 && g == 0) atomicOr(fault, APK_FAULT_CACHE_RANGE);
             kc = ok ? k_cache + pos * kv_dim : nullptr;  // nullptr: the row's cache store is skipped
-            vc = ok ? v_cache + pos * kv_dim : nullptr;
-            vrow = v + row * kv_dim;
         }
-#define APK_QK_K(N, F) qk_item<T, HD, 1, KV, PAIRS, BIAS, N, LDSC, F>(base, n_kv, g, kw, trow, eps, l, sub, rot, kc, vrow, vc, kb, vb, vrow, lmem)
+#define APK_QK_K(N, F) qk_item<T, HD, 1, KV, PAIRS, BIAS, N, LDSC, F>(base, n_kv, g, kw, trow, eps, l, sub, rot, kc, kb, lmem)
         if (NORM && kw) { if (full) APK_QK_K(NORM, true); else APK_QK_K(NORM, false); }
         else { if (full) APK_QK_K(false, true); else APK_QK_K(false, false); }
 #undef APK_QK_K
+    } else {
+        if constexpr (KV) {
+            const uint32_t w2 = wid - nk_items, row = w2 / gk;
+            const uint32_t pos = cache_pos[row];
+            v_item<T, HD, BIAS>(v + row * kv_dim, n_kv, (int)(w2 - row * gk), pos < capacity ? v_cache + pos * kv_dim : nullptr, vb, lane);
+        }
     }
 }
 // fp16 tiles: one pass per wave, constants in LDS, workgroups of two waves, up to 64 registers (8 waves per SIMD);
@@ -341,7 +351,7 @@ template <> struct qk_shape<f16_t> { static constexpr bool LDSC = true; static c
 // The same with the K/V cache store fused in: rotated k and the row's v narrowed to fp16
 // at cache row cache_pos[row] (one launch instead of QK-norm+RoPE, then two narrowing copies).
 #define APK_QK_KV(PFX, NORM, T, TN, HD, ITER, PAIRS, PN)                                                           \
-    extern "C" __global__ APK_QK_OCC(T, 5) void PFX##_##PN##kv_##TN##_hd##HD##_i##ITER(                               \
+    extern "C" __global__ APK_QK_OCC(T, 6) void PFX##_##PN##kv_##TN##_hd##HD##_i##ITER(                               \
         T* q, T* k, const T* v, const float* qw, const float* kw, const float* rope, const uint32_t* cache_pos,   \
         f16_t* k_cache, f16_t* v_cache, uint32_t capacity, int rows, int n_q, int n_kv, float eps, uint32_t* fault, int rot) { \
         qknorm_rope_body<T, HD, ITER, true, PAIRS, false, NORM, qk_shape<T>::LDSC, qk_shape<T>::BLOCK>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x, (T*)v, \
@@ -356,7 +366,7 @@ template <> struct qk_shape<f16_t> { static constexpr bool LDSC = true; static c
         qknorm_rope_body<T, HD, ITER, false, PAIRS, true, NORM, qk_shape<T>::LDSC, qk_shape<T>::BLOCK>(q, k, qw, kw, rope, rows, n_q, n_kv, eps, rot, blockIdx.x, nullptr, \
                                                                 nullptr, nullptr, nullptr, 0, nullptr, qb, kb, nullptr); \
     }                                                                                                             \
-    extern "C" __global__ APK_QK_OCC(T, 4) void PFX##_##PN##kv_bias_##TN##_hd##HD##_i##ITER(                          \
+    extern "C" __global__ APK_QK_OCC(T, 6) void PFX##_##PN##kv_bias_##TN##_hd##HD##_i##ITER(                          \
         T* q, T* k, T* v, const float* qw, const float* kw, const float* rope, const uint32_t* cache_pos,         \
         f16_t* k_cache, f16_t* v_cache, uint32_t capacity, int rows, int n_q, int n_kv, float eps, uint32_t* fault, int rot, \
         const float* qb, const float* kb, const float* vb) {                                                      \
