@@ -424,6 +424,26 @@ int plan_scatter(size_t rows, size_t k, size_t cols, int dtype, apk_plan* p) {
     return APK_OK;
 }
 
+// the caller holds the context (CallScope).  scratch: one 128-byte line per row, zero on entry (the kernel re-arms it).
+int argmax_locked(apk_ctx* c, const float* logits, size_t rows, size_t n, uint32_t* out, void* scratch) {
+    if (rows == 0) return APK_OK;
+    if (!logits || !out || !scratch) return fail(APK_DECLINE_NULL, "apk_argmax_rows: NULL tensor");
+    if (n == 0 || n > 0xffffffffu || rows > (1u << 20)) return fail(APK_DECLINE_SHAPE, "apk_argmax_rows: sizes out of range");
+    if (int rc = set_device(c)) return rc;
+    // Enough workgroups per row to spread a vocabulary-sized row over the chip, and no more: the parts of a row merge
+    // through two atomics on one cache line, which serialise (38 parts of 4 K logits per row: 9.4 us for 64 x 151 936
+    // logits; 19 parts of 8 K logits, workgroups of 512 lanes: 9.2; 128 parts: 16).  A few rows keep the finer split.
+    const unsigned block = rows >= 16 ? 512 : 256;
+    size_t parts = (n + 16 * block - 1) / (16 * block);  // one pass of four 16-byte loads per lane
+    if (parts > 64) parts = 64;
+    if (parts < 1) parts = 1;
+    while (parts > 1 && rows * parts > 8192) parts /= 2;
+    uint64_t n64 = n;
+    int parts_i = (int)parts;
+    void* args[] = {&logits, &n64, &parts_i, &scratch, &out};
+    return launch_keyed(c, OP_ARGMAX, 0, [] { return std::string("apk_argmax_rows"); }, (unsigned)(rows * parts), block, 0, args);
+}
+
 }  // namespace
 
 #pragma GCC visibility push(default)
@@ -1377,8 +1397,7 @@ int apk_argmax_rows(apk_ctx* c, const float* logits, size_t rows, size_t n, uint
     if (!c) return fail(APK_DECLINE_NULL, "apk_argmax_rows: ctx is NULL");
     CallScope s(c);
     if (rows == 0) return APK_OK;
-    if (!logits || !out) return fail(APK_DECLINE_NULL, "apk_argmax_rows: NULL tensor");
-    if (n == 0 || n > 0xffffffffu || rows > (1u << 20)) return fail(APK_DECLINE_SHAPE, "apk_argmax_rows: sizes out of range");
+    if (rows > (1u << 20)) return fail(APK_DECLINE_SHAPE, "apk_argmax_rows: sizes out of range");
     if (int rc = set_device(c)) return rc;
     if (rows > c->argmax_rows_cap) {
         if (c->capturing || c->graphs_with_argmax)
@@ -1394,17 +1413,8 @@ int apk_argmax_rows(apk_ctx* c, const float* logits, size_t rows, size_t n, uint
         HIP_TRY(hipMemsetAsync(c->argmax_scratch, 0, cap * 128, c->stream));
         c->argmax_rows_cap = cap;
     }
-    // enough workgroups per row to spread a vocabulary-sized row over the chip: ~4 K logits each
-    // (one pass of 4 16-byte loads per lane)
-    size_t parts = (n + 4095) / 4096;
-    if (parts > 64) parts = 64;
-    if (parts < 1) parts = 1;
-    while (parts > 1 && rows * parts > 8192) parts /= 2;
-    uint64_t n64 = n;
-    int parts_i = (int)parts;
-    void* args[] = {&logits, &n64, &parts_i, &c->argmax_scratch, &out};
     if (c->capturing) c->capture_argmax = true;
-    return launch_keyed(c, OP_ARGMAX, 0, [] { return std::string("apk_argmax_rows"); }, (unsigned)(rows * parts), 256, 0, args);
+    return argmax_locked(c, logits, rows, n, out, c->argmax_scratch);
 }
 
 /* ------------------------------------------------------------- launch plans */

@@ -8,47 +8,62 @@
 // workgroup of a row (counted next to it) writes out[row] and re-arms both words.
 // scratch: one 128-byte line per row (word 0: running best, word 1: arrivals), so the
 // atomics of different rows never share a cache line.
-extern "C" __global__ __launch_bounds__(256) void apk_argmax_rows(const float* logits, uint64_t n, int parts,
-                                                                 unsigned long long* scratch, uint32_t* out) {
-    __shared__ unsigned long long wbest[4];
+// The fold costs three integer operations per logit: non-negative floats order as signed integers of their bits
+// and negative ones in reverse, so a lane keeps the signed maximum and minimum of its raw tiles, picks the maximum
+// if it is non-negative and the minimum otherwise (the lane's largest value under total_cmp either way), and finds
+// the pick's position with one more sweep over the registers, in index order, so that the last of equal values
+// wins.  (A 64-bit (key, index) compare per logit was ten operations and showed next to the stream: 8.7 us against
+// 8.0 us for 64 x 151 936 logits before the merge.)
+extern "C" __global__ __launch_bounds__(1024) void apk_argmax_rows(const float* logits, uint64_t n, int parts,
+                                                                  unsigned long long* scratch, uint32_t* out) {
+    __shared__ unsigned long long wbest[16];
     const uint32_t row = blockIdx.x / parts, part = blockIdx.x % parts;
     unsigned long long* best = scratch + (uint64_t)row * 16;
     uint32_t* done = (uint32_t*)(best + 1);
     const float* lr = logits + (uint64_t)row * n;
     unsigned long long b = 0;
-    auto fold = [&](float v, uint64_t i) {
-        const unsigned long long cand = ((unsigned long long)total_order_key(v) << 32) | (unsigned long long)i;
-        b = cand > b ? cand : b;  // equal keys: the higher index is the larger word
-    };
     uint64_t lo, hi;
     if ((n & 3) == 0) {  // rows are 16-byte aligned: 16-byte tiles, 4 loads in flight per lane
         const uint64_t ntile = n >> 2, per = (ntile + parts - 1) / parts;
         lo = (uint64_t)part * per;
         hi = min(lo + per, ntile);
-        const f32x4* lt = (const f32x4*)lr;
+        const u32x4* lt = (const u32x4*)lr;
         for (uint64_t i0 = lo + threadIdx.x; i0 < hi; i0 += 4 * blockDim.x) {
-            f32x4 t[4];
+            u32x4 t[4];
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
+            for (int j = 0; j < 4; j++) {  // a tile past the end re-reads the lane's first tile (valid logits of this part)
                 const uint64_t i = i0 + (uint64_t)j * blockDim.x;
                 t[j] = __builtin_nontemporal_load(lt + (i < hi ? i : i0));
             }
+            int32_t imax = INT32_MIN, imin = INT32_MAX;
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const uint64_t i = i0 + (uint64_t)j * blockDim.x;
-                if (i < hi) {
-                    fold(t[j].x, 4 * i);
-                    fold(t[j].y, 4 * i + 1);
-                    fold(t[j].z, 4 * i + 2);
-                    fold(t[j].w, 4 * i + 3);
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int32_t r = (int32_t)t[j][e];
+                    imax = max(imax, r);
+                    imin = min(imin, r);
                 }
+            const int32_t pick = imax >= 0 ? imax : imin;
+            uint32_t slot = 0;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {  // a re-read tile repeats an earlier index: it must not shadow a later one
+                const bool live = i0 + (uint64_t)j * blockDim.x < hi;
+#pragma unroll
+                for (int e = 0; e < 4; e++) slot = live && (int32_t)t[j][e] == pick ? (uint32_t)(4 * j + e) : slot;
             }
+            const uint64_t idx = 4 * (i0 + (uint64_t)(slot >> 2) * blockDim.x) + (slot & 3);
+            const unsigned long long cand = ((unsigned long long)total_order_key(__builtin_bit_cast(float, pick)) << 32) | idx;
+            b = cand > b ? cand : b;  // equal keys: the higher index is the larger word
         }
     } else {
         const uint64_t per = (n + parts - 1) / parts;
         lo = (uint64_t)part * per;
         hi = min(lo + per, n);
-        for (uint64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) fold(lr[i], i);
+        for (uint64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) {
+            const unsigned long long cand = ((unsigned long long)total_order_key(lr[i]) << 32) | (unsigned long long)i;
+            b = cand > b ? cand : b;
+        }
     }
     b = wave_max_u64(b);
     if ((threadIdx.x & 63) == 0) wbest[threadIdx.x >> 6] = b;

@@ -1204,20 +1204,37 @@ def test_moe_shared_expert_hits(be, ora, rows, k, n_expert, n, f16):
                                                got[2].data_ptr(), ghr.data_ptr(), ghw.data_ptr()))
 
 
-@pytest.mark.parametrize("rows,n", [(1, 151936), (64, 151936), (3, 1000), (5, 7), (2, 16384), (300, 4096)])
+@pytest.mark.parametrize("rows,n", [(1, 151936), (64, 151936), (3, 1000), (5, 7), (2, 16384), (300, 4096), (2048, 4096), (17, 8196),
+                                    (128, 262144), (40, 20000), (16, 151937)])
 def test_argmax_rows(be, ora, rows, n):
+    """(128, 262144) is the largest grid the host produces (rows * parts = 8192 workgroups, 64 arrivals per row);
+    (2048, 4096) and (17, 8196) leave lanes with re-read tiles next to live ones; (16, 151937) is a ragged row."""
     g = synth().rng(5, rows + n)
     logits = synth().normal_f32(g, (rows, n))
     if n >= 1000:
         logits[0, [17, 900, 333]] = 9.0  # exact ties: the higher index wins
         if rows > 1:
             logits[1, :] = -1.5  # all equal: the last index
+        if rows > 2:
+            logits[2, :] = -np.abs(logits[2, :])  # every value negative: the integer order of the bits is reversed
+            logits[2, [5, n - 3]] = -0.0  # the largest of them, twice
+        if rows > 4:
+            logits[3, [40, n // 2]] = np.float32(np.nan)  # +NaN is the largest value under total_cmp, the last one wins
+            logits[4, n // 3] = np.float32(np.inf)
+            logits[4, 7] = -np.float32(np.nan)  # -NaN is the smallest
+            for r in range(5, rows):  # planted ties at random places, some a workgroup part apart, some in one lane's tiles
+                m = np.float32(logits[r].max() + 1.0)
+                at = g.integers(0, n, size=3)
+                logits[r, at] = m
+                logits[r, min(int(at[0]) + 2048, n - 1)] = m
     want = [ora.argmax_last(logits[r]) for r in range(rows)]
+    x = dev(logits)
     for _ in range(2):  # the per-row scratch is re-armed by the kernel: a second call sees clean state
-        got = host(be.argmax_rows(dev(logits)))
+        got = host(be.argmax_rows(x))
         assert got.tolist() == want
     if n >= 1000:
-        assert want[0] == 900 and (rows == 1 or want[1] == n - 1)
+        assert want[0] == 900 and (rows == 1 or want[1] == n - 1) and (rows <= 2 or want[2] == n - 3)
+        assert rows <= 4 or (want[3] == n // 2 and want[4] == n // 3)
 
 
 def test_permute_declines_and_faults(be):
