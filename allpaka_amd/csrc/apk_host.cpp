@@ -5,6 +5,7 @@
 // failing, and hipModuleLaunchKernel.  No device code in this translation unit:
 // it builds with a plain host C++ compiler against the HIP runtime API.
 #include "apk_hip.h"
+#include "apk_internal.h"
 
 #include <hip/hip_runtime_api.h>
 
@@ -68,7 +69,7 @@ std::vector<std::string> all_kernel_names() {
                                   "apk_moe_permute", "apk_gather_rows", "apk_scatter_rows_t1", "apk_scatter_rows_t2", "apk_argmax_rows", "apk_add_rmsnorm_ragged_f32", "apk_add_rmsnorm_ragged_f16", "apk_copy",
                                   "apk_qknorm_rope_generic_f32", "apk_qknorm_rope_generic_f16", "apk_route_topk_wide", "apk_route_topk_e64", "apk_route_topk_e128", "apk_route_group_small_e64", "apk_route_group_small_e128",
                                   "apk_route_group_small_e256", "apk_route_group_small_e1024", "apk_add_assign_f32", "apk_add_assign_f16", "apk_softmax_rows", "apk_moe_count", "apk_moe_rank",
-                                  "apk_add_bias_rows_f32", "apk_add_bias_rows_f16", "apk_moe_shared_hits", "apk_cast_f32_f16", "apk_cast_f16_f32"};
+                                  "apk_add_bias_rows_f32", "apk_add_bias_rows_f16", "apk_moe_shared_hits", "apk_cast_f32_f16", "apk_cast_f16_f32", "apk_zero_u64"};
     for (const char* t : {"f32", "f16"}) {
         for (const char* f : {"q5k", "q6k", "q2k", "q3k", "q5_0", "f16", "f32", "bf16"}) v.push_back(std::string("apk_embed_") + f + "_" + t);
         for (int c : kAddnormTiles) v.push_back(std::string("apk_add_rmsnorm_") + t + "_c" + std::to_string(c));
@@ -114,6 +115,15 @@ struct apk_ctx {
     std::map<uintptr_t, Mapping> attached;
     std::atomic<uint64_t> calls{0}, dispatches{0}, encode_ns{0}, wait_ns{0};
 };
+
+int apk_fail(int status, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+    return status;
+}
+int apk_ctx_device(apk_ctx* c) { return c ? c->device : -1; }
 
 struct apk_graph {
     hipGraph_t graph = nullptr;
@@ -424,12 +434,18 @@ int plan_scatter(size_t rows, size_t k, size_t cols, int dtype, apk_plan* p) {
     return APK_OK;
 }
 
-// the caller holds the context (CallScope).  scratch: one 128-byte line per row, zero on entry (the kernel re-arms it).
-int argmax_locked(apk_ctx* c, const float* logits, size_t rows, size_t n, uint32_t* out, void* scratch) {
+// the caller holds the context (CallScope).  scratch: one 128-byte line per row, zero on entry (the kernel re-arms
+// it) unless clear_first asks for a fill kernel ahead of the launch.
+int argmax_locked(apk_ctx* c, const float* logits, size_t rows, size_t n, uint32_t* out, void* scratch, bool clear_first) {
     if (rows == 0) return APK_OK;
     if (!logits || !out || !scratch) return fail(APK_DECLINE_NULL, "apk_argmax_rows: NULL tensor");
     if (n == 0 || n > 0xffffffffu || rows > (1u << 20)) return fail(APK_DECLINE_SHAPE, "apk_argmax_rows: sizes out of range");
     if (int rc = set_device(c)) return rc;
+    if (clear_first) {
+        uint64_t words = (uint64_t)rows * 16;
+        void* zargs[] = {&scratch, &words};
+        if (int rc = launch(c, "apk_zero_u64", (unsigned)((words + 255) / 256), 256, 0, zargs)) return rc;
+    }
     // Enough workgroups per row to spread a vocabulary-sized row over the chip, and no more: the parts of a row merge
     // through two atomics on one cache line, which serialise (38 parts of 4 K logits per row: 9.4 us for 64 x 151 936
     // logits; 19 parts of 8 K logits, workgroups of 512 lanes: 9.2; 128 parts: 16).  A few rows keep the finer split.
@@ -481,6 +497,7 @@ int apk_init(int device, apk_ctx** out) {
     c->device = device;
     int rc = [&]() -> int {
         HIP_TRY(hipSetDevice(device));
+        if (int rs = apk_noalloc_setup(device)) return rs;  // the address of the static scratch of apk_argmax_rows_noalloc on this device
         HIP_TRY(hipModuleLoadData(&c->module, apk_kernels_co));
         for (const std::string& name : all_kernel_names()) {
             hipFunction_t f = nullptr;
@@ -1414,7 +1431,7 @@ int apk_argmax_rows(apk_ctx* c, const float* logits, size_t rows, size_t n, uint
         c->argmax_rows_cap = cap;
     }
     if (c->capturing) c->capture_argmax = true;
-    return argmax_locked(c, logits, rows, n, out, c->argmax_scratch);
+    return argmax_locked(c, logits, rows, n, out, c->argmax_scratch, false);
 }
 
 /* ------------------------------------------------------------- launch plans */
@@ -1480,3 +1497,11 @@ int apk_copy(apk_ctx* c, const void* src, void* dst, size_t bytes) {
 
 }  // extern "C"
 #pragma GCC visibility pop
+
+// (hidden: shared with apk_noalloc.hip, not part of the C ABI)
+// The launch both argmax entries share; scratch: 128 bytes per row.
+int apk_argmax_launch(apk_ctx* c, const float* logits, size_t rows, size_t n, uint32_t* out, void* scratch, bool clear_first) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_argmax_rows: ctx is NULL");
+    CallScope s(c);
+    return argmax_locked(c, logits, rows, n, out, scratch, clear_first);
+}

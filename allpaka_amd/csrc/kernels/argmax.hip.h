@@ -83,3 +83,10 @@ extern "C" __global__ __launch_bounds__(1024) void apk_argmax_rows(const float* 
         }
     }
 }
+
+// Zero fill of 8-byte words (the scratch lines of apk_argmax_rows_noalloc ahead of its launch: a fill kernel, not a
+// memset, so that the call can sit inside a recording).
+extern "C" __global__ __launch_bounds__(256) void apk_zero_u64(unsigned long long* p, uint64_t n) {
+    const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0ull;
+}

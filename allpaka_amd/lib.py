@@ -78,6 +78,7 @@ SYMBOLS = {
     "apk_scatter_rows": (_i, [_vp, _vp, _vp, _sz, _sz, _sz, _sz, _vp, _i]),
     "apk_moe_combine_add_rmsnorm": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _sz, _sz, _f, _i]),
     "apk_argmax_rows": (_i, [_vp, _vp, _sz, _sz, _vp]),
+    "apk_argmax_rows_noalloc": (_i, [_vp, _vp, _sz, _sz, _vp]),
     "apk_copy": (_i, [_vp, _vp, _vp, _sz]),
     "apk_rope_inv_freq": (_i, [_sz, _f, _vp]),
     "apk_route_group": (_i, [_vp, _vp, _vp, _sz, _sz, _sz, _i, _f, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),

@@ -387,6 +387,14 @@ int apk_moe_combine_add_rmsnorm(apk_ctx* ctx, void* x, const void* flat, const u
  * Uses a small per-context scratch (128 bytes per row, allocated on first use). */
 int apk_argmax_rows(apk_ctx* ctx, const float* logits, size_t rows, size_t n, uint32_t* out);
 
+/* apk_argmax_rows for callers that cannot allocate: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc.  No counterpart in the reference (its hosts allocate their arenas up front).  Same result
+ * as apk_argmax_rows; allocates nothing, ever: the 128 bytes of scratch per row live in a static device array
+ * of the library, 2048 rows = 256 KiB per GPU, held until the process ends.  More than 2048 rows are declined
+ * (APK_DECLINE_SHAPE).  May be recorded (apk_capture_begin .. _end).  Every call on a GPU shares that GPU's array:
+ * calls that overlap on one GPU -- two contexts, or one context from two host threads without its lock -- race. */
+int apk_argmax_rows_noalloc(apk_ctx* ctx, const float* logits, size_t rows, size_t n, uint32_t* out);
+
 /* dst = src, `bytes` a multiple of 16: the plain stream kernel the bandwidth
  * figures of the other kernels are calibrated against. */
 int apk_copy(apk_ctx* ctx, const void* src, void* dst, size_t bytes);
