@@ -49,6 +49,8 @@ def _dt(t):
 def _ptr(t):
     if t is None:
         return None
+    if isinstance(t, int):  # a device address from Backend.resolve
+        return t
     assert t.is_cuda and t.is_contiguous(), "device-resident contiguous tensors only"
     return t.data_ptr()
 
@@ -89,6 +91,45 @@ class Backend:
         f = C.c_uint32()
         check(self.L.apk_take_faults(self.h, C.byref(f)))
         return f.value
+
+    # ---- ownership: gpu::attach / detach / resolve_w (gpu/stub.rs:37-41, gpu/cuda/runtime/select.rs:80-84)
+    @staticmethod
+    def _host_range(a):
+        assert a.flags["C_CONTIGUOUS"], "a contiguous host array"
+        return a.ctypes.data, a.nbytes
+
+    def attach(self, mapping):
+        """gpu::attach(mapping) -> bool: the host array's bytes are copied to the device once and keyed by host address;
+        the same mapping again adds an owner, a range inside an attached one needs no copy."""
+        p, n = self._host_range(mapping)
+        rc = self.L.apk_attach(self.h, p, n)
+        if rc < 0:
+            check(rc)
+        return rc == 0
+
+    def detach(self, mapping):
+        """gpu::detach(mapping): drops one owner; silent when the mapping was not attached.  Raises Declined while a
+        recorded graph is alive (graphs bake in device addresses)."""
+        p, n = self._host_range(mapping)
+        rc = self.L.apk_detach_range(self.h, p, n)
+        if rc not in (0, _l.DECLINE_NOT_ATTACHED):
+            check(rc)
+
+    def owners(self, mapping):
+        p, n = self._host_range(mapping)
+        v = C.c_size_t()
+        check(self.L.apk_attached_owners(self.h, p, n, C.byref(v)))
+        return v.value
+
+    def resolve(self, host_slice):
+        """resolve_w: the device address of a host array inside an attached mapping, or None for foreign memory."""
+        p, n = self._host_range(host_slice)
+        dev = C.c_void_p()
+        rc = self.L.apk_resolve(self.h, p, n, C.byref(dev))
+        if rc == _l.DECLINE_NOT_ATTACHED:
+            return None
+        check(rc)
+        return dev.value
 
     def _enter(self):
         # torch owns the buffers and fills them on its own stream
@@ -518,6 +559,26 @@ class QuantMat:
         if rb * n_out != data.numel() * data.element_size():
             raise ValueError(f"{n_out}x{n_in} needs {rb * n_out} bytes, got {data.numel() * data.element_size()}")
         self.b, self.data, self.ty, self.n_out, self.n_in, self.row_bytes = backend, data, ty, n_out, n_in, rb
+
+    @classmethod
+    def from_mapping(cls, backend, host_bytes, ty, n_out, n_in):
+        """QuantMat::new over a borrowed slice of an attached mapping (`data: &'a [u8]`, quantmat/mod.rs:39-66): the
+        table is used where attach put it, named by its host address.  Foreign memory raises Declined, as the
+        reference's accelerator declines it (its caller then runs the CPU path)."""
+        ty = int(ty)
+        rb = backend.L.apk_row_bytes(ty, n_in)
+        if ty < 0 or ty > 9:
+            raise ValueError(f"unsupported ggml type {ty}")
+        if rb == 0:
+            raise ValueError(f"row length {n_in} is not a whole number of blocks")
+        if rb * n_out != host_bytes.nbytes:
+            raise ValueError(f"{n_out}x{n_in} needs {rb * n_out} bytes, got {host_bytes.nbytes}")
+        dev = backend.resolve(host_bytes)
+        if dev is None:
+            raise Declined(_l.DECLINE_NOT_ATTACHED, "the table is not inside an attached mapping")
+        self = cls.__new__(cls)
+        self.b, self.data, self.ty, self.n_out, self.n_in, self.row_bytes = backend, dev, ty, n_out, n_in, rb
+        return self
 
     def row(self, j, dtype=torch.float32):
         out = torch.empty(self.n_in, dtype=dtype, device=self.b.device)

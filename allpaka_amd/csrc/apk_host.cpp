@@ -54,6 +54,7 @@ uint64_t now_ns() {
 struct Mapping {
     void* dev;
     size_t len;
+    size_t owners;  // attaches of exactly this (base, len) not yet detached
 };
 
 // Every kernel of the embedded code object, resolved once at apk_init so that a
@@ -111,6 +112,7 @@ struct apk_ctx {
     size_t permute_counts_cap = 0;       // in u32
     bool capture_permute = false;
     size_t graphs_with_permute = 0;
+    size_t live_graphs = 0;  // recorded graphs not yet destroyed: they hold device addresses, also inside attached mappings
     std::mutex mu;
     std::map<uintptr_t, Mapping> attached;
     std::atomic<uint64_t> calls{0}, dispatches{0}, encode_ns{0}, wait_ns{0};
@@ -618,12 +620,29 @@ int apk_d2h(apk_ctx* c, void* host_dst, const void* dev_src, size_t bytes) {
     return APK_OK;
 }
 
+// gpu::attach / detach keep the reference's ownership rules (gpu/cuda/runtime/device.rs:588-621): a mapping is keyed
+// by (host address, length) and counts its owners; attaching a range that lies inside an attached mapping succeeds
+// without a copy and without a count; the last detach of a key frees the device copy.  A range that overlaps an
+// attached mapping without lying inside it is declined (the two copies could name one host address twice).
 int apk_attach(apk_ctx* c, const void* host_base, size_t len) {
     if (!c || !host_base || !len) return fail(APK_DECLINE_NULL, "apk_attach: NULL or empty mapping");
     std::lock_guard<std::mutex> lock(c->mu);
     NOT_WHILE_CAPTURING(c, "apk_attach");
     if (int rc = set_device(c)) return rc;
-    if (c->attached.count((uintptr_t)host_base)) return APK_OK;  // already resident
+    const uintptr_t b = (uintptr_t)host_base;
+    if (b + len < b) return fail(APK_DECLINE_SHAPE, "apk_attach: the range wraps the address space");
+    auto same = c->attached.find(b);
+    if (same != c->attached.end() && same->second.len == len) {
+        same->second.owners++;
+        return APK_OK;  // already resident: one more owner
+    }
+    for (const auto& kv : c->attached) {
+        const uintptr_t s0 = kv.first, s1 = kv.first + kv.second.len;
+        if (b >= s0 && b + len <= s1) return APK_OK;  // inside an attached mapping: no copy, not counted
+        if (b < s1 && s0 < b + len)
+            return fail(APK_DECLINE_SHAPE, "apk_attach: [%p, +%zu) overlaps the attached mapping [%p, +%zu) without lying inside it",
+                        host_base, len, (void*)s0, kv.second.len);
+    }
     void* dev = nullptr;
     HIP_TRY(hipMalloc(&dev, len));
     hipError_t e = hipMemcpy(dev, host_base, len, hipMemcpyHostToDevice);
@@ -631,21 +650,34 @@ int apk_attach(apk_ctx* c, const void* host_base, size_t len) {
         (void)hipFree(dev);
         return hip_fail(e, "apk_attach: hipMemcpy");
     }
-    c->attached[(uintptr_t)host_base] = Mapping{dev, len};
+    c->attached[b] = Mapping{dev, len, 1};
     return APK_OK;
 }
-int apk_detach(apk_ctx* c, const void* host_base) {
+// Drops one owner of the mapping attached as exactly (host_base, len); len 0 names whatever mapping starts at
+// host_base.  The last owner frees the device copy, after the stream has drained.  The reference drops its own
+// recorded graphs at that point (they bake in device addresses, device.rs:604-621); here recorded graphs belong to
+// the caller, so the last detach is declined while any is alive: destroy them first.
+int apk_detach_range(apk_ctx* c, const void* host_base, size_t len) {
     if (!c) return fail(APK_DECLINE_NULL, "apk_detach: ctx is NULL");
     std::lock_guard<std::mutex> lock(c->mu);
     NOT_WHILE_CAPTURING(c, "apk_detach");
     auto it = c->attached.find((uintptr_t)host_base);
-    if (it == c->attached.end()) return fail(APK_DECLINE_NOT_ATTACHED, "apk_detach: mapping is not attached");
+    if (it == c->attached.end() || (len && it->second.len != len))
+        return fail(APK_DECLINE_NOT_ATTACHED, "apk_detach: no mapping was attached as [%p, +%zu)", host_base, len);
+    if (it->second.owners > 1) {
+        it->second.owners--;
+        return APK_OK;
+    }
+    if (c->live_graphs)
+        return fail(APK_DECLINE_CAPTURE, "apk_detach: %zu recorded graph(s) may hold addresses inside the mapping (destroy them first)",
+                    c->live_graphs);
     if (int rc = set_device(c)) return rc;
     HIP_TRY(hipStreamSynchronize(c->stream));
     HIP_TRY(hipFree(it->second.dev));
     c->attached.erase(it);
     return APK_OK;
 }
+int apk_detach(apk_ctx* c, const void* host_base) { return apk_detach_range(c, host_base, 0); }
 int apk_resolve(apk_ctx* c, const void* host_ptr, size_t len, void** dev_out) {
     if (!c || !dev_out) return fail(APK_DECLINE_NULL, "apk_resolve: NULL argument");
     std::lock_guard<std::mutex> lock(c->mu);
@@ -660,6 +692,14 @@ int apk_resolve(apk_ctx* c, const void* host_ptr, size_t len, void** dev_out) {
     }
     *dev_out = nullptr;
     return fail(APK_DECLINE_NOT_ATTACHED, "apk_resolve: foreign memory (not inside an attached mapping)");
+}
+// gpu::is_attached for one mapping: the owners of the mapping attached as exactly (host_base, len); 0: not attached.
+int apk_attached_owners(apk_ctx* c, const void* host_base, size_t len, size_t* owners) {
+    if (!c || !owners) return fail(APK_DECLINE_NULL, "apk_attached_owners: NULL argument");
+    std::lock_guard<std::mutex> lock(c->mu);
+    auto it = c->attached.find((uintptr_t)host_base);
+    *owners = (it != c->attached.end() && it->second.len == len) ? it->second.owners : 0;
+    return APK_OK;
 }
 
 int apk_timer_begin(apk_ctx* c) {
@@ -729,6 +769,7 @@ int apk_capture_end(apk_ctx* c, apk_graph** out) {
     if (gr->uses_argmax) c->graphs_with_argmax++;
     gr->uses_permute = c->capture_permute;
     if (gr->uses_permute) c->graphs_with_permute++;
+    c->live_graphs++;
     *out = gr;
     return APK_OK;
 }
@@ -769,6 +810,7 @@ int apk_graph_destroy(apk_ctx* c, apk_graph* g) {
     HIP_TRY(hipStreamSynchronize(c->stream));  // a replay may still be running
     if (g->uses_argmax && c->graphs_with_argmax) c->graphs_with_argmax--;
     if (g->uses_permute && c->graphs_with_permute) c->graphs_with_permute--;
+    if (c->live_graphs) c->live_graphs--;
     if (g->exec) (void)hipGraphExecDestroy(g->exec);
     if (g->graph) (void)hipGraphDestroy(g->graph);
     delete g;

@@ -48,6 +48,8 @@ SYMBOLS = {
     "apk_d2h": (_i, [_vp, _vp, _vp, _sz]),
     "apk_attach": (_i, [_vp, _vp, _sz]),
     "apk_detach": (_i, [_vp, _vp]),
+    "apk_detach_range": (_i, [_vp, _vp, _sz]),
+    "apk_attached_owners": (_i, [_vp, _vp, _sz, C.POINTER(_sz)]),
     "apk_resolve": (_i, [_vp, _vp, _sz, C.POINTER(_vp)]),
     "apk_timer_begin": (_i, [_vp]),
     "apk_timer_end": (_i, [_vp, C.POINTER(_f)]),

@@ -80,6 +80,27 @@ template <typename T> class Dev {
     size_t n_;
 };
 
+// The accelerator surface's ownership calls (gpu/stub.rs:37-41; gpu/cuda/mod.rs:41-63): a host weight mapping is
+// copied to device memory once and weights are then named by their host address inside it.
+namespace gpu {
+// gpu::attach(mapping) -> bool: false where the reference returns false (no device, or the range overlaps another).
+inline bool attach(const uint8_t* mapping, size_t len) { return apk_attach(Gpu::get().ctx(), mapping, len) == APK_OK; }
+// gpu::detach(mapping): releases one attach of exactly this mapping; silent when it was not attached, as the reference.
+inline void detach(const uint8_t* mapping, size_t len) { (void)apk_detach_range(Gpu::get().ctx(), mapping, len); }
+// owners of exactly this mapping (0: not attached)
+inline size_t owners(const uint8_t* mapping, size_t len) {
+    size_t n = 0;
+    check(apk_attached_owners(Gpu::get().ctx(), mapping, len, &n));
+    return n;
+}
+// resolve_w (gpu/cuda/runtime/select.rs:80-84): the device address of a host slice inside an attached mapping, or
+// nullptr for foreign memory.
+inline const void* resolve(const void* host, size_t len) {
+    void* dev = nullptr;
+    return apk_resolve(Gpu::get().ctx(), host, len, &dev) == APK_OK ? dev : nullptr;
+}
+}  // namespace gpu
+
 namespace ops {
 
 // ops::rmsnorm(x, weight, eps): in place over one row (norm.rs:115).
@@ -245,7 +266,23 @@ class QuantMat {
         if (rb == 0) throw Error("row length is not a whole number of blocks");
         if (rb * n_out != data.size()) throw Error("byte count does not match n_out x n_in");
         dev_.reset(new Dev<uint8_t>(data.data(), data.size()));
+        table_ = dev_->ptr();
     }
+    // QuantMat::new over a borrowed slice of the model file (quantmat/mod.rs:39-66: `data: &'a [u8]`).  Bytes inside
+    // an attached mapping are used where they already are on the device (resident() is true, nothing is copied); a
+    // slice of foreign memory -- the same bytes on the heap, say -- gets a device copy of its own.
+    QuantMat(const uint8_t* data, size_t bytes, GgmlType ty, size_t n_out, size_t n_in) : ty_((int)ty), n_out_(n_out), n_in_(n_in) {
+        const size_t rb = apk_row_bytes(ty_, n_in);
+        if (ty_ < 0 || ty_ > 9) throw Error("unsupported ggml type");
+        if (rb == 0) throw Error("row length is not a whole number of blocks");
+        if (rb * n_out != bytes) throw Error("byte count does not match n_out x n_in");
+        table_ = gpu::resolve(data, bytes);
+        if (!table_) {
+            dev_.reset(new Dev<uint8_t>(data, bytes));
+            table_ = dev_->ptr();
+        }
+    }
+    bool resident() const { return !dev_; }  // the table lives inside an attached mapping
     std::vector<float> row(size_t j) const {
         std::vector<float> out(n_in_);
         row_into(j, out);
@@ -256,7 +293,7 @@ class QuantMat {
         if (dst.size() != n_in_) throw Error("row_into destination has the wrong length");
         const uint32_t id = (uint32_t)j;
         Dev<float> dout(n_in_);
-        check(apk_embed_rows_host_ids(Gpu::get().ctx(), ty_, dev_->ptr(), n_out_, n_in_, &id, 1, dout.ptr(), APK_F32));
+        check(apk_embed_rows_host_ids(Gpu::get().ctx(), ty_, table_, n_out_, n_in_, &id, 1, dout.ptr(), APK_F32));
         dout.read_back(dst.data());
     }
     // rows [row0, row0 + count) as f32, one launch, no id list (the same rows as row_into in a loop)
@@ -264,7 +301,7 @@ class QuantMat {
         std::vector<float> out(count * n_in_);
         if (count == 0) return out;
         Dev<float> dout(out.size());
-        check(apk_dequant_rows(Gpu::get().ctx(), ty_, dev_->ptr(), n_out_, n_in_, row0, count, dout.ptr(), APK_F32));
+        check(apk_dequant_rows(Gpu::get().ctx(), ty_, table_, n_out_, n_in_, row0, count, dout.ptr(), APK_F32));
         dout.read_back(out.data());
         return out;
     }
@@ -272,7 +309,8 @@ class QuantMat {
   private:
     int ty_;
     size_t n_out_, n_in_;
-    std::unique_ptr<Dev<uint8_t>> dev_;
+    std::unique_ptr<Dev<uint8_t>> dev_;  // the table's own device copy, when it is not inside an attached mapping
+    const void* table_ = nullptr;
 };
 
 // model::route_gated(logits, k, gating, norm, scale, bias) -> best-first (expert, weight) (moe.rs:601-616).

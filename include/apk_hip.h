@@ -119,12 +119,23 @@ int apk_free(apk_ctx* ctx, void* dev);
 /* Stream-ordered copies; the host buffer must stay valid until apk_sync. */
 int apk_h2d(apk_ctx* ctx, void* dev_dst, const void* host_src, size_t bytes);
 int apk_d2h(apk_ctx* ctx, void* host_dst, const void* dev_src, size_t bytes);
-/* gpu::attach(mapping) / detach (gpu/stub.rs:37-41): copies a host weight mapping
- * to device memory and keys it by host address, so weights are then named by
- * their host address inside the mapping (gpu/cuda/runtime/select.rs:80-84). */
+/* gpu::attach(mapping) / detach (gpu/stub.rs:37-41): copies a host weight mapping to device memory and keys it by
+ * host address, so weights are then named by their host address inside the mapping
+ * (gpu/cuda/runtime/select.rs:80-84).  The reference's ownership rules (gpu/cuda/runtime/device.rs:588-621): a
+ * mapping is keyed by (host_base, len) and counts its owners -- attaching the same key again adds an owner, no
+ * copy; a range inside an attached mapping succeeds without a copy and without a count; a range that overlaps one
+ * without lying inside it is declined (APK_DECLINE_SHAPE).  apk_detach_range drops one owner of exactly that key
+ * (apk_detach: of whatever mapping starts at host_base); the last owner frees the device copy after the stream has
+ * drained.  Unknown keys are APK_DECLINE_NOT_ATTACHED.  Where the reference drops its own recorded graphs on the
+ * last detach, recorded graphs here belong to the caller: while any apk_graph is alive the last detach is declined
+ * (APK_DECLINE_CAPTURE) -- destroy the graphs first, they bake in device addresses. */
 int apk_attach(apk_ctx* ctx, const void* host_base, size_t len);
 int apk_detach(apk_ctx* ctx, const void* host_base);
-/* Device address of a host address inside an attached mapping. */
+int apk_detach_range(apk_ctx* ctx, const void* host_base, size_t len);
+/* Owners of the mapping attached as exactly (host_base, len); 0 when it is not attached (gpu::is_attached, per mapping). */
+int apk_attached_owners(apk_ctx* ctx, const void* host_base, size_t len, size_t* owners);
+/* Device address of a host address inside an attached mapping (resolve_w, gpu/cuda/runtime/select.rs:80-84);
+ * a range that is not wholly inside one is APK_DECLINE_NOT_ATTACHED and *dev_out is NULL. */
 int apk_resolve(apk_ctx* ctx, const void* host_ptr, size_t len, void** dev_out);
 
 /* Elapsed device time between two points of the stream (hipEvent based). */

@@ -212,6 +212,35 @@ static void q8_0_is_scale_times_value() {  // crates/allpaka-gguf/src/dequant.rs
     CHECK(second.size() == 32 && second == m2.row(1));
     CHECK(throws<Declined>([&] { m2.dequant_rows(1, 2); }));
 }
+// The same bytes opened twice (crates/allpaka-backend/tests/gpu_parity.rs:139-208): inside an attached mapping the table is
+// used where it is on the device; as a heap copy it is foreign memory and gets a device copy of its own.  Owners are
+// counted per (address, length) (gpu/cuda/runtime/device.rs:588-621).
+static void weights_are_named_by_host_address_inside_an_attached_mapping() {
+    std::vector<uint8_t> file(64 + 34 * 4 + 32, 0);  // a "model file": 64 bytes of header, a 2 x 64 Q8_0 table
+    uint8_t* table = file.data() + 64;
+    for (int b = 0; b < 4; b++) {
+        table[34 * b] = 0x00; table[34 * b + 1] = 0x38;  // scale 0.5
+        for (int i = 0; i < 32; i++) table[34 * b + 2 + i] = (uint8_t)(int8_t)(b * 32 + i - 60);
+    }
+    CHECK(gpu::resolve(table, 34 * 4) == nullptr && gpu::owners(file.data(), file.size()) == 0);
+    CHECK(gpu::attach(file.data(), file.size()) && gpu::attach(file.data(), file.size()));
+    CHECK(gpu::owners(file.data(), file.size()) == 2);
+    CHECK(gpu::attach(table, 34) && gpu::owners(file.data(), file.size()) == 2);  // inside: no copy, no count
+    CHECK(!gpu::attach(file.data() + 8, file.size()));                             // runs off the end: declined
+    QuantMat resident(table, 34 * 4, GgmlType::Q8_0, 2, 64);
+    std::vector<uint8_t> heap(table, table + 34 * 4);
+    QuantMat foreign(heap.data(), heap.size(), GgmlType::Q8_0, 2, 64);
+    CHECK(resident.resident() && !foreign.resident());
+    CHECK(resident.row(1) == foreign.row(1) && resident.row(0)[0] == 0.5f * -60.0f && resident.row(1)[63] == 0.5f * 67.0f);
+    CHECK(throws<Error>([&] { QuantMat bad(table, 34 * 4 - 1, GgmlType::Q8_0, 2, 64); }));
+    CHECK((const uint8_t*)gpu::resolve(table + 34, 34) - (const uint8_t*)gpu::resolve(file.data(), 1) == 64 + 34);
+    CHECK(gpu::resolve(table, file.size()) == nullptr);  // runs off the end of the mapping
+    gpu::detach(file.data(), file.size());
+    CHECK(gpu::owners(file.data(), file.size()) == 1 && gpu::resolve(table, 34) != nullptr);
+    gpu::detach(file.data(), file.size());
+    CHECK(gpu::owners(file.data(), file.size()) == 0 && gpu::resolve(table, 34) == nullptr);
+    gpu::detach(file.data(), file.size());  // silent when nothing is attached
+}
 static void route_picks_the_top_k_and_renormalises() {  // crates/allpaka-model/tests/gpu_eligible_forward.rs:88-97
     std::vector<float> logp = {std::log(0.1f), std::log(0.5f), std::log(0.15f), std::log(0.25f)};
     auto picked = route_gated(logp, 2, Gating::Softmax, true, 1.0f, nullptr);
@@ -391,6 +420,7 @@ int main() {
         {"partial_rotary_rotates_the_head_and_passes_the_tail", partial_rotary_rotates_the_head_and_passes_the_tail},
         {"device_rope_rows_match_the_host_table", device_rope_rows_match_the_host_table},
         {"q8_0_is_scale_times_value", q8_0_is_scale_times_value},
+        {"weights_are_named_by_host_address_inside_an_attached_mapping", weights_are_named_by_host_address_inside_an_attached_mapping},
         {"route_picks_the_top_k_and_renormalises", route_picks_the_top_k_and_renormalises},
         {"moe_group_orders_rows_by_expert_then_token", moe_group_orders_rows_by_expert_then_token},
         {"gather_then_combine_is_the_weighted_sum_of_the_hits", gather_then_combine_is_the_weighted_sum_of_the_hits},
