@@ -153,13 +153,14 @@ DEV void route_group_small_body(const float* logits, const float* bias, int rows
     __shared__ uint32_t s_ids[APK_FUSED_ROUTE_TOKENS * 64];
     __shared__ float s_w[APK_FUSED_ROUTE_TOKENS * 64];
     __shared__ uint32_t wave_cnt[16], wave_used[16];
+    __shared__ float s_scores[APK_FUSED_ROUTE_TOKENS][EPL > 4 ? 64 * EPL : 1];
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     if (tid < n_expert) mask[tid] = 0u;
     __syncthreads();
     if (wv < rows) {  // uniform per wave: wave wv routes token wv
         uint32_t id;
         float w;
-        route_token<EPL>(logits + (uint64_t)wv * n_expert, bias, n_expert, k, norm, scale, sigmoid, lane, id, w);
+        route_token<EPL>(logits + (uint64_t)wv * n_expert, bias, n_expert, k, norm, scale, sigmoid, lane, id, w, s_scores[wv]);
         if (lane < k) {
             ids[wv * k + lane] = id;
             wout[wv * k + lane] = w;

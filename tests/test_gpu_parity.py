@@ -1019,12 +1019,62 @@ def test_route_topk(be, ora, rows, n_expert, k, norm, scale):
     s = synth()
     logits = s.normal_f32(s.rng(4, rows * n_expert + k), (rows, n_expert))
     want_ids, want_w = ora.route_rows(logits, k, ora.SOFTMAX, norm, scale, threads=4)
-    # the two selection orders (on probabilities as the CPU does, on raw logits as the device does) agree here
-    for r in range(rows):
-        assert np.array_equal(want_ids[r], ora.topk_by_logits(logits[r], k))
     ids, w = be.route_rows(dev(logits), k, norm=norm, scale=scale)
     assert np.array_equal(host(ids), want_ids)  # bit-exact indices
-    assert rel_err_f32(host(w), want_w) <= TOL_F32
+    # the device's scores are the reference's bit for bit (its libm's expf, its one-after-the-other sum), so the weights are too
+    assert np.array_equal(host(w).view(np.uint32), want_w.view(np.uint32))
+
+
+def test_route_where_distinct_logits_share_a_score(be, ora):
+    """The reference selects on the scores (moe.rs:552-582), so two DISTINCT logits that round to one score are a tie
+    there, broken by the lower index -- where an order taken on the raw logits puts the larger logit first.  Rows built
+    by search on the CPU: a pair inside the top-k, a pair straddling its boundary, scores that underflow to zero next to
+    masked (-inf) experts, and sigmoid scores that saturate at 1.  On each the two orders differ (asserted, or the row
+    pins nothing) and the device takes the reference's."""
+    import allpaka_amd as apk
+
+    s = synth()
+    g = s.rng(4, 4242)
+
+    def pair_with_one_score(row, i, j, lo, hi, k):
+        """row[i] = v, row[j] = the next float above v, for the first v in [lo, hi) where the oracle's scores are equal"""
+        v = np.float32(lo)
+        while v < hi:
+            row[i], row[j] = v, np.nextafter(v, np.float32(np.inf))
+            sc = row.copy()
+            ora.softmax(sc)
+            if sc[i] == sc[j] and row[i] != row[j]:
+                return
+            v = np.nextafter(np.float32(v + 1e-3), np.float32(np.inf))
+        raise AssertionError("no collapsing pair found")
+
+    rows = []
+    a = (0.3 * s.normal_f32(g, 128) - 3.0).astype(np.float32)  # everything else well below
+    a[5] = 8.0  # the pair's spacing (an ulp of 0.1) is far below an ulp of logit - max
+    pair_with_one_score(a, 10, 20, 0.05, 0.5, 8)  # both inside the top 8: the reference lists 10 before 20
+    rows.append((a, 8, ora.SOFTMAX))
+    b = (0.3 * s.normal_f32(g, 128) - 3.0).astype(np.float32)
+    b[[1, 2, 3, 4, 6, 7, 8]] = np.float32([9.0, 8.5, 8.0, 7.9, 7.8, 7.7, 7.6])  # seven sure picks
+    pair_with_one_score(b, 30, 40, 0.05, 0.5, 8)  # the eighth: index 30 by the scores, index 40 by the logits
+    rows.append((b, 8, ora.SOFTMAX))
+    c = s.normal_f32(g, 128)
+    c[0] = 200.0  # every other score underflows to zero: the rest of the picks are the lowest indices
+    c[[2, 3]] = -np.inf
+    rows.append((c, 8, ora.SOFTMAX))
+    d = s.normal_f32(g, 64)
+    d[[50, 9, 33]] = np.float32([21.0, 20.0, 30.0])  # sigmoid saturates at 1.0f for all three
+    rows.append((d, 4, ora.SIGMOID))
+    for row, k, gating in rows:
+        want_ids, want_w = ora.route_gated(row, k, gating, True, 1.0)
+        if gating == ora.SOFTMAX:
+            assert not np.array_equal(want_ids, ora.topk_by_logits(row, k)), "the row does not separate the two orders"
+        got = be.route_gated(dev(row), k, apk.Gating.Softmax if gating == ora.SOFTMAX else apk.Gating.Sigmoid, True, 1.0)
+        assert [e for e, _ in got] == list(want_ids), (list(want_ids), got)
+        assert np.array_equal(np.float32([x for _, x in got]), want_w)
+    assert list(ora.route_gated(rows[0][0], 8)[0]).index(10) + 1 == list(ora.route_gated(rows[0][0], 8)[0]).index(20)
+    assert 30 in ora.route_gated(rows[1][0], 8)[0] and 40 not in ora.route_gated(rows[1][0], 8)[0]
+    assert list(ora.route_gated(rows[2][0], 8)[0]) == [0, 1, 2, 3, 4, 5, 6, 7]
+    assert list(ora.route_gated(rows[3][0], 4, ora.SIGMOID)[0])[:3] == [9, 33, 50]
 
 
 def test_route_reference_vectors_ties_sigmoid_bias(be, ora):
@@ -1036,17 +1086,17 @@ def test_route_reference_vectors_ties_sigmoid_bias(be, ora):
             wi, ww = ora.route_gated(base, k, int(gating), norm, 1.5)
             got = be.route_gated(dev(base), k, gating, norm, 1.5)
             assert [e for e, _ in got] == list(wi)
-            assert np.allclose([x for _, x in got], ww, rtol=1e-5, atol=0)
+            assert np.array_equal(np.float32([x for _, x in got]), ww)
     bias = np.float32([0.5 + (i % 7) * 0.01 for i in range(256)])
     wi, ww = ora.route_gated(base, 8, ora.SIGMOID, True, 2.5, bias)
     got = be.route_gated(dev(base), 8, apk.Gating.Sigmoid, True, 2.5, dev(bias))
-    assert [e for e, _ in got] == list(wi) and np.allclose([x for _, x in got], ww, rtol=1e-5, atol=0)
+    assert [e for e, _ in got] == list(wi) and np.array_equal(np.float32([x for _, x in got]), ww)
     # softmax with a selection bias: selection on score + bias, weights from the scores
     lg = synth().normal_f32(synth().rng(4, 5), 128)
     b2 = synth().normal_f32(synth().rng(4, 6), 128, 0.0, 0.01)
     wi, ww = ora.route_gated(lg, 8, ora.SOFTMAX, True, 1.0, b2)
     got = be.route_gated(dev(lg), 8, apk.Gating.Softmax, True, 1.0, dev(b2))
-    assert [e for e, _ in got] == list(wi) and np.allclose([x for _, x in got], ww, rtol=1e-5, atol=0)
+    assert [e for e, _ in got] == list(wi) and np.array_equal(np.float32([x for _, x in got]), ww)
     # exact ties: the lower index wins, inside the top-k and at its boundary
     t = np.zeros(128, np.float32)
     t[[3, 9, 12, 100]] = 2.0
