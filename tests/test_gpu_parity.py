@@ -1077,6 +1077,32 @@ def test_route_where_distinct_logits_share_a_score(be, ora):
     assert list(ora.route_gated(rows[3][0], 4, ora.SIGMOID)[0])[:3] == [9, 33, 50]
 
 
+def test_router_exp_is_the_host_libm_exp_over_its_whole_range(be, ora):
+    """The device restates glibc's expf; sigmoid gating without renormalisation returns 1 / (1 + expf(-logit)) for
+    every expert (k = n), so a sweep of logits from below the underflow edge to above the overflow edge compares the two
+    implementations bit for bit: 2 M arguments, every binade of the range, the special values and the branch edges."""
+    import allpaka_amd as apk
+
+    g = synth().rng(4, 99)
+    n, rows = 64, 32768
+    mag = np.exp(g.uniform(np.log(1e-8), np.log(120.0), size=rows * n)).astype(np.float32)
+    x = (mag * np.where(g.integers(0, 2, size=rows * n) == 1, 1, -1)).astype(np.float32)
+    edges = np.float32([0.0, -0.0, 88.0, -88.0, 88.72283, 88.72284, 88.7228, -103.97, -103.972, -103.98, -103.27, -103.28, 104.0, -104.0,
+                        np.inf, -np.inf, 87.99999, -87.99999, 1e-30, -1e-30, 0.5, -0.5, 17.328, -17.328])
+    x[: len(edges)] = edges
+    x = x.reshape(rows, n)
+    ids, w = be.route_rows(dev(x), n, gating=apk.Gating.Sigmoid, norm=False, scale=1.0)
+    want_ids, want_w = ora.route_rows(x, n, ora.SIGMOID, False, 1.0, threads=4)
+    assert np.array_equal(host(ids), want_ids)
+    assert np.array_equal(host(w).view(np.uint32), want_w.view(np.uint32))
+    # softmax rows spread over the same range (arguments logit - max from 0 down to -220)
+    y = (-np.abs(x[:2048]) * 1.9).astype(np.float32)
+    y[:, 0] = 0.0
+    ids, w = be.route_rows(dev(y), 8, gating=apk.Gating.Softmax, norm=False, scale=1.0)
+    want_ids, want_w = ora.route_rows(y, 8, ora.SOFTMAX, False, 1.0, threads=4)
+    assert np.array_equal(host(ids), want_ids) and np.array_equal(host(w).view(np.uint32), want_w.view(np.uint32))
+
+
 def test_route_reference_vectors_ties_sigmoid_bias(be, ora):
     import allpaka_amd as apk
 
@@ -1366,6 +1392,120 @@ def test_scatter_rows_is_the_permutation(be, rows, k, cols, f16):
     want[hit_row.long()] = src.repeat_interleave(k, dim=0)
     assert be.take_faults() == 0
     assert torch.equal(out, want)
+
+
+def test_full_size_qknorm_rope_prefill_rows(be, ora):
+    """Qwen3-32B at T=2048, 64 q + 8 kv heads of 128, fp16, the chunk's own table rows 0..2047 (the benchmark's headline
+    launch of this op): a row subset against the oracle bit for bit, every row against the same row launched alone
+    (batch == sequential, gpu_eligible_forward.rs:33-66), plain and with the K/V cache store fused in."""
+    s = synth()
+    T, n_q, n_kv, hd = 2048, 64, 8, 128
+    gen = torch.Generator(device="cuda").manual_seed(4321)
+    q0 = torch.randn((T, n_q * hd), generator=gen, device="cuda").half()
+    k0 = torch.randn((T, n_kv * hd), generator=gen, device="cuda").half()
+    v0 = torch.randn((T, n_kv * hd), generator=gen, device="cuda").half()
+    g = s.rng(2, 2048)
+    qw, kw = s.normal_f32(g, hd, 1.0, 0.05), s.normal_f32(g, hd, 1.0, 0.05)
+    ropes = ora.rope_table(list(range(T)), ora.rope_inv_freq(hd, 1e6))
+    dqw, dkw, dropes = dev(qw), dev(kw), dev(ropes)
+    q, k = q0.clone(), k0.clone()
+    be.qknorm_rope_neox(q, k, dqw, dkw, dropes, n_q, n_kv, hd, 1e-6)
+    pick = [0, 1, 2, 511, 1024, 1777, 2046, 2047]
+    wq, wk = host(q0[pick]).copy(), host(k0[pick]).copy()
+    ora.qknorm_rope_rows(wq, wk, n_q, n_kv, hd, qw, kw, np.ascontiguousarray(ropes[pick]), 1e-6)
+    assert np.array_equal(host(q[pick]), wq) and np.array_equal(host(k[pick]), wk)  # the reference's f32 result, rounded once
+    for r in (0, 1000, 2047):  # a row of the batch equals the row launched alone
+        q1, k1 = q0[r:r + 1].clone(), k0[r:r + 1].clone()
+        be.qknorm_rope_neox(q1, k1, dqw, dkw, dropes[r:r + 1].clone(), n_q, n_kv, hd, 1e-6)
+        assert torch.equal(q1[0], q[r]) and torch.equal(k1[0], k[r])
+    # with the cache store: the same q and k, and the cache planes hold k (rotated) and v at the rows' positions
+    pos = torch.arange(T, dtype=torch.int32, device="cuda").flip(0).contiguous()  # cache row 2047 - r
+    kc = torch.zeros((T, n_kv * hd), dtype=torch.float16, device="cuda")
+    vc = torch.zeros_like(kc)
+    q2, k2 = q0.clone(), k0.clone()
+    be.qknorm_rope_kv_store(q2, k2, v0, dqw, dkw, dropes, pos, kc, vc, n_q, n_kv, hd, 1e-6)
+    assert be.take_faults() == 0
+    assert torch.equal(q2, q) and torch.equal(k2, k)
+    assert torch.equal(kc.flip(0), k) and torch.equal(vc.flip(0), v0)  # fp16 activations: both narrowings are the identity
+    wkc, wvc = np.zeros((T, n_kv * hd), np.uint16), np.zeros((T, n_kv * hd), np.uint16)
+    ora.kv_store_rows(wk, host(v0[pick]).copy(), np.array([T - 1 - r for r in pick], np.uint32), wkc, wvc)
+    rows_c = [T - 1 - r for r in pick]
+    assert np.array_equal(host(kc[rows_c]), wkc[rows_c]) and np.array_equal(host(vc[rows_c]), wvc[rows_c])
+
+
+def test_full_size_moe_swiglu_and_prefill_swiglu_f32(be, ora):
+    """The f32 SwiGLU launches of the benchmark at their exact sizes: the MoE layer's grouped [8192 x 768] (1.57 M tiles: the
+    single-wave-workgroup shape of the streaming kernels, which smaller f32 cases never reach), the whole tensor against
+    the oracle; and the dense prefill [2048 x 25600] on a row subset plus a relaunch of a slice."""
+    gen = torch.Generator(device="cuda").manual_seed(99)
+    gate = torch.randn((8192, 768), generator=gen, device="cuda")
+    up = torch.randn((8192, 768), generator=gen, device="cuda")
+    want = host(gate).copy()
+    ora.swiglu(want.reshape(-1), host(up).reshape(-1).copy())
+    be.swiglu(gate, up)
+    got = host(gate)
+    assert rel_err_f32(got, want) <= TOL_F32 and close_idiom(got, want)
+    T, F = 2048, 25600
+    gate = torch.randn((T, F), generator=gen, device="cuda")
+    up = torch.randn((T, F), generator=gen, device="cuda")
+    g0 = gate.clone()
+    be.swiglu(gate, up)
+    pick = [0, 1023, 2047]
+    want = host(g0[pick]).copy()
+    ora.swiglu(want.reshape(-1), host(up[pick]).reshape(-1).copy())
+    assert rel_err_f32(host(gate[pick]), want) <= TOL_F32 and close_idiom(host(gate[pick]), want)
+    part = g0[1500:1503].clone()
+    be.swiglu(part, up[1500:1503].clone())
+    assert torch.equal(part, gate[1500:1503])
+
+
+def _device_table(rows, row_bytes, seed, tame):
+    """A [rows x row_bytes] table of random bytes built on the device (nothing this size crosses the bus), its f16 scale
+    fields tamed to small positive values by `tame(table)`."""
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    table = torch.randint(0, 256, (rows, row_bytes), generator=gen, device="cuda", dtype=torch.uint8)
+    tame(table, gen)
+    return table
+
+
+def test_full_vocabulary_embedding_tables(be, ora):
+    """The embedding gathers at the vocabulary's real size, 151 936 rows: Q8_0 [151936 x 1024] (165 MB, configs 0 and 1) and
+    Q4_K [151936 x 5120] (438 MB, config 2), built on the device; ids include row 0 and row 151 935; only the gathered
+    table rows come back to the host, where the oracle decodes them (QuantMat::row_into, quantmat/mod.rs:75-89)."""
+    import allpaka_amd as apk
+
+    vocab = 151936
+
+    def tame_q8(t, gen):  # [d: f16][32 x i8] per 34 bytes: d = |N(0, 0.02)| / 127, some of them f16 subnormals
+        v = t.view(vocab, -1, 34)
+        d = (torch.randn((vocab, v.shape[1], 1), generator=gen, device="cuda").abs() * (0.02 / 127.0)).half()
+        v[:, :, 0:2] = d.view(torch.uint8).reshape(vocab, v.shape[1], 2)
+
+    def tame_q4k(t, gen):  # [d: f16][dmin: f16][12 scale bytes][128 nibble bytes] per 144 bytes
+        v = t.view(vocab, -1, 144)
+        d = (torch.randn((vocab, v.shape[1], 2), generator=gen, device="cuda").abs() * (0.02 / 63.0)).half()
+        v[:, :, 0:4] = d.view(torch.uint8).reshape(vocab, v.shape[1], 4)
+
+    g = synth().rng(0, 151936)
+    for fmt_name, n_in, rb, tame, T in (("Q8_0", 1024, 1088, tame_q8, 512), ("Q4K", 5120, 2880, tame_q4k, 2048)):
+        table = _device_table(vocab, rb, 7 + n_in, tame)
+        ids = g.integers(0, vocab, size=T, dtype=np.uint32)
+        ids[[0, 1, 2, T - 1]] = [0, vocab - 1, vocab - 1, 0]
+        d_ids = dev(ids)
+        qm = apk.QuantMat(be, table.view(-1), ora.FMT[fmt_name], vocab, n_in)
+        for out_dtype in (torch.float32, torch.float16):
+            out = torch.zeros((T, n_in), dtype=out_dtype, device="cuda")
+            qm.rows_into(d_ids, out)
+            picked = host(table[d_ids.long()]).reshape(-1)  # the T gathered rows as a T-row table of their own
+            want = ora.embed_rows(picked, ora.FMT[fmt_name], T, n_in, np.arange(T, dtype=np.uint32), out_f16=out_dtype == torch.float16)
+            assert np.array_equal(host(out), want), (fmt_name, out_dtype)
+        last = ora.embed_rows(host(table[vocab - 1]).reshape(-1), ora.FMT[fmt_name], 1, n_in, np.zeros(1, np.uint32))[0]
+        assert np.array_equal(host(qm.row(vocab - 1)), last)  # QuantMat::row of the table's last row
+        with pytest.raises(ValueError):  # one past the table's last row: rejected on the host, as the callers reject it
+            bad = ids.copy()
+            bad[5] = vocab
+            qm.rows_into(dev(bad), out)
+        del table, qm
 
 
 # ----------------------------------------------- full-size property checks
