@@ -46,3 +46,20 @@ def q4_k_table(g, rows, n_in):
     dd = (np.abs(g.standard_normal((rows, nsb, 2))) * 0.02 / 63.0).astype(np.float32).astype(np.float16)
     blk[:, :, 0:4] = dd.view(np.uint8).reshape(rows, nsb, 4)
     return blk.reshape(rows, nsb * 144)
+
+
+def layer_inputs(model, rows, salt=0):
+    """The inputs of one decoder layer's fused ops at `rows` tokens, f32, from one seeded generator: what both legs of the
+    benchmark run on (the device leg narrows the activations to its activation type, the CPU leg takes them as they
+    are).  x, delta [rows, hidden]; gamma1, gamma2 [hidden]; q [rows, n_q*hd], k [rows, n_kv*hd]; qw, kw [hd];
+    gate, up [rows, ffn]."""
+    m = MODELS[model]
+    g = rng(2, 1000 + salt)
+    H, hd = m["hidden"], m["head_dim"]
+    return dict(
+        x=normal_f32(g, (rows, H)), delta=normal_f32(g, (rows, H)),
+        gamma1=normal_f32(g, H, 1.0, 0.05), gamma2=normal_f32(g, H, 1.0, 0.05),
+        q=normal_f32(g, (rows, m["n_q"] * hd)), k=normal_f32(g, (rows, m["n_kv"] * hd)),
+        qw=normal_f32(g, hd, 1.0, 0.05), kw=normal_f32(g, hd, 1.0, 0.05),
+        gate=normal_f32(g, (rows, m["ffn"])), up=normal_f32(g, (rows, m["ffn"])),
+    )

@@ -29,9 +29,21 @@ sys.path.insert(0, ROOT)
 PEAK_GBS = 8000.0  # MI355X HBM3E peak
 COLD_BYTES = 640e6  # every op rotates through at least this many distinct bytes
 
-# FETCH_SIZE / WRITE_SIZE of the dominant kernel (rocprofv3 --pmc, KiB per dispatch,
-# scaled by the same counters on apk_copy of a known size); see profiles/.
-TRAFFIC_BYTES_PER_LAUNCH = 314546888
+# HBM traffic of the dominant kernel per launch (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, KiB per dispatch, scaled by
+# the same counters on apk_copy of a known size): read from the committed summary of those runs, so that the figure
+# travels with the profile it came from; None when the summary has no row for the kernel.
+TRAFFIC_PROFILE = os.path.join("profiles", "layer-ops_qwen3-32b_T2048_f16_hbm-traffic.md")
+
+
+def traffic_from_profile(kernel):
+    import re
+
+    try:
+        text = open(os.path.join(ROOT, TRAFFIC_PROFILE)).read()
+    except OSError:
+        return None
+    m = re.search(r"^\| " + re.escape(kernel) + r" \| \d+ \| \d+ \| (\d+) \|", text, re.M)
+    return int(m.group(1)) if m else None
 
 
 def main():
@@ -106,19 +118,26 @@ def main():
     H, NQ, NKV, HD, FF, EPS = m["hidden"], m["n_q"], m["n_kv"], m["head_dim"], m["ffn"], m["eps"]
     T = args.rows
     b = 2
-    gamma1 = 1 + 0.05 * randn(H, torch.float32)
-    gamma2 = 1 + 0.05 * randn(H, torch.float32)
-    qw = 1 + 0.05 * randn(HD, torch.float32)
-    kw = 1 + 0.05 * randn(HD, torch.float32)
+    # one seeded set of layer inputs (allpaka_amd/synth.py), the same values the CPU leg runs on; the device keeps
+    # them as fp16 and every pool set below is a copy of it (the pools only defeat the last-level cache)
+    lay = synth.layer_inputs("qwen3-32b", T)
+
+    def up16(a):
+        return torch.from_numpy(a).to(dev).half()
+
+    src = {name: up16(lay[name]) for name in ("x", "delta", "q", "k", "gate", "up")}
+    gamma1, gamma2 = torch.from_numpy(lay["gamma1"]).to(dev), torch.from_numpy(lay["gamma2"]).to(dev)
+    qw, kw = torch.from_numpy(lay["qw"]).to(dev), torch.from_numpy(lay["kw"]).to(dev)
     inv = torch.tensor(np.float32(m["theta"]) ** (-2.0 * np.arange(HD // 2, dtype=np.float32) / np.float32(HD)), device=dev)
     pos = torch.arange(T, dtype=torch.int32, device=dev)
     rope = torch.empty((T, HD // 2, 2), dtype=torch.float32, device=dev)
     torch.cuda.synchronize()
     apklib.check(L.apk_rope_table(h, p(pos), p(inv), T, HD // 2, p(rope)))
     sync()
-    an = pool(3 * T * H * b, lambda: dict(x=randn((T, H)), d=randn((T, H)), h=torch.empty((T, H), dtype=torch.float16, device=dev)))
-    qk = pool(T * (NQ + NKV) * HD * b, lambda: dict(q=randn((T, NQ * HD)), k=randn((T, NKV * HD))))
-    sw = pool(2 * T * FF * b, lambda: dict(gate=randn((T, FF)), up=randn((T, FF))))
+    an = pool(3 * T * H * b, lambda: dict(x=src["x"].clone(), d=src["delta"].clone(), h=torch.empty((T, H), dtype=torch.float16, device=dev)))
+    qk = pool(T * (NQ + NKV) * HD * b, lambda: dict(q=src["q"].clone(), k=src["k"].clone()))
+    sw = pool(2 * T * FF * b, lambda: dict(gate=src["gate"].clone(), up=src["up"].clone()))
+    del src
     torch.cuda.synchronize()
 
     def op_addnorm(i, gamma=gamma1, rows=T):
@@ -297,7 +316,7 @@ def main():
     # ------------------------------------------------------------ cpu baseline
     cpu = None
     if not args.no_cpu_baseline:
-        cpu = cpu_baseline(np, T, H, NQ, NKV, HD, FF, EPS)
+        cpu = cpu_baseline(np, lay, T, H, NQ, NKV, HD, FF, EPS)
 
     layer_bytes = 2 * bytes_addnorm + bytes_qkrope + bytes_swiglu
     out = {
@@ -318,7 +337,8 @@ def main():
                                "distinct buffers so every launch streams from HBM",
                    "launches_per_layer": 4, "rows": T},
         "roofline": {"bound": "hbm", "kernel": "apk_swiglu_f16", "achieved": dom["GBps"], "peak": PEAK_GBS, "unit": "GB/s",
-                     "frac": round(dom["GBps"] / PEAK_GBS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH,
+                     "frac": round(dom["GBps"] / PEAK_GBS, 4), "traffic": traffic_from_profile("apk_swiglu_f16"),
+                     "traffic_source": TRAFFIC_PROFILE,
                      "algorithmic_bytes_per_launch": dom["bytes"], "avg_launch_us": dom["us"]},
         "layer_algorithmic_bytes": int(layer_bytes),
         "layer_GBps": round(layer_bytes / us_layer_events / 1e3, 1),
@@ -333,7 +353,8 @@ def main():
 
 
 def other_shapes(args, L, h, apklib, synth, torch, gen, dev, randn, pool, p, timed, record, reps, m, qw, kw, rope):
-    """Embedding gathers, the Qwen3-0.6B f32 shapes and the MoE layer ops."""
+    """Embedding gathers, the Qwen3-0.6B f32 shapes and the MoE layer ops (inputs from a seeded device generator: these
+    shapes have no CPU leg of their own in the timed step)."""
     F16, F32 = apklib.F16, apklib.F32
     H, HD, EPS, T = m["hidden"], m["head_dim"], m["eps"], args.rows
     check = apklib.check
@@ -386,7 +407,8 @@ def other_shapes(args, L, h, apklib, synth, torch, gen, dev, randn, pool, p, tim
     ids0 = torch.randint(0, V0, (8, T0), generator=gen, device=dev, dtype=torch.int32)
     torch.cuda.synchronize()
     for rows, label in ((1, "T=1"), (T0, f"T={T0}")):
-        note = "launch-bound" if rows == 1 else None
+        # T=512 at this width moves 2.7-18 MB per launch (0.3-2.3 us at peak): still the launch, not the stream
+        note = "launch-bound"
         us = timed(lambda i: check(L.apk_embed_rows(h, apklib.FMT_Q8_0, p(q8), V0, H0, p(ids0[i % 8]), rows,
                                                     p(an0[i % len(an0)]["d"]), F32)), 200)
         record("embed_rows Q8_0->f32", f"qwen3-0.6b {label}", us, rows * (1088 + 4 + H0 * 4), note=note)
@@ -478,28 +500,34 @@ def other_shapes(args, L, h, apklib, synth, torch, gen, dev, randn, pool, p, tim
     for rows in (1, 64):
         us = timed(lambda i: check(L.apk_argmax_rows(h, p(lg[i % 17]), rows, V, p(pick))), 200)
         record("argmax_rows", f"{rows} x {V} logits f32", us, rows * V * 4 + rows * 4, note="launch-bound" if rows == 1 else None)
+    del lg, ga
+    # the plain-copy ceilings at the byte counts of the MoE layer's launches and of the greedy pick (a copy moves half
+    # of the bytes in and half out; the pick only reads, which this library has no plain kernel for)
+    cp_pool = torch.zeros(int(COLD_BYTES * 1.1), dtype=torch.uint8, device=dev)
+    torch.cuda.synchronize()
+    for name, nb in (("swiglu [8192x768] f32 and of scatter_rows", 3 * TM * K * FM * 4),
+                     ("moe_combine + add + rmsnorm", TM * K * HM * 4 + 3 * TM * HM * 4 + HM * 4 + TM * K * 8),
+                     ("argmax_rows 64 x 151936", 64 * V * 4)):
+        half = nb // 2 // 4096 * 4096
+        nset = cp_pool.numel() // (2 * half)
+        us = timed(lambda i: check(L.apk_copy(h, p(cp_pool) + (i % nset) * 2 * half, p(cp_pool) + (i % nset) * 2 * half + half, half)), reps)
+        record(f"copy (plain stream) of the bytes of {name}", f"{2 * half / 1e6:.1f} MB moved", us, 2 * half, note="ceiling at this size")
+    del cp_pool
 
 
-def cpu_baseline(np, T, H, NQ, NKV, HD, FF, EPS):
-    """The CPU oracle on the same layer chain (f32 activations: the reference's
-    CPU path has no other), whole T rows, a few repetitions (~10-20 s)."""
+def cpu_baseline(np, lay, T, H, NQ, NKV, HD, FF, EPS):
+    """The CPU oracle on the same layer chain and the same seeded inputs as the device leg (f32 activations: the
+    reference's CPU path has no other), whole T rows, a few repetitions (~10-20 s)."""
     import oracle as ora
 
     ora.build()
     cores = os.cpu_count() or 1
-    g = np.random.default_rng(7)
-    x = g.standard_normal((T, H), dtype=np.float32)
-    d = g.standard_normal((T, H), dtype=np.float32)
+    x, d, gamma = lay["x"].copy(), lay["delta"], lay["gamma1"]
     hbuf = np.empty_like(x)
-    gamma = (1 + 0.05 * g.standard_normal(H)).astype(np.float32)
-    q = g.standard_normal((T, NQ * HD), dtype=np.float32)
-    k = g.standard_normal((T, NKV * HD), dtype=np.float32)
-    qw = (1 + 0.05 * g.standard_normal(HD)).astype(np.float32)
-    kw = (1 + 0.05 * g.standard_normal(HD)).astype(np.float32)
+    q, k, qw, kw = lay["q"].copy(), lay["k"].copy(), lay["qw"], lay["kw"]
     inv = ora.rope_inv_freq(HD, 1e6)
     ropes = ora.rope_table(list(range(T)), inv)
-    gate = g.standard_normal((T, FF), dtype=np.float32)
-    up = g.standard_normal((T, FF), dtype=np.float32)
+    gate, up = lay["gate"].copy(), lay["up"]
 
     def layer():
         ora.add_assign_par(x.reshape(-1), d.reshape(-1), cores)          # prefill.rs:246
