@@ -9,14 +9,20 @@
 // the tile of its NeoX partners in the second half (EPL = 8 fp16 / 4 f32
 // elements each), so the rotation needs no cross-lane traffic, every global
 // access is a full 16-byte tile and the LPH = HD/2/EPL lanes of a head cover
-// contiguous runs.  A wave owns (row, q or k, group of HPW*ITER consecutive
-// heads), HPW = 64/LPH heads per pass: one tensor per wave means one norm
-// weight per wave and no per-element selects; the row's [sin, cos] tile and
-// the weight are loaded once and reused over ITER passes (q: ITERQ passes,
-// k: 1 pass -- under GQA k has few heads).  Waves are kept short (ITERQ 1 or 2, about
-// 4 KB of heads each): a wave that carries a row's 64 q heads in 8 passes lives as long as
-// the whole launch, and a batch a few rows beyond one resident round of such waves
-// (2061 rows instead of 2048) then takes 15 % longer; short waves fill in evenly.
+// contiguous runs.  A wave owns (row, q or k, group of HPW consecutive heads), HPW = 64/LPH
+// heads, and makes ONE pass (about 2-4 KB of heads): one tensor per wave means one norm weight
+// per wave and no per-element selects.  Longer waves were measured and dropped: two or four
+// passes per wave hold more registers per resident byte and lose 2-8 % over 1024..8192 rows, and
+// a wave that carries a row's 64 q heads in 8 passes lives as long as the whole launch, so that a
+// batch a few rows beyond one resident round (2061 rows instead of 2048) takes 15 % longer;
+// short waves fill in evenly.  (ITERQ stays a template parameter of the item; every kernel sets 1.)
+// Wave order: workgroups take items in plain index order, which the dispatcher deals round the eight
+// chiplets (XCDs, an L2 each).  The 9 waves that share a row's sin/cos line (64 + 8 heads of 128) so sit on 4-5
+// chiplets and the 1 MB table of 2048 rows is fetched 4.6 times: +5 % on the kernel's HBM reads (FETCH_SIZE).
+// Giving each chiplet rows of its own removes those reads (FETCH_SIZE then +0.3 %) and was measured slower all the
+// same: 13.7 us (rows dealt c, c + 8, ...) and 14.2 us (eight contiguous shares) against 13.5 us in plain order for
+// 2048 rows, three runs each on one machine -- the chip moving through memory as one front is worth more than
+// the 3.7 MB.  Plain order stays.
 // Arithmetic: the reference's, for both activation types (see `headstat`): f64 statistics,
 // (x as f64 * scale) as f32 * w, then the four products and two sums of the rotation,
 // not contracted.  fp16 results are that f32 result rounded once.
