@@ -20,11 +20,17 @@
  *                              pairing, cached==naive bit-identical, partial
  *                              rotary) + numpy closed form.
  *   silu/swiglu/softmax      : reference vectors + numpy closed form.
- *   route_gated/route        : reference vectors; exact ties at the k boundary
- *                              are implementation-defined in the reference
- *                              (unstable select) and are resolved here as
- *                              "lower index wins" -- that single choice is
- *                              parity unpinned by construction.
+ *   route_gated/route        : reference vectors.  Equal selection values
+ *                              (bit-equal logits, or distinct logits whose
+ *                              scores round to one f32) INSIDE the top k are
+ *                              pinned: the reference's stable sort
+ *                              (moe.rs:581) leaves them in index order, as
+ *                              here.  Equal values that STRADDLE the k
+ *                              boundary are implementation-defined in the
+ *                              reference (select_nth_unstable_by, moe.rs:579)
+ *                              and are resolved here as "lower index wins" --
+ *                              that single choice is parity unpinned by
+ *                              construction.
  *   moe_group                : brute force + invariants on small inputs.
  *   *_f16 activations        : the reference has no fp16 activations; these are
  *                              defined here as widen -> f32 reference op -> one
