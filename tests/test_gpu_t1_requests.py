@@ -361,3 +361,127 @@ def test_token_request_through_the_library_matches_the_cpu_path(case):
         if top[1] - top[0] > 1e-2 * scale:
             assert got_pick[r] == want_pick[r]
         assert got_pick[r] == int(np.flatnonzero(got_logits[r] == got_logits[r].max())[-1])  # and always its own logits' last maximum
+
+
+# ---- a batched decode step: PrefillAttnReq with `multi` and `fusion`, then GroupedFfnReq with host-built lists ---------
+def test_batched_decode_step_with_one_cache_per_session():
+    """gpu/types.rs:302-365 and :406-467.  Row i is one token of session i: its K/V go to `multi[i].cache` at
+    `multi[i].pos` and it attends over that cache's first pos + 1 positions (MultiRow); `fusion` supplies the two norms
+    and the router; the positions are staged on the device and the rotary rows are built there from them
+    (multi_stage with set_rope_inv_freq done).  The routed FFN then gets `groups`, `tok` and the CSR lists from the HOST
+    (the reference's CUDA arm rebuilds them on the host from the downloaded logits, gpu/cuda/ffn_grouped.rs:22-120), gathers
+    row-side, and folds `fused.next_norm` into the combine."""
+    import torch
+
+    import oracle as ora
+    from allpaka_amd import synth
+    from allpaka_amd.backend import Backend
+
+    ora.build()
+    g = synth.rng(4, 4242)
+    H, hd, nq, nkv, E, k_used, eff, cap, eps = 256, 64, 4, 2, 8, 2, 128, 16, 1e-6
+    kv, group, m = nkv * hd, nq // nkv, 3
+    positions = np.array([5, 0, 11], np.uint32)  # each session at its own position
+    nf = lambda shape, std=1.0, mean=0.0: synth.normal_f32(g, shape, mean, std)
+    wq, wk, wv, wo = nf((nq * hd, H), 1 / 16), nf((kv, H), 1 / 16), nf((kv, H), 1 / 16), nf((H, nq * hd), 1 / 16)
+    attn_norm, ffn_norm, next_norm = nf(H, 0.1, 1.0), nf(H, 0.1, 1.0), nf(H, 0.1, 1.0)
+    q_norm, k_norm = nf(hd, 0.1, 1.0), nf(hd, 0.1, 1.0)
+    router = nf((E, H), 1 / 16)
+    Wg, Wu, Wd = nf((E, eff, H), 1 / 16), nf((E, eff, H), 1 / 16), nf((E, H, eff), 1 / 11)
+    x0 = nf((m, H))
+    # one cache region per session: [K plane | V plane], each [cap][kv] f16, filled up to the session's position
+    caches = []
+    for p in positions:
+        c = np.zeros(2 * cap * kv, np.uint16)
+        for off in (0, cap * kv):
+            c[off : off + int(p) * kv] = synth.to_f16_bits(nf(int(p) * kv, 0.5))
+        caches.append(c)
+    inv = ora.rope_inv_freq(hd, 1e6)
+    scale = 1.0 / np.sqrt(hd)
+
+    # ---------------- CPU path
+    x = x0.copy()
+    h = np.zeros_like(x)
+    ora.add_rmsnorm_rows(x, None, h, attn_norm, eps)
+    q, k, v = (np.ascontiguousarray(h @ w.T, np.float32) for w in (wq, wk, wv))
+    ropes = ora.rope_table(positions, inv)  # PrefillAttnReq.ropes: m * rot_dim / 2 (sin, cos) pairs
+    ora.qknorm_rope_rows(q, k, nq, nkv, hd, q_norm, k_norm, ropes, eps)
+    host_caches = [c.copy() for c in caches]
+    att = np.zeros((m, nq * hd), np.float32)
+    for i in range(m):
+        kc, vc = host_caches[i][: cap * kv].reshape(cap, kv), host_caches[i][cap * kv :].reshape(cap, kv)
+        ora.kv_store_rows(k[i : i + 1], v[i : i + 1], positions[i : i + 1], kc, vc)
+        n_pos = int(positions[i]) + 1
+        kf = ora.f16_bits_to_f32(kc[:n_pos].copy()).reshape(n_pos, nkv, hd)
+        vf = ora.f16_bits_to_f32(vc[:n_pos].copy()).reshape(n_pos, nkv, hd)
+        for hq in range(nq):
+            s = (kf[:, hq // group, :] @ q[i, hq * hd : (hq + 1) * hd]) * np.float32(scale)
+            pr = np.exp(s - s.max())
+            pr /= pr.sum()
+            att[i, hq * hd : (hq + 1) * hd] = pr @ vf[:, hq // group, :]
+    ora.add_rmsnorm_rows(x, np.ascontiguousarray(att @ wo.T, np.float32), h, ffn_norm, eps)
+    logits = np.ascontiguousarray(h @ router.T, np.float32)
+    ids, w = ora.route_rows(logits, k_used, norm=True)
+    groups, tok, tok_off, hit_row, hit_w = ora.moe_group(ids, w, E)  # GroupedFfnReq.groups / tok, GroupedCombine lists
+    xe = ora.gather_rows(h, tok)
+    flat = np.zeros((tok.size, H), np.float32)
+    for e, row0, rows in groups:
+        gg = np.ascontiguousarray(xe[row0 : row0 + rows] @ Wg[e].T, np.float32)
+        uu = np.ascontiguousarray(xe[row0 : row0 + rows] @ Wu[e].T, np.float32)
+        ora.swiglu(gg, uu)
+        flat[row0 : row0 + rows] = gg @ Wd[e].T
+    ora.moe_combine_add_rmsnorm(x, flat, tok_off, hit_row, hit_w, h, next_norm, eps)
+    want_x, want_h = x, h
+
+    # ---------------- the same step through the library
+    be = Backend(0)
+    try:
+        dev = be.device
+        up = lambda a: torch.from_numpy(np.array(a, copy=True, order="C")).to(dev)
+        x = up(x0)
+        h = torch.empty_like(x)
+        be.add_rmsnorm_rows(x, None, h, up(attn_norm), eps)  # fusion.attn_norm over the resident residual rows
+        q, k, v = ((h @ up(w).T).contiguous() for w in (wq, wk, wv))
+        pos_dev = up(positions.view(np.int32))  # multi_stage: the positions, staged once for the step
+        table = be.rope_table(pos_dev, up(inv))  # ... and the rotary rows built from them on the device
+        assert np.max(np.abs(table.cpu().numpy().reshape(ropes.shape) - ropes)) <= 1e-6
+        regions = [up(c.view(np.int16)).view(torch.float16) for c in caches]  # gpu::wrap_region of every session's cache
+        att = torch.zeros((m, nq * hd), dtype=torch.float32, device=dev)
+        for i in range(m):  # one call per distinct (cache, k_off, v_off): here one row each
+            kc, vc = regions[i][: cap * kv].view(cap, kv), regions[i][cap * kv :].view(cap, kv)
+            be.attn_prologue_rows(q[i : i + 1], k[i : i + 1], v[i : i + 1], nq, nkv, hd, eps, table[i : i + 1], q_norm=up(q_norm), k_norm=up(k_norm),
+                                  cache_pos=pos_dev[i : i + 1], k_cache=kc, v_cache=vc)
+            n_pos = int(positions[i]) + 1
+            kf = kc[:n_pos].float().view(n_pos, nkv, hd).repeat_interleave(group, dim=1)
+            vf = vc[:n_pos].float().view(n_pos, nkv, hd).repeat_interleave(group, dim=1)
+            s = torch.einsum("phd,hd->hp", kf, q[i].view(nq, hd)) * scale
+            att[i] = torch.einsum("hp,phd->hd", torch.softmax(s, dim=1), vf).reshape(-1)
+        be.add_rmsnorm_rows(x, (att @ up(wo).T).contiguous(), h, up(ffn_norm), eps)  # fusion.ffn_norm
+        dev_logits = (h @ up(router).T).contiguous()  # fusion.router: what prefill_attn_block returns
+        # the host builds the lists from the downloaded logits, as the reference's CUDA arm does, and hands them over
+        ids_h, w_h = ora.route_rows(dev_logits.cpu().numpy(), k_used, norm=True)
+        groups_h, tok_h, tok_off_h, hit_row_h, hit_w_h = ora.moe_group(ids_h, w_h, E)
+        assert np.array_equal(ids_h, ids)  # the same experts as on the CPU path (the logits differ in their last bits only)
+        tok_d = up(tok_h.view(np.int32))
+        xe = be.gather_rows(h, tok_d)  # GroupedFfnReq.x / tok: the row-side permute
+        flat = torch.zeros((tok_h.size, H), dtype=torch.float32, device=dev)
+        for e, row0, rows in groups_h.tolist():
+            gg = (xe[row0 : row0 + rows] @ up(Wg[e]).T).contiguous()
+            uu = (xe[row0 : row0 + rows] @ up(Wu[e]).T).contiguous()
+            be.swiglu(gg, uu)
+            flat[row0 : row0 + rows] = gg @ up(Wd[e]).T
+        be.moe_combine_add_rmsnorm(x, flat, up(tok_off_h.view(np.int32)), up(hit_row_h.view(np.int32)), up(hit_w_h), h, up(next_norm), eps)
+        assert be.take_faults() == 0
+        got_x, got_h = x.cpu().numpy(), h.cpu().numpy()
+        got_caches = [r.view(torch.int16).cpu().numpy().view(np.uint16) for r in regions]
+    finally:
+        be.close()
+    for i in range(m):  # each session's cache: one new row at its own position, nothing else touched
+        for off in (0, cap * kv):
+            lo, hi = off + int(positions[i]) * kv, off + (int(positions[i]) + 1) * kv
+            assert np.array_equal(got_caches[i][off:lo], caches[i][off:lo]) and np.array_equal(got_caches[i][hi : off + cap * kv], caches[i][hi : off + cap * kv])
+            a, b = ora.f16_bits_to_f32(got_caches[i][lo:hi].copy()), ora.f16_bits_to_f32(host_caches[i][lo:hi].copy())
+            assert np.any(got_caches[i][lo:hi] != 0) and np.max(np.abs(a - b)) <= 2e-3 * max(1.0, float(np.max(np.abs(b))))
+    rms = lambda a: float(np.sqrt(np.mean(a.astype(np.float64) ** 2)))
+    assert np.max(np.abs(got_x - want_x)) <= 2e-3 * rms(want_x)
+    assert np.max(np.abs(got_h - want_h)) <= 2e-3 * rms(want_h)
