@@ -191,7 +191,8 @@ def main():
     # The practical ceiling at each op's size: a plain copy (one 16-byte tile per lane, out of place) moving
     # the same number of bytes.  Every launch pays a fixed ~2 us before it streams at ~6.8 TB/s, so a
     # ~76 MB op cannot reach the fraction of peak a 300 MB op does.
-    cp_pool = torch.zeros(int(COLD_BYTES * 1.1), dtype=torch.uint8, device=dev)
+    cp_pool = torch.empty(int(COLD_BYTES * 1.1) // 4 * 4, dtype=torch.uint8, device=dev)
+    cp_pool.view(torch.float32).normal_()  # not zeros: a stream of zeros runs 3-4 % faster than one of activations
     torch.cuda.synchronize()
     for name, nb in (("add_rmsnorm", bytes_addnorm), ("qknorm_rope_neox", bytes_qkrope), ("embed_rows Q4_K->f16", T * (2880 + 4 + H * 2))):
         half = nb // 2 // 4096 * 4096
@@ -503,7 +504,8 @@ def other_shapes(args, L, h, apklib, synth, torch, gen, dev, randn, pool, p, tim
     del lg, ga
     # the plain-copy ceilings at the byte counts of the MoE layer's launches and of the greedy pick (a copy moves half
     # of the bytes in and half out; the pick only reads, which this library has no plain kernel for)
-    cp_pool = torch.zeros(int(COLD_BYTES * 1.1), dtype=torch.uint8, device=dev)
+    cp_pool = torch.empty(int(COLD_BYTES * 1.1) // 4 * 4, dtype=torch.uint8, device=dev)
+    cp_pool.view(torch.float32).normal_()  # not zeros: a stream of zeros runs 3-4 % faster than one of activations
     torch.cuda.synchronize()
     for name, nb in (("swiglu [8192x768] f32 and of scatter_rows", 3 * TM * K * FM * 4),
                      ("moe_combine + add + rmsnorm", TM * K * HM * 4 + 3 * TM * HM * 4 + HM * 4 + TM * K * 8),
@@ -512,6 +514,12 @@ def other_shapes(args, L, h, apklib, synth, torch, gen, dev, randn, pool, p, tim
         nset = cp_pool.numel() // (2 * half)
         us = timed(lambda i: check(L.apk_copy(h, p(cp_pool) + (i % nset) * 2 * half, p(cp_pool) + (i % nset) * 2 * half + half, half)), reps)
         record(f"copy (plain stream) of the bytes of {name}", f"{2 * half / 1e6:.1f} MB moved", us, 2 * half, note="ceiling at this size")
+    # SwiGLU reads two streams and writes one; the same access mix with no arithmetic at all (a += b) is its nearer ceiling
+    n_sw = TM * K * FM
+    nset = cp_pool.numel() // (2 * n_sw * 4)
+    us = timed(lambda i: check(L.apk_add_assign(h, p(cp_pool) + (i % nset) * 2 * n_sw * 4, p(cp_pool) + (i % nset) * 2 * n_sw * 4 + n_sw * 4, n_sw, F32)), reps)
+    record("add_assign (two reads + one write, no arithmetic) at the size of swiglu [8192x768] f32", f"{3 * n_sw * 4 / 1e6:.1f} MB moved", us, 3 * n_sw * 4,
+           note="ceiling of this access mix")
     del cp_pool
 
 
