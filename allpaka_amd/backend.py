@@ -108,12 +108,14 @@ class Backend:
         return rc == 0
 
     def detach(self, mapping):
-        """gpu::detach(mapping): drops one owner; silent when the mapping was not attached.  Raises Declined while a
-        recorded graph is alive (graphs bake in device addresses)."""
+        """gpu::detach(mapping) -> bool: drops one owner; False (and nothing else) when the mapping was not attached.
+        The last owner frees the device copy; graphs recorded while the mapping was attached decline their replays
+        from then on (they hold the old addresses), as the reference drops its own graphs there."""
         p, n = self._host_range(mapping)
         rc = self.L.apk_detach_range(self.h, p, n)
         if rc not in (0, _l.DECLINE_NOT_ATTACHED):
             check(rc)
+        return rc == 0
 
     def owners(self, mapping):
         p, n = self._host_range(mapping)
@@ -495,10 +497,11 @@ class Backend:
 
     def moe_combine_add_rmsnorm(self, x, flat, tok_off, hit_row, hit_w, h, gamma, eps):
         """x[t] += sum over the token's hits of hit_w * flat[hit_row] (add_scaled_slice order), then
-        h = rmsnorm(x) * gamma (moe.rs:298-333 + the residual add + the next norm); h=None: no norm."""
+        h = rmsnorm(x) * gamma (moe.rs:298-333 + the residual add + the next norm); h=None: no norm.
+        tok_off=None: every token has flat.shape[0] / rows hits (no shared expert), token t's at [t*k, (t+1)*k)."""
         n = flat.shape[1]
         rows = x.numel() // n
-        assert x.numel() == rows * n and tok_off.numel() == rows + 1 and flat.dtype == x.dtype
+        assert x.numel() == rows * n and (tok_off is None or tok_off.numel() == rows + 1) and flat.dtype == x.dtype
         assert h is None or (h.numel() >= rows * n and gamma is not None and gamma.numel() == n)
         self._enter()
         check(self.L.apk_moe_combine_add_rmsnorm(self.h, _ptr(x), _ptr(flat), _ptr(tok_off), _ptr(hit_row), _ptr(hit_w),
@@ -559,12 +562,15 @@ class QuantMat:
         if rb * n_out != data.numel() * data.element_size():
             raise ValueError(f"{n_out}x{n_in} needs {rb * n_out} bytes, got {data.numel() * data.element_size()}")
         self.b, self.data, self.ty, self.n_out, self.n_in, self.row_bytes = backend, data, ty, n_out, n_in, rb
+        self.host = None
 
     @classmethod
     def from_mapping(cls, backend, host_bytes, ty, n_out, n_in):
         """QuantMat::new over a borrowed slice of an attached mapping (`data: &'a [u8]`, quantmat/mod.rs:39-66): the
-        table is used where attach put it, named by its host address.  Foreign memory raises Declined, as the
-        reference's accelerator declines it (its caller then runs the CPU path)."""
+        table is used where attach put it, named by its host address, and the address is resolved again at every call
+        (resolve_w, gpu/cuda/runtime/select.rs:80-84) -- the QuantMat takes no owner, so once the mapping is detached
+        every call raises Declined and launches nothing.  Foreign memory raises Declined, as the reference's
+        accelerator declines it (its caller then runs the CPU path)."""
         ty = int(ty)
         rb = backend.L.apk_row_bytes(ty, n_in)
         if ty < 0 or ty > 9:
@@ -577,8 +583,18 @@ class QuantMat:
         if dev is None:
             raise Declined(_l.DECLINE_NOT_ATTACHED, "the table is not inside an attached mapping")
         self = cls.__new__(cls)
-        self.b, self.data, self.ty, self.n_out, self.n_in, self.row_bytes = backend, dev, ty, n_out, n_in, rb
+        self.b, self.data, self.ty, self.n_out, self.n_in, self.row_bytes = backend, None, ty, n_out, n_in, rb
+        self.host = host_bytes
         return self
+
+    def _table(self):
+        """the table's device address for this call"""
+        if self.host is None:
+            return _ptr(self.data)
+        dev = self.b.resolve(self.host)
+        if dev is None:
+            raise Declined(_l.DECLINE_NOT_ATTACHED, "the table's mapping is no longer attached")
+        return dev
 
     def row(self, j, dtype=torch.float32):
         out = torch.empty(self.n_in, dtype=dtype, device=self.b.device)
@@ -592,7 +608,7 @@ class QuantMat:
             raise ValueError(f"row_into destination has {dst.numel()} elements, expected {self.n_in}")
         ids = (C.c_uint32 * 1)(j)
         self.b._enter()
-        check(self.b.L.apk_embed_rows_host_ids(self.b.h, self.ty, _ptr(self.data), self.n_out, self.n_in, ids, 1, _ptr(dst), _dt(dst)))
+        check(self.b.L.apk_embed_rows_host_ids(self.b.h, self.ty, self._table(), self.n_out, self.n_in, ids, 1, _ptr(dst), _dt(dst)))
         self.b.sync()
 
     def dequant_rows(self, row0, count, dtype=torch.float16):
@@ -600,7 +616,7 @@ class QuantMat:
         reference's dequant_rows_f16 ahead of a dense GEMM (gpu/cuda/runtime/gemm.rs:213-260)."""
         out = torch.empty((count, self.n_in), dtype=dtype, device=self.b.device)
         self.b._enter()
-        check(self.b.L.apk_dequant_rows(self.b.h, self.ty, _ptr(self.data), self.n_out, self.n_in, row0, count, _ptr(out), _dt(out)))
+        check(self.b.L.apk_dequant_rows(self.b.h, self.ty, self._table(), self.n_out, self.n_in, row0, count, _ptr(out), _dt(out)))
         self.b._leave()
         return out
 
@@ -612,9 +628,9 @@ class QuantMat:
             raise ValueError("destination size")
         self.b._enter()
         if embed_scale == 1.0:
-            check(self.b.L.apk_embed_rows(self.b.h, self.ty, _ptr(self.data), self.n_out, self.n_in, _ptr(ids), t, _ptr(dst), _dt(dst)))
+            check(self.b.L.apk_embed_rows(self.b.h, self.ty, self._table(), self.n_out, self.n_in, _ptr(ids), t, _ptr(dst), _dt(dst)))
         else:
-            check(self.b.L.apk_embed_rows_scaled(self.b.h, self.ty, _ptr(self.data), self.n_out, self.n_in, _ptr(ids), t,
+            check(self.b.L.apk_embed_rows_scaled(self.b.h, self.ty, self._table(), self.n_out, self.n_in, _ptr(ids), t,
                                                  embed_scale, _ptr(dst), _dt(dst)))
         self.b.sync()
         if self.b.take_faults() & _l.FAULT_TOKEN_RANGE:

@@ -17,6 +17,7 @@
 #include <cmath>
 #include <cstring>
 #include <map>
+#include <set>
 #include <mutex>
 #include <string>
 #include <unordered_map>
@@ -55,6 +56,7 @@ struct Mapping {
     void* dev;
     size_t len;
     size_t owners;  // attaches of exactly this (base, len) not yet detached
+    uint64_t serial;  // the context's clock when the copy was made (graphs recorded later may hold addresses inside it)
 };
 
 // Every kernel of the embedded code object, resolved once at apk_init so that a
@@ -112,7 +114,8 @@ struct apk_ctx {
     size_t permute_counts_cap = 0;       // in u32
     bool capture_permute = false;
     size_t graphs_with_permute = 0;
-    size_t live_graphs = 0;  // recorded graphs not yet destroyed: they hold device addresses, also inside attached mappings
+    std::set<apk_graph*> live_graphs;  // recorded graphs not yet destroyed: they hold device addresses, also inside attached mappings
+    uint64_t clock = 0;  // counts attaches that copied and recordings that ended: orders a graph against a mapping
     std::mutex mu;
     std::map<uintptr_t, Mapping> attached;
     std::atomic<uint64_t> calls{0}, dispatches{0}, encode_ns{0}, wait_ns{0};
@@ -133,6 +136,8 @@ struct apk_graph {
     size_t nodes = 0;
     bool uses_argmax = false;
     bool uses_permute = false;
+    uint64_t born = 0;   // the context's clock when the recording ended
+    bool stale = false;  // a mapping that was attached while this was recorded has been freed since: never replayed again
 };
 
 namespace {
@@ -650,13 +655,15 @@ int apk_attach(apk_ctx* c, const void* host_base, size_t len) {
         (void)hipFree(dev);
         return hip_fail(e, "apk_attach: hipMemcpy");
     }
-    c->attached[b] = Mapping{dev, len, 1};
+    c->attached[b] = Mapping{dev, len, 1, ++c->clock};
     return APK_OK;
 }
 // Drops one owner of the mapping attached as exactly (host_base, len); len 0 names whatever mapping starts at
-// host_base.  The last owner frees the device copy, after the stream has drained.  The reference drops its own
-// recorded graphs at that point (they bake in device addresses, device.rs:604-621); here recorded graphs belong to
-// the caller, so the last detach is declined while any is alive: destroy them first.
+// host_base.  The last owner frees the device copy, after the stream has drained.  A recorded graph bakes in device
+// addresses, so the reference drops its graphs at that point (device.rs:604-621: a later attach at the same host
+// address must never run on the old copy); here graphs belong to the caller, so every live graph that was recorded
+// while this mapping was attached is marked stale instead: apk_graph_launch declines it from then on, and the
+// caller records again after attaching the new file.
 int apk_detach_range(apk_ctx* c, const void* host_base, size_t len) {
     if (!c) return fail(APK_DECLINE_NULL, "apk_detach: ctx is NULL");
     std::lock_guard<std::mutex> lock(c->mu);
@@ -668,11 +675,10 @@ int apk_detach_range(apk_ctx* c, const void* host_base, size_t len) {
         it->second.owners--;
         return APK_OK;
     }
-    if (c->live_graphs)
-        return fail(APK_DECLINE_CAPTURE, "apk_detach: %zu recorded graph(s) may hold addresses inside the mapping (destroy them first)",
-                    c->live_graphs);
     if (int rc = set_device(c)) return rc;
-    HIP_TRY(hipStreamSynchronize(c->stream));
+    HIP_TRY(hipStreamSynchronize(c->stream));  // replays in flight included
+    for (apk_graph* g : c->live_graphs)
+        if (g->born > it->second.serial) g->stale = true;
     HIP_TRY(hipFree(it->second.dev));
     c->attached.erase(it);
     return APK_OK;
@@ -769,7 +775,8 @@ int apk_capture_end(apk_ctx* c, apk_graph** out) {
     if (gr->uses_argmax) c->graphs_with_argmax++;
     gr->uses_permute = c->capture_permute;
     if (gr->uses_permute) c->graphs_with_permute++;
-    c->live_graphs++;
+    gr->born = ++c->clock;
+    c->live_graphs.insert(gr);
     *out = gr;
     return APK_OK;
 }
@@ -789,6 +796,9 @@ int apk_graph_launch(apk_ctx* c, apk_graph* g) {
     if (!c || !g) return fail(APK_DECLINE_NULL, "apk_graph_launch: NULL argument");
     CallScope s(c);
     NOT_WHILE_CAPTURING(c, "apk_graph_launch");
+    if (g->stale)
+        return fail(APK_DECLINE_NOT_ATTACHED, "apk_graph_launch: a weight mapping that was attached when this graph was recorded has been "
+                                              "detached since; the graph holds its old device addresses -- record it again");
     if (int rc = set_device(c)) return rc;
     HIP_TRY(hipGraphLaunch(g->exec, c->stream));
     c->dispatches += g->nodes;
@@ -810,7 +820,7 @@ int apk_graph_destroy(apk_ctx* c, apk_graph* g) {
     HIP_TRY(hipStreamSynchronize(c->stream));  // a replay may still be running
     if (g->uses_argmax && c->graphs_with_argmax) c->graphs_with_argmax--;
     if (g->uses_permute && c->graphs_with_permute) c->graphs_with_permute--;
-    if (c->live_graphs) c->live_graphs--;
+    c->live_graphs.erase(g);
     if (g->exec) (void)hipGraphExecDestroy(g->exec);
     if (g->graph) (void)hipGraphDestroy(g->graph);
     delete g;
@@ -1425,8 +1435,12 @@ int apk_moe_combine_add_rmsnorm(apk_ctx* c, void* x, const void* flat, const uin
     const int es = elem_size(dtype);
     if (!es) return fail(APK_DECLINE_UNSUPPORTED, "apk_moe_combine_add_rmsnorm: dtype %d", dtype);
     if (rows == 0) return APK_OK;
-    if (!x || !flat || !tok_off || !hit_row || !hit_w || (h && !gamma))
+    if (!x || !flat || !hit_row || !hit_w || (h && !gamma))
         return fail(APK_DECLINE_NULL, "apk_moe_combine_add_rmsnorm: NULL tensor");
+    // no tok_off list: every token has the same number of hits, total_rows / rows of them, token t's at [t*k, (t+1)*k)
+    if (!tok_off && total_rows % rows)
+        return fail(APK_DECLINE_SHAPE, "apk_moe_combine_add_rmsnorm: without tok_off every token has total_rows / rows hits, and %zu is "
+                                       "not a multiple of %zu", total_rows, rows);
     const size_t vec = 16 / es;
     if (n == 0 || n % vec) return fail(APK_DECLINE_SHAPE, "apk_moe_combine_add_rmsnorm: n=%zu is not a multiple of %zu", n, vec);
     if (!aligned16(x) || !aligned16(flat) || (h && !aligned16(h)) || (gamma && !aligned16(gamma)))
@@ -1447,7 +1461,8 @@ int apk_moe_combine_add_rmsnorm(apk_ctx* c, void* x, const void* flat, const uin
     if (int rc = set_device(c)) return rc;
     int n_i = (int)n;
     uint32_t total32 = (uint32_t)total_rows;
-    void* args[] = {&x, &flat, &tok_off, &hit_row, &hit_w, &total32, &h, &gamma, &n_i, &eps, &c->fault_dev};
+    uint32_t uniform_k = tok_off ? 0u : (uint32_t)(total_rows / rows);
+    void* args[] = {&x, &flat, &tok_off, &hit_row, &hit_w, &total32, &h, &gamma, &n_i, &eps, &c->fault_dev, &uniform_k};
     const std::string which = std::string("apk_combine_add_rmsnorm_") + (dtype == APK_F32 ? "f32" : "f16") + "_c" + std::to_string(nch);
     return launch(c, which, (unsigned)rows, (unsigned)(waves * 64), 0, args);
 }
@@ -1456,7 +1471,9 @@ int apk_argmax_rows(apk_ctx* c, const float* logits, size_t rows, size_t n, uint
     if (!c) return fail(APK_DECLINE_NULL, "apk_argmax_rows: ctx is NULL");
     CallScope s(c);
     if (rows == 0) return APK_OK;
-    if (rows > (1u << 20)) return fail(APK_DECLINE_SHAPE, "apk_argmax_rows: sizes out of range");
+    // the argument checks come before anything is allocated or declined for the scratch's sake
+    if (!logits || !out) return fail(APK_DECLINE_NULL, "apk_argmax_rows: NULL tensor");
+    if (n == 0 || n > 0xffffffffu || rows > (1u << 20)) return fail(APK_DECLINE_SHAPE, "apk_argmax_rows: sizes out of range");
     if (int rc = set_device(c)) return rc;
     if (rows > c->argmax_rows_cap) {
         if (c->capturing || c->graphs_with_argmax)

@@ -13,14 +13,23 @@
 template <typename T, int NCH, int HB>
 DEV void combine_add_rmsnorm_body(T* x, const T* flat, const uint32_t* tok_off, const uint32_t* hit_row,
                                   const float* hit_w, uint32_t total_rows, T* h, const float* gamma, int n, float eps,
-                                  uint32_t* fault) {
+                                  uint32_t* fault, uint32_t uniform_k) {
     constexpr int VEC = io<T>::VEC;
     typedef typename stat<T>::acc_t acc_t;
     __shared__ acc_t part[16];
     const int nchunks = n / VEC;
     const uint64_t row = blockIdx.x;
     T* xr = x + row * (uint64_t)n;
-    const uint32_t h0 = tok_off[row], h1 = tok_off[row + 1];
+    // The token's hits.  Without a tok_off list every token has uniform_k hits (a routed layer without a shared
+    // expert: the list would read row * k), and the first dependent load of the chain tok_off -> hit_row -> rows is gone.
+    uint32_t h0, h1;
+    if (tok_off) {
+        h0 = tok_off[row];
+        h1 = tok_off[row + 1];
+    } else {
+        h0 = (uint32_t)row * uniform_k;
+        h1 = h0 + uniform_k;
+    }
     int cidx[NCH];
     typename io<T>::raw_t xraw[NCH];
 #pragma unroll
@@ -36,11 +45,9 @@ DEV void combine_add_rmsnorm_body(T* x, const T* flat, const uint32_t* tok_off, 
     // HB hits at a time: their row numbers and weights first (uniform for the workgroup), then
     // every tile of all HB expert rows in flight at once, then the multiply-adds in hit order (the
     // order is the contract: one rounding per hit).  Slots past the token's last hit re-read its
-    // last row (a cache hit) and add nothing.
-    for (uint32_t kb = h0; kb < h1; kb += HB) {
-        uint32_t r[HB];
-        float w[HB];
-        bool use[HB];
+    // last row (a cache hit) and add nothing.  The row numbers and weights of the first 2*HB hits (a token's eight
+    // experts) are fetched together up front, so the second batch of rows does not wait for a second index fetch.
+    auto fetch = [&](uint32_t kb, uint32_t* r, float* w, bool* use) {
         bool bad = false;
 #pragma unroll
         for (int j = 0; j < HB; j++) {
@@ -53,6 +60,8 @@ DEV void combine_add_rmsnorm_body(T* x, const T* flat, const uint32_t* tok_off, 
             r[j] = in_range ? r[j] : 0u;
         }
         if (bad && threadIdx.x == 0) atomicOr(fault, APK_FAULT_ROW_RANGE);
+    };
+    auto batch = [&](const uint32_t* r, const float* w, const bool* use) {
         typename io<T>::raw_t d[HB][NCH];
 #pragma unroll
         for (int j = 0; j < HB; j++)
@@ -70,6 +79,20 @@ DEV void combine_add_rmsnorm_body(T* x, const T* flat, const uint32_t* tok_off, 
                     for (int i = 0; i < VEC; i++) acc[c][i] = __builtin_fmaf(a[i], w[j], acc[c][i]);
                 }
             }
+        }
+    };
+    if (h1 > h0) {  // uniform
+        uint32_t r0[HB], r1[HB];
+        float w0[HB], w1[HB];
+        bool u0[HB], u1[HB];
+        fetch(h0, r0, w0, u0);
+        const bool second = h1 - h0 > (uint32_t)HB;
+        if (second) fetch(h0 + HB, r1, w1, u1);
+        batch(r0, w0, u0);
+        if (second) batch(r1, w1, u1);
+        for (uint32_t kb = h0 + 2 * HB; kb < h1; kb += HB) {
+            fetch(kb, r0, w0, u0);
+            batch(r0, w0, u0);
         }
     }
     float v[NCH][VEC];
@@ -115,8 +138,8 @@ DEV void combine_add_rmsnorm_body(T* x, const T* flat, const uint32_t* tok_off, 
 #define APK_COMBINE(T, TN, NCH)                                                                                        \
     extern "C" __global__ __launch_bounds__(1024) void apk_combine_add_rmsnorm_##TN##_c##NCH(                         \
         T* x, const T* flat, const uint32_t* tok_off, const uint32_t* hit_row, const float* hit_w, uint32_t total_rows, \
-        T* h, const float* gamma, int n, float eps, uint32_t* fault) {                                                 \
-        combine_add_rmsnorm_body<T, NCH, 4>(x, flat, tok_off, hit_row, hit_w, total_rows, h, gamma, n, eps, fault);    \
+        T* h, const float* gamma, int n, float eps, uint32_t* fault, uint32_t uniform_k) {                             \
+        combine_add_rmsnorm_body<T, NCH, 4>(x, flat, tok_off, hit_row, hit_w, total_rows, h, gamma, n, eps, fault, uniform_k); \
     }
 APK_COMBINE(float, f32, 1) APK_COMBINE(float, f32, 2) APK_COMBINE(float, f32, 4)
 APK_COMBINE(f16_t, f16, 1) APK_COMBINE(f16_t, f16, 2) APK_COMBINE(f16_t, f16, 4)

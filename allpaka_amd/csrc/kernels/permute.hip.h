@@ -154,6 +154,10 @@ DEV void route_group_small_body(const float* logits, const float* bias, int rows
     __shared__ float s_w[APK_FUSED_ROUTE_TOKENS * 64];
     __shared__ uint32_t wave_cnt[16], wave_used[16];
     __shared__ float s_scores[APK_FUSED_ROUTE_TOKENS][EPL > 4 ? 64 * EPL : 1];
+    // the widest router (1024 experts) keeps 16 tokens x 1024 scores here: 80 KiB of LDS with the tables above, more
+    // than the 64 KiB of earlier parts of the family -- this code object is built for gfx950 (160 KiB per workgroup) only
+    static_assert(sizeof(mask) + sizeof(s_row0) + sizeof(s_ids) + sizeof(s_w) + sizeof(wave_cnt) + sizeof(wave_used) +
+                      sizeof(s_scores) <= 160 * 1024, "LDS budget of a gfx950 workgroup");
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     if (tid < n_expert) mask[tid] = 0u;
     __syncthreads();

@@ -159,6 +159,9 @@ DEV void qk_item(T* base, int nheads, int g, const float* w, const float* trow, 
                 if (i < HD) *(f32x2*)(lmem + HD + i) = st_w[j];
             }
         }
+        // other lanes of this wave read these entries back below: the wave barrier keeps the compiler from moving
+        // those reads above the writes (it emits no instruction; a wave's LDS operations complete in order)
+        __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
@@ -343,8 +346,8 @@ DEV void qknorm_rope_body(T* q, T* k, const float* qw, const float* kw, const fl
 // f32 tiles: one pass per wave, constants in registers, workgroups of four waves.
 template <typename T> struct qk_shape { static constexpr bool LDSC = false; static constexpr int BLOCK = 256; };
 template <> struct qk_shape<f16_t> { static constexpr bool LDSC = true; static constexpr int BLOCK = 128; };
-// Resident waves per SIMD the compiler is to allow for (W16 for the fp16 kernels: the register ceiling that the
-// variant meets without spilling -- 80 plain or with biases, 96 with the cache store, 128 with both; f32: 128).
+// Resident waves per SIMD the compiler is to allow for: every fp16 variant is built for 6 (up to 85 registers; the
+// plain and the cache-store kernels come out at 62-71, i.e. 7-8 resident waves, none spills), the f32 variants for 4.
 #define APK_QK_OCC(T, W16) __launch_bounds__(qk_shape<T>::BLOCK) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 2 ? W16 : 4)))
 // One kernel per (norm or not, pairing, cache store, biases, type, head size).  PFX: apk_qknorm_rope
 // (a norm weight for q and / or k) or apk_rope (none for either); PN: pairs_ or nothing.  The argument lists are the

@@ -79,8 +79,9 @@ DEV void route_token(const float* lr, const float* bias, int n_expert, int k, in
         }
         // in index order, every lane the same chain of additions.  Up to 256 experts the scores come out of the lanes'
         // registers one by one (scores past n_expert are +0 and change nothing); wider routers walk the wave's own
-        // copy in LDS (in order within the wave: no barrier).
+        // copy in LDS (a wave's LDS operations complete in order; the wave barrier pins the compiler's order).
         float sum = 0.0f;
+        if constexpr (EPL > 4) __builtin_amdgcn_wave_barrier();  // the walk below reads what other lanes stored above
         if constexpr (EPL <= 4) {
 #pragma unroll
             for (int j = 0; j < EPL; j++)

@@ -85,8 +85,16 @@ template <typename T> class Dev {
 namespace gpu {
 // gpu::attach(mapping) -> bool: false where the reference returns false (no device, or the range overlaps another).
 inline bool attach(const uint8_t* mapping, size_t len) { return apk_attach(Gpu::get().ctx(), mapping, len) == APK_OK; }
-// gpu::detach(mapping): releases one attach of exactly this mapping; silent when it was not attached, as the reference.
-inline void detach(const uint8_t* mapping, size_t len) { (void)apk_detach_range(Gpu::get().ctx(), mapping, len); }
+// gpu::detach(mapping): releases one attach of exactly this mapping; silent when it was not attached, as the reference
+// (false then).  Any other status is an error of the device and is thrown: the caller must never believe a mapping
+// gone that is still resident.  The last owner frees the copy, and graphs recorded while it was attached decline
+// their replays from then on.
+inline bool detach(const uint8_t* mapping, size_t len) {
+    const int rc = apk_detach_range(Gpu::get().ctx(), mapping, len);
+    if (rc == APK_DECLINE_NOT_ATTACHED) return false;
+    check(rc);
+    return true;
+}
 // owners of exactly this mapping (0: not attached)
 inline size_t owners(const uint8_t* mapping, size_t len) {
     size_t n = 0;
@@ -269,15 +277,19 @@ class QuantMat {
         table_ = dev_->ptr();
     }
     // QuantMat::new over a borrowed slice of the model file (quantmat/mod.rs:39-66: `data: &'a [u8]`).  Bytes inside
-    // an attached mapping are used where they already are on the device (resident() is true, nothing is copied); a
-    // slice of foreign memory -- the same bytes on the heap, say -- gets a device copy of its own.
+    // an attached mapping are used where they already are on the device (resident() is true, nothing is copied) and
+    // are named by their host address, resolved again at every call (resolve_w, gpu/cuda/runtime/select.rs:80-84):
+    // the QuantMat takes no owner, so after the mapping's last detach every call throws Declined and launches nothing.
+    // A slice of foreign memory -- the same bytes on the heap, say -- gets a device copy of its own.
     QuantMat(const uint8_t* data, size_t bytes, GgmlType ty, size_t n_out, size_t n_in) : ty_((int)ty), n_out_(n_out), n_in_(n_in) {
         const size_t rb = apk_row_bytes(ty_, n_in);
         if (ty_ < 0 || ty_ > 9) throw Error("unsupported ggml type");
         if (rb == 0) throw Error("row length is not a whole number of blocks");
         if (rb * n_out != bytes) throw Error("byte count does not match n_out x n_in");
-        table_ = gpu::resolve(data, bytes);
-        if (!table_) {
+        if (gpu::resolve(data, bytes)) {
+            host_ = data;
+            host_bytes_ = bytes;
+        } else {
             dev_.reset(new Dev<uint8_t>(data, bytes));
             table_ = dev_->ptr();
         }
@@ -293,7 +305,7 @@ class QuantMat {
         if (dst.size() != n_in_) throw Error("row_into destination has the wrong length");
         const uint32_t id = (uint32_t)j;
         Dev<float> dout(n_in_);
-        check(apk_embed_rows_host_ids(Gpu::get().ctx(), ty_, table_, n_out_, n_in_, &id, 1, dout.ptr(), APK_F32));
+        check(apk_embed_rows_host_ids(Gpu::get().ctx(), ty_, table(), n_out_, n_in_, &id, 1, dout.ptr(), APK_F32));
         dout.read_back(dst.data());
     }
     // rows [row0, row0 + count) as f32, one launch, no id list (the same rows as row_into in a loop)
@@ -301,16 +313,25 @@ class QuantMat {
         std::vector<float> out(count * n_in_);
         if (count == 0) return out;
         Dev<float> dout(out.size());
-        check(apk_dequant_rows(Gpu::get().ctx(), ty_, table_, n_out_, n_in_, row0, count, dout.ptr(), APK_F32));
+        check(apk_dequant_rows(Gpu::get().ctx(), ty_, table(), n_out_, n_in_, row0, count, dout.ptr(), APK_F32));
         dout.read_back(out.data());
         return out;
     }
 
   private:
+    // the table's device address for this call: its own copy, or wherever the attached mapping holds it now
+    const void* table() const {
+        if (!host_) return table_;
+        void* dev = nullptr;
+        check(apk_resolve(Gpu::get().ctx(), host_, host_bytes_, &dev));  // Declined once the mapping is detached
+        return dev;
+    }
     int ty_;
     size_t n_out_, n_in_;
     std::unique_ptr<Dev<uint8_t>> dev_;  // the table's own device copy, when it is not inside an attached mapping
     const void* table_ = nullptr;
+    const uint8_t* host_ = nullptr;      // a borrowed slice inside an attached mapping (resolved per call)
+    size_t host_bytes_ = 0;
 };
 
 // model::route_gated(logits, k, gating, norm, scale, bias) -> best-first (expert, weight) (moe.rs:601-616).

@@ -126,9 +126,12 @@ int apk_d2h(apk_ctx* ctx, void* host_dst, const void* dev_src, size_t bytes);
  * copy; a range inside an attached mapping succeeds without a copy and without a count; a range that overlaps one
  * without lying inside it is declined (APK_DECLINE_SHAPE).  apk_detach_range drops one owner of exactly that key
  * (apk_detach: of whatever mapping starts at host_base); the last owner frees the device copy after the stream has
- * drained.  Unknown keys are APK_DECLINE_NOT_ATTACHED.  Where the reference drops its own recorded graphs on the
- * last detach, recorded graphs here belong to the caller: while any apk_graph is alive the last detach is declined
- * (APK_DECLINE_CAPTURE) -- destroy the graphs first, they bake in device addresses. */
+ * drained.  Unknown keys are APK_DECLINE_NOT_ATTACHED.  The reference drops its own recorded graphs on the last
+ * detach (they bake in device addresses, and a new file attached at the same host address must never run on the old
+ * copy: gpu/cuda/mod.rs:51-54); recorded graphs here belong to the caller, so the last detach of a mapping marks
+ * every live apk_graph that was recorded while the mapping was attached as stale: apk_graph_launch declines it
+ * (APK_DECLINE_NOT_ATTACHED, nothing launched) until it is destroyed.  Graphs recorded before the mapping was
+ * attached cannot hold its addresses and keep working. */
 int apk_attach(apk_ctx* ctx, const void* host_base, size_t len);
 int apk_detach(apk_ctx* ctx, const void* host_base);
 int apk_detach_range(apk_ctx* ctx, const void* host_base, size_t len);
@@ -163,7 +166,8 @@ int apk_capture_begin(apk_ctx* ctx);
 int apk_capture_end(apk_ctx* ctx, apk_graph** out);
 /* Ends the recording and throws it away (prefill_abort, gpu/cuda/prefill.rs:180). */
 int apk_capture_abort(apk_ctx* ctx);
-/* Enqueues one replay on the context's stream (asynchronous, ordered like an op). */
+/* Enqueues one replay on the context's stream (asynchronous, ordered like an op).  APK_DECLINE_NOT_ATTACHED for a
+ * graph recorded while a mapping was attached that has been freed since (see apk_detach_range). */
 int apk_graph_launch(apk_ctx* ctx, apk_graph* graph);
 /* Number of kernel launches one replay performs. */
 int apk_graph_nodes(apk_graph* graph, size_t* nodes);
@@ -345,8 +349,10 @@ int apk_moe_permute(apk_ctx* ctx, const uint32_t* ids, const float* w, size_t ro
  * bit; ONE launch for a decode-sized batch (rows <= 16), where the two launches
  * cost a launch latency each and the second waits for the first.  The reference's accelerators route
  * and group inside one command buffer as well (GroupedRoute of a GroupedFfnReq, gpu/types.rs:406-416,
- * :446-467; the Metal route_scatter kernel, gpu/shaders/kernels.metal:2223).  Larger batches run the
- * two entries. */
+ * :446-467; the Metal route_scatter / route_fused kernels, gpu/shaders/kernels.metal:2223-2424).  Larger
+ * batches run the two entries: a single launch whose last-arriving workgroup groups the picks was measured
+ * at 1024 tokens x 128 experts and is slower (three dependent device-scope round trips -- write-through
+ * acknowledgement, arrival count, re-read of the picks -- cost more than the second launch they replace). */
 int apk_route_group(apk_ctx* ctx, const float* logits, const float* bias, size_t rows, size_t n_expert, size_t k,
                     int norm, float scale, int sigmoid, uint32_t* ids, float* w, uint32_t* table, uint32_t* n_used,
                     uint32_t* tok, uint32_t* tok_off, uint32_t* hit_row, float* hit_w);
@@ -385,7 +391,10 @@ int apk_scatter_rows(apk_ctx* ctx, const void* src, const uint32_t* hit_row, siz
  * (model/prefill.rs:155/314); the reference's accelerators fuse the same three
  * (combine_rows_resnorm, gpu/shaders/kernels.metal:1905-1974; GroupedCombine.next_norm,
  * gpu/types.rs:429-443).  flat: [total_rows][n] expert down-projection rows of dtype;
- * tok_off/hit_row/hit_w: the CSR lists of apk_moe_permute.  h (and gamma) may be NULL:
+ * tok_off/hit_row/hit_w: the CSR lists of apk_moe_permute.  tok_off may be NULL when every token has the same
+ * number of hits (a routed layer without a shared expert: tok_off[t] would read t * k): the hits of token t are
+ * then [t * k, (t + 1) * k) with k = total_rows / rows (total_rows not a multiple of rows: APK_DECLINE_SHAPE), and
+ * the launch is faster for the dependent load it no longer makes.  h (and gamma) may be NULL:
  * combine and residual only.  A hit >= total_rows is skipped and raises APK_FAULT_ROW_RANGE. */
 int apk_moe_combine_add_rmsnorm(apk_ctx* ctx, void* x, const void* flat, const uint32_t* tok_off,
                                 const uint32_t* hit_row, const float* hit_w, size_t total_rows, void* h,

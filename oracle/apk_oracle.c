@@ -14,7 +14,13 @@
  *                              65536-code comparison against numpy float16.
  *   scale_min_k4, Q8_0, Q4_K : the reference's own known-answer vectors, plus a
  *                              second independent numpy decoder on random bytes.
- *   Q5_0/Q2_K/Q3_K/Q5_K/Q6_K : the reference's own bit-layout vectors.
+ *   Q2_K/Q3_K/Q5_K/Q6_K      : the reference's own bit-layout vectors.
+ *   Q5_0                     : the reference holds no vector for it; pinned by a
+ *                              hand-worked block (high bits at elements 0, 15,
+ *                              16, 31, one-bit and one-nibble walks) and by a
+ *                              second numpy decoder written from ggml's published
+ *                              dequantize_row_q5_0 on random bytes.
+ *   F16/BF16/F32 rows        : hand-worked bit patterns; bf16 over all 65536 codes.
  *   sum_sq/rmsnorm*          : reference vectors + numpy float64 closed form.
  *   rope_*                   : reference vectors (identity at pos 0, one-hot
  *                              pairing, cached==naive bit-identical, partial
@@ -22,15 +28,24 @@
  *   silu/swiglu/softmax      : reference vectors + numpy closed form.
  *   route_gated/route        : reference vectors.  Equal selection values
  *                              (bit-equal logits, or distinct logits whose
- *                              scores round to one f32) INSIDE the top k are
- *                              pinned: the reference's stable sort
- *                              (moe.rs:581) leaves them in index order, as
- *                              here.  Equal values that STRADDLE the k
- *                              boundary are implementation-defined in the
- *                              reference (select_nth_unstable_by, moe.rs:579)
- *                              and are resolved here as "lower index wins" --
- *                              that single choice is parity unpinned by
- *                              construction.
+ *                              scores round to one f32) are parity unpinned
+ *                              wherever they occur, unless k == n: the
+ *                              reference first runs select_nth_unstable_by
+ *                              (moe.rs:579), which leaves order[..k] in an
+ *                              unspecified order, and the stable sort that
+ *                              follows (moe.rs:581) keeps equal values in THAT
+ *                              order, not in index order.  Which of two equal
+ *                              values across the k boundary is kept, the order
+ *                              of equal picks inside the top k, and (with a
+ *                              selection bias, where equal selection values
+ *                              need not have equal scores) the summation order
+ *                              of `total` are therefore implementation-defined
+ *                              in the reference.  The oracle resolves all of
+ *                              them as "lower index first".  Without a bias
+ *                              equal picks have equal scores, so ids as a set
+ *                              inside the top k and every weight are still the
+ *                              reference's; only the order of the equal ids is
+ *                              the oracle's choice.
  *   moe_group                : brute force + invariants on small inputs.
  *   *_f16 activations        : the reference has no fp16 activations; these are
  *                              defined here as widen -> f32 reference op -> one

@@ -235,11 +235,19 @@ static void weights_are_named_by_host_address_inside_an_attached_mapping() {
     CHECK(throws<Error>([&] { QuantMat bad(table, 34 * 4 - 1, GgmlType::Q8_0, 2, 64); }));
     CHECK((const uint8_t*)gpu::resolve(table + 34, 34) - (const uint8_t*)gpu::resolve(file.data(), 1) == 64 + 34);
     CHECK(gpu::resolve(table, file.size()) == nullptr);  // runs off the end of the mapping
-    gpu::detach(file.data(), file.size());
+    CHECK(gpu::detach(file.data(), file.size()));
     CHECK(gpu::owners(file.data(), file.size()) == 1 && gpu::resolve(table, 34) != nullptr);
-    gpu::detach(file.data(), file.size());
+    CHECK(gpu::detach(file.data(), file.size()));
     CHECK(gpu::owners(file.data(), file.size()) == 0 && gpu::resolve(table, 34) == nullptr);
-    gpu::detach(file.data(), file.size());  // silent when nothing is attached
+    CHECK(!gpu::detach(file.data(), file.size()));  // silent when nothing is attached
+    // the borrowed QuantMat holds no owner: with the mapping gone it declines instead of reading freed memory,
+    // and a new file attached at the same address is what it reads next
+    CHECK(throws<Declined>([&] { resident.row(1); }));
+    CHECK(throws<Declined>([&] { resident.dequant_rows(0, 2); }));
+    for (int i = 0; i < 32; i++) table[34 * 2 + 2 + i] = (uint8_t)(int8_t)(i - 7);  // row 1, first block: new quants
+    CHECK(gpu::attach(file.data(), file.size()));
+    CHECK(resident.row(1)[0] == 0.5f * -7.0f && resident.row(1)[31] == 0.5f * 24.0f);
+    CHECK(gpu::detach(file.data(), file.size()));
 }
 static void route_picks_the_top_k_and_renormalises() {  // crates/allpaka-model/tests/gpu_eligible_forward.rs:88-97
     std::vector<float> logp = {std::log(0.1f), std::log(0.5f), std::log(0.15f), std::log(0.25f)};

@@ -90,31 +90,62 @@ def test_attach_resolve_run_detach():
         lib.check(L.apk_detach_range(h, base, total))
         assert n_owners(base, total) == 1
         lib.check(L.apk_resolve(h, base, 16, C.byref(dev)))  # still resident
-        # a recorded graph bakes in device addresses: the last detach is declined while it is alive
+        # a recorded graph bakes in device addresses; attach and detach cannot run inside a recording
         gr = C.c_void_p()
         lib.check(L.apk_capture_begin(h))
         assert L.apk_attach(h, base, total) == CAPTURE and L.apk_detach(h, base) == CAPTURE  # not inside a recording
         lib.check(L.apk_embed_rows(h, lib.FMT_Q4K, d_table, vocab, H, d_ids.data_ptr(), t, rows.data_ptr(), lib.F32))
         lib.check(L.apk_capture_end(h, C.byref(gr)))
-        assert L.apk_detach(h, base) == CAPTURE and b"graph" in L.apk_last_error()
         rows.zero_()
         torch.cuda.synchronize()
         lib.check(L.apk_graph_launch(h, gr))
         lib.check(L.apk_sync(h))
-        assert np.array_equal(rows.cpu().numpy(), want_rows)  # the mapping was still there
-        lib.check(L.apk_graph_destroy(h, gr))
-        lib.check(L.apk_detach(h, base))  # the last owner: the device copy goes
+        assert np.array_equal(rows.cpu().numpy(), want_rows)  # the mapping is still there
+        # a graph recorded before the mapping was attached again below is untouched by that mapping's detach
+        early = C.c_void_p()
+        hs.zero_()
+        x.zero_()
+        lib.check(L.apk_capture_begin(h))
+        lib.check(L.apk_swiglu(h, hs.data_ptr(), x.data_ptr(), hs.numel(), lib.F32))
+        lib.check(L.apk_capture_end(h, C.byref(early)))
+        lib.check(L.apk_detach(h, base))  # the last owner: the device copy goes, with the graphs alive
         assert n_owners(base, total) == 0
         assert L.apk_resolve(h, base, 16, C.byref(dev)) == NOT_ATTACHED and dev.value is None
         assert L.apk_detach(h, base) == NOT_ATTACHED
         assert L.apk_detach(h, _addr(heap_copy)) == NOT_ATTACHED  # never attached
-        # a new mapping at the same host address gets a fresh copy (the reason detach must free: gpu/cuda/mod.rs:51-54)
+        # both graphs were recorded while the mapping was attached: they hold its freed addresses (or may) and are
+        # never replayed again -- declined, nothing launched (the reference drops its graphs here, device.rs:604-621)
+        rows.fill_(-1.0)
+        torch.cuda.synchronize()
+        assert L.apk_graph_launch(h, gr) == NOT_ATTACHED and b"record it again" in L.apk_last_error()
+        assert L.apk_graph_launch(h, early) == NOT_ATTACHED
+        lib.check(L.apk_sync(h))
+        assert float(rows.min()) == -1.0 and float(rows.max()) == -1.0
+        # a new mapping at the same host address gets a fresh copy (the reason detach must free: gpu/cuda/mod.rs:51-54):
+        # changed bytes are what runs, and the stale graph stays stale
         mapping[: table.nbytes] = synth.q4_k_table(g, vocab, H).reshape(-1)
         lib.check(L.apk_attach(h, base, total))
         lib.check(L.apk_resolve(h, base, table.nbytes, C.byref(d_table)))
         lib.check(L.apk_embed_rows(h, lib.FMT_Q4K, d_table, vocab, H, d_ids.data_ptr(), t, rows.data_ptr(), lib.F32))
         lib.check(L.apk_sync(h))
-        assert np.array_equal(rows.cpu().numpy(), ora.embed_rows(mapping[: table.nbytes], ora.FMT["Q4K"], vocab, H, ids))
+        new_rows = ora.embed_rows(mapping[: table.nbytes], ora.FMT["Q4K"], vocab, H, ids)
+        assert np.array_equal(rows.cpu().numpy(), new_rows) and not np.array_equal(new_rows, want_rows)
+        assert L.apk_graph_launch(h, gr) == NOT_ATTACHED
+        # a graph recorded now replays; one recorded before an unrelated, later mapping came and went does too
+        fresh = C.c_void_p()
+        lib.check(L.apk_capture_begin(h))
+        lib.check(L.apk_embed_rows(h, lib.FMT_Q4K, d_table, vocab, H, d_ids.data_ptr(), t, rows.data_ptr(), lib.F32))
+        lib.check(L.apk_capture_end(h, C.byref(fresh)))
+        other = np.zeros(4096, np.uint8)
+        lib.check(L.apk_attach(h, _addr(other), other.nbytes))
+        lib.check(L.apk_detach(h, _addr(other)))  # attached after `fresh` was recorded: cannot be inside it
+        rows.zero_()
+        torch.cuda.synchronize()
+        lib.check(L.apk_graph_launch(h, fresh))
+        lib.check(L.apk_sync(h))
+        assert np.array_equal(rows.cpu().numpy(), new_rows)
+        for gx in (gr, early, fresh):
+            lib.check(L.apk_graph_destroy(h, gx))
         lib.check(L.apk_detach(h, base))
     finally:
         L.apk_shutdown(h)
@@ -149,9 +180,23 @@ def test_host_mirror_names_weights_by_host_address():
         assert np.array_equal(qm.row(299).cpu().numpy(), ora.embed_rows(table, ora.FMT["Q8_0"], vocab, H, ids[:1])[0])
         with pytest.raises(ValueError):
             apk.QuantMat.from_mapping(be, view[:-1], apk.GgmlType.Q8_0, vocab, H)
-        be.detach(mapping)
-        be.detach(mapping)
-        be.detach(mapping)  # silent, as the reference
+        assert be.detach(mapping) and be.detach(mapping)
+        assert not be.detach(mapping)  # silent, as the reference
         assert be.owners(mapping) == 0 and be.resolve(view) is None
+        # the QuantMat borrowed its bytes and holds no owner: with the mapping gone every call declines, nothing launches
+        d0 = be.stats()[1]
+        out.fill_(7.0)
+        for call in (lambda: qm.row(0), lambda: qm.rows_into(torch.from_numpy(ids.view(np.int32)).cuda(), out),
+                     lambda: qm.dequant_rows(0, 2)):
+            with pytest.raises(apk.Declined):
+                call()
+        assert be.stats()[1] == d0 and float(out.min()) == 7.0
+        # attached again (new bytes at the same address): the same QuantMat reads the new copy
+        table2 = synth.q8_0_table(g, vocab, H).reshape(-1)
+        mapping[64 : 64 + table.nbytes] = table2
+        assert be.attach(mapping)
+        qm.rows_into(torch.from_numpy(ids.view(np.int32)).cuda(), out)
+        assert np.array_equal(out.cpu().numpy(), ora.embed_rows(table2, ora.FMT["Q8_0"], vocab, H, ids))
+        assert be.detach(mapping)
     finally:
         be.close()

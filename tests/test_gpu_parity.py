@@ -1160,7 +1160,7 @@ def test_route_reference_vectors_ties_sigmoid_bias(be, ora):
 @pytest.mark.parametrize("rows,n_expert,k", [(1, 128, 8), (6, 128, 8), (16, 128, 8), (16, 64, 6), (13, 256, 8), (16, 1024, 64), (5, 512, 10),
                                             (16, 16, 16), (1, 4, 4), (15, 60, 3), (9, 128, 16), (12, 1000, 25), (2, 64, 64), (16, 65, 1),
                                             # beyond one launch: the two entries run
-                                            (17, 128, 8), (64, 128, 8), (300, 24, 5)])
+                                            (17, 128, 8), (64, 128, 8), (300, 24, 5), (1024, 128, 8), (2049, 128, 8)])
 @pytest.mark.parametrize("gating", ["softmax", "sigmoid_bias"])
 def test_route_group_equals_router_then_grouping(be, ora, rows, n_expert, k, gating):
     """The one-launch router + grouping of a decode-sized batch against the oracle, and bit for bit against
@@ -1220,6 +1220,8 @@ def test_moe_permute_and_gather_bit_exact(be, ora, rows, k, n_expert):
 @pytest.mark.parametrize("rows,k,n_expert,n,f16", [(1024, 8, 128, 2048, False), (1, 8, 128, 2048, False), (33, 4, 16, 512, True),
                                                     (300, 8, 128, 2048, True), (7, 1, 4, 8192, False), (5, 3, 8, 64, True)])
 def test_moe_combine_add_rmsnorm(be, ora, rows, k, n_expert, n, f16):
+    import allpaka_amd as apk
+
     s = synth()
     g = s.rng(4, rows * 5 + n)
     logits = s.normal_f32(g, (rows, n_expert))
@@ -1242,6 +1244,14 @@ def test_moe_combine_add_rmsnorm(be, ora, rows, k, n_expert, n, f16):
     tx2 = dev(x)
     be.moe_combine_add_rmsnorm(tx2, dev(flat), dev(tok_off), dev(hit_row), dev(hit_w), None, None, 1e-6)
     assert torch.equal(tx2, tx)
+    # without the tok_off list: every token has k hits, at [t*k, (t+1)*k) -- the same launch minus one dependent load
+    assert np.array_equal(tok_off, np.arange(rows + 1, dtype=np.uint32) * k)
+    tx3, th3 = dev(x), torch.zeros_like(dev(x))
+    be.moe_combine_add_rmsnorm(tx3, dev(flat), None, dev(hit_row), dev(hit_w), th3, dev(gamma), 1e-6)
+    assert torch.equal(tx3, tx) and torch.equal(th3, th)
+    if rows > 1:  # hits that do not divide among the tokens cannot do without the list
+        with pytest.raises(apk.Declined):
+            be.moe_combine_add_rmsnorm(dev(x), dev(flat)[:-1], None, dev(hit_row), dev(hit_w), None, None, 1e-6)
 
 
 @pytest.mark.parametrize("rows,k,n_expert,n,f16", [(1024, 8, 128, 2048, False), (1, 8, 128, 2048, True), (33, 4, 16, 512, True),

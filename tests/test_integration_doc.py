@@ -130,10 +130,37 @@ def test_the_arm_has_an_item_for_every_entry_of_the_stub_arm():
     assert used and sorted(used - set(c)) == []
 
 
+def test_the_printed_build_script_builds_every_source_the_makefile_links():
+    """The library links what allpaka_amd/csrc/Makefile says it links; the build.rs printed for the Rust side must
+    name each of those sources (or the object built from it), or the crate would fail to link."""
+    mk = open(os.path.join(ROOT, "allpaka_amd", "csrc", "Makefile")).read()
+    link = re.search(r"^\$\(OUT\):.*\n\t(.*)$", mk, flags=re.M).group(1)
+    linked = re.findall(r"\b(apk_[a-z_]+\.(?:cpp|S|o|hip))\b", link)
+    assert "apk_host.cpp" in linked and "apk_embed.S" in linked and len(linked) >= 3
+    # an object stands for the source its rule compiles; the embedded code object for apk_kernels.hip
+    sources = set()
+    for f in linked:
+        if f.endswith(".o"):
+            rule = re.search(r"^" + re.escape(f) + r":\s*(\S+)", mk, flags=re.M)
+            assert rule, f"no rule for {f}"
+            sources.add(rule.group(1))
+        else:
+            sources.add(f)
+    sources.add("apk_kernels.hip")
+    md = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    start = md.index("// crates/allpaka-hip-sys/build.rs")
+    build_rs = md[start:md.index("\n```", start)]
+    missing = sorted(f for f in sources if f not in build_rs)
+    assert missing == [], f"build.rs in INTEGRATION.md does not build {missing}"
+    # every file it names exists in this repository
+    for f in re.findall(r"\{src\}/(apk_[a-z_]+\.[a-zA-Z]+)", build_rs):
+        assert os.path.exists(os.path.join(ROOT, "allpaka_amd", "csrc", f)), f
+
+
 def test_every_entry_named_in_the_mapping_tables_exists():
     md = open(os.path.join(ROOT, "INTEGRATION.md")).read()
     c = header_functions()
-    structs = {"apk_attn_prologue", "apk_plan", "apk_ctx", "apk_graph", "apk_hip", "apk_status", "apk_dq_fmt", "apk_kernels", "apk_embed", "apk_host"}
+    structs = {"apk_attn_prologue", "apk_plan", "apk_ctx", "apk_graph", "apk_hip", "apk_status", "apk_dq_fmt", "apk_kernels", "apk_embed", "apk_host", "apk_noalloc", "apk_noalloc_setup"}
     named = set(re.findall(r"\bapk_[a-z0-9_]+\b", md))
     unknown = sorted(n for n in named if n not in c and n not in structs)
     assert unknown == [], unknown

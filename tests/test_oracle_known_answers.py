@@ -278,6 +278,120 @@ def test_q8_0_and_q4_k_vs_independent_numpy_decoder(ora):
     assert np.array_equal(got.view(np.uint32), _np_q4_k(raw).view(np.uint32))
 
 
+def test_q5_0_hand_worked_block(ora):
+    # crates/allpaka-gguf/src/dequant.rs:128-141 -- the reference holds no Q5_0 vector of its own, so this block is
+    # worked out by hand from the layout it documents (and ggml publishes): bytes 0-1 f16 scale d, bytes 2-5 a
+    # little-endian 32-bit mask qh, bytes 6-21 nibbles; out[j] = d * ((qs[j] & 15 | bit j of qh << 4) - 16),
+    # out[j + 16] = d * ((qs[j] >> 4 | bit (j + 16) of qh << 4) - 16).
+    block = np.zeros(22, np.uint8)
+    block[0:2] = f16le(ora, 1.0)
+    # high bits set for elements 0, 15, 16 and 31: qh = 1 | 1 << 15 | 1 << 16 | 1 << 31 = 0x80018001, little-endian
+    block[2:6] = [0x01, 0x80, 0x01, 0x80]
+    qs = np.zeros(16, np.uint8)
+    qs[0] = 0xA3   # low nibble 3 -> element 0, high nibble 10 -> element 16
+    qs[1] = 0x5F   # low nibble 15 -> element 1, high nibble 5 -> element 17
+    qs[7] = 0x10   # low nibble 0 -> element 7, high nibble 1 -> element 23
+    qs[15] = 0xF0  # low nibble 0 -> element 15, high nibble 15 -> element 31
+    block[6:22] = qs
+    want = np.full(32, -16.0, np.float32)  # nibble 0, no high bit: 0 - 16
+    want[0] = 3 + 16 - 16       # element 0 has its high bit: 3
+    want[16] = 10 + 16 - 16     # element 16 has its high bit: 10
+    want[1] = 15 - 16           # -1
+    want[17] = 5 - 16           # -11
+    want[7] = 0 - 16
+    want[23] = 1 - 16           # -15
+    want[15] = 0 + 16 - 16      # element 15: high bit only: 0
+    want[31] = 15 + 16 - 16     # element 31: the largest value, 15
+    out = ora.dequant(Q5_0, block, 32)
+    assert np.array_equal(out, want), (out, want)
+    assert out.min() == -16.0 and out.max() == 15.0
+    # the scale multiplies: d = 0.5 halves every value; a negative d flips the signs
+    block[0:2] = f16le(ora, 0.5)
+    assert np.array_equal(ora.dequant(Q5_0, block, 32), want * np.float32(0.5))
+    block[0:2] = f16le(ora, -2.0)
+    assert np.array_equal(ora.dequant(Q5_0, block, 32), want * np.float32(-2.0))
+    # one bit of qh at a time moves exactly one element by 16 d, and it is element `bit`
+    block[0:2] = f16le(ora, 1.0)
+    for bit in range(32):
+        b2 = block.copy()
+        b2[2:6] = np.frombuffer(struct.pack("<I", 0x80018001 ^ (1 << bit)), np.uint8)
+        diff = ora.dequant(Q5_0, b2, 32) - want
+        assert np.flatnonzero(diff).tolist() == [bit] and abs(diff[bit]) == 16.0
+    # one nibble at a time: the low nibble of byte j is element j, the high nibble element j + 16
+    for j in range(16):
+        for shift, elem in ((0, j), (4, j + 16)):
+            b2 = block.copy()
+            b2[6 + j] ^= 1 << shift
+            assert np.flatnonzero(ora.dequant(Q5_0, b2, 32) - want).tolist() == [elem]
+
+
+def _np_q5_0(raw):
+    """Independent second decoder of Q5_0, vectorised, from ggml's published dequantize_row_q5_0 (which shifts the
+    mask as ((qh >> j) << 4) & 0x10 and (qh >> (j + 12)) & 0x10 rather than testing bit j and bit j + 16)."""
+    b = raw.reshape(-1, 22)
+    d = b[:, 0:2].copy().view(np.float16).astype(np.float32)           # [blocks, 1]
+    qh = b[:, 2:6].copy().view("<u4").astype(np.uint32)                # [blocks, 1]
+    j = np.arange(16, dtype=np.uint32)[None, :]
+    xh0 = ((qh >> j) << np.uint32(4)) & np.uint32(0x10)
+    xh1 = (qh >> (j + np.uint32(12))) & np.uint32(0x10)
+    qs = b[:, 6:22].astype(np.uint32)
+    x0 = ((qs & 0xF) | xh0).astype(np.int32) - 16
+    x1 = ((qs >> 4) | xh1).astype(np.int32) - 16
+    return (np.concatenate([x0, x1], axis=1).astype(np.float32) * d).astype(np.float32).reshape(-1)
+
+
+def test_q5_0_vs_independent_numpy_decoder(ora):
+    rng = np.random.default_rng(50)
+    nb = 512
+    raw = rng.integers(0, 256, size=22 * nb, dtype=np.uint8)
+    blk = raw.reshape(-1, 22)
+    sc = rng.integers(0, 0x3C00, size=nb, dtype=np.uint16) | (rng.integers(0, 2, size=nb, dtype=np.uint16) << 15)
+    sc[:8] = np.arange(8, dtype=np.uint16)  # zero and the smallest f16 subnormals
+    blk[:, 0:2] = sc.view(np.uint8).reshape(-1, 2)
+    got = ora.dequant(Q5_0, raw, 32 * nb)
+    assert np.array_equal(got.view(np.uint32), _np_q5_0(raw).view(np.uint32))
+    # every 5-bit code appears in both halves of some block and decodes to code - 16
+    for code in range(32):
+        block = np.zeros(22, np.uint8)
+        block[0:2] = f16le(ora, 1.0)
+        block[6:22] = (code & 15) | ((code & 15) << 4)
+        block[2:6] = 0xFF if code & 16 else 0
+        assert np.all(ora.dequant(Q5_0, block, 32) == code - 16)
+
+
+def test_f16_bf16_f32_rows_hand_worked(ora):
+    # crates/allpaka-gguf/src/dequant.rs:38-41 with allpaka-dtype's byte converters (lib.rs:188-192, 200-320): rows of
+    # plain little-endian values.  Bit patterns written out by hand:
+    #   f16 : 0x3C00 = 1, 0xC000 = -2, 0x3555 = 0.333251953125, 0x7BFF = 65504, 0x0001 = 2^-24, 0x8000 = -0
+    #   bf16: the upper half of the f32 pattern -- 0x3F80 = 1, 0xC000 = -2, 0x3EAB = 0.333984375 (0x3EAB0000),
+    #         0x7F7F = 3.3895313892515355e38, 0x0001 = 2^-133 (an f32 subnormal, 0x00010000), 0x8000 = -0
+    #   f32 : the pattern itself
+    f16_bytes = np.array([0x3C00, 0xC000, 0x3555, 0x7BFF, 0x0001, 0x8000], "<u2").view(np.uint8)
+    want16 = np.array([1.0, -2.0, 0.333251953125, 65504.0, 2.0 ** -24, -0.0], np.float32)
+    got = ora.dequant(F16, f16_bytes, 6)
+    assert np.array_equal(got.view(np.uint32), want16.view(np.uint32))
+    bf_bytes = np.array([0x3F80, 0xC000, 0x3EAB, 0x7F7F, 0x0001, 0x8000], "<u2").view(np.uint8)
+    wantbf = np.array([1.0, -2.0, 0.333984375, 3.3895313892515355e38, 2.0 ** -133, -0.0], np.float32)
+    got = ora.dequant(BF16, bf_bytes, 6)
+    assert np.array_equal(got.view(np.uint32), wantbf.view(np.uint32))
+    assert np.array_equal(got.view(np.uint32), np.array([0x3F800000, 0xC0000000, 0x3EAB0000, 0x7F7F0000, 0x00010000, 0x80000000], np.uint32))
+    # bf16 -> f32 is "shift left by 16" for every one of the 65536 patterns (NaNs included: the payload is kept)
+    codes = np.arange(65536, dtype="<u2")
+    got = ora.dequant(BF16, codes.view(np.uint8), 65536)
+    assert np.array_equal(got.view(np.uint32), codes.astype(np.uint32) << 16)
+    # byte order: swapping the two bytes of a value changes it (0x3F80 = 1.0, 0x803F = -5.7e-39 as bf16)
+    assert ora.dequant(BF16, np.array([0x3F, 0x80], np.uint8), 1).view(np.uint32)[0] == 0x803F0000
+    f32_vals = np.array([1.0, -2.0, 1.0 / 3.0, 3.4028234663852886e38, 1e-45, -0.0], np.float32)
+    raw = np.frombuffer(struct.pack("<6I", 0x3F800000, 0xC0000000, 0x3EAAAAAB, 0x7F7FFFFF, 0x00000001, 0x80000000), np.uint8)
+    got = ora.dequant(F32, raw, 6)
+    assert np.array_equal(got.view(np.uint32), f32_vals.view(np.uint32))
+    # rows through the gather: row 1 of a 2-row F16 / BF16 / F32 table is the second half of the bytes
+    for fmt, width, vals in ((F16, 2, f16_bytes), (BF16, 2, bf_bytes), (F32, 4, raw)):
+        table = np.concatenate([np.zeros(6 * width, np.uint8), vals])
+        row = ora.embed_rows(table, fmt, 2, 6, [1])
+        assert np.array_equal(row.reshape(-1).view(np.uint32), ora.dequant(fmt, vals, 6).view(np.uint32))
+
+
 def test_q4_k_all_nibble_sub_block_cases(ora):
     # brute force: every (byte value, sub-block pair) with distinct scales/mins
     for pair in range(4):
