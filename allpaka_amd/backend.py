@@ -314,6 +314,29 @@ class Backend:
         if not self._recording and self.take_faults() & _l.FAULT_CACHE_RANGE:
             raise AssertionError("position past capacity")
 
+    def qknorm_rope_pos(self, q, k, q_norm, k_norm, positions, inv_freq, n_q, n_kv, head_dim, eps, adjacent_pairs=False,
+                        rot_dim=None, v=None, k_cache=None, v_cache=None):
+        """The QK-norm + RoPE step of a decode-sized batch (at most 64 rows) with the angles taken from the rows' positions
+        inside the launch: rope_sin_cos(pos, inv_freq) per row (rope.rs:18-22) instead of a table; with k_cache / v_cache
+        (fp16 [capacity, n_kv*head_dim]) also KvCache::store_at at row positions[r] (kv.rs:682-697).  The reference's
+        rmsnorm_rope_freq_dpos / rmsnorm_rope_store_freq_dpos (gpu/cuda/kernels.rs:577-671)."""
+        rows = q.numel() // (n_q * head_dim) if n_q else k.numel() // (n_kv * head_dim)
+        rot = head_dim if rot_dim is None else rot_dim
+        assert q.numel() == rows * n_q * head_dim and k.numel() == rows * n_kv * head_dim and q.dtype == k.dtype
+        assert positions.numel() == rows and positions.dtype == torch.int32
+        assert inv_freq.dtype == torch.float32 and inv_freq.numel() == rot // 2
+        cap = 0
+        if k_cache is not None:
+            assert v is not None and v.numel() == k.numel() and v.dtype == k.dtype and v_cache is not None
+            assert k_cache.dtype == v_cache.dtype == torch.float16 and k_cache.shape == v_cache.shape and k_cache.shape[1] == n_kv * head_dim
+            cap = k_cache.shape[0]
+        self._enter()
+        check(self.L.apk_qknorm_rope_pos(self.h, _ptr(q), _ptr(k), _ptr(v), _ptr(q_norm), _ptr(k_norm), _ptr(positions), _ptr(inv_freq),
+                                         _ptr(k_cache), _ptr(v_cache), cap, rows, n_q, n_kv, head_dim, rot, 1 if adjacent_pairs else 0, eps, _dt(q)))
+        self._leave()
+        if k_cache is not None and not self._recording and self.take_faults() & _l.FAULT_CACHE_RANGE:
+            raise AssertionError("position past capacity")
+
     def cast(self, src, dtype):
         """allpaka_dtype::f32_to_f16 / f16_to_f32 over a tensor (dtype/src/lib.rs:129-184), bit for bit."""
         assert src.dtype in (torch.float32, torch.float16) and dtype in (torch.float32, torch.float16) and dtype != src.dtype

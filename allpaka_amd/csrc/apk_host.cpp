@@ -70,7 +70,7 @@ std::vector<std::string> all_kernel_names() {
     std::vector<std::string> v = {"apk_swiglu_f32", "apk_swiglu_f16", "apk_geglu_tanh_f32", "apk_geglu_tanh_f16", "apk_rope_table", "apk_embed_q4k_f32",
                                   "apk_embed_q4k_f16", "apk_embed_q8_0_f32", "apk_embed_q8_0_f16", "apk_route_topk",
                                   "apk_moe_permute", "apk_gather_rows", "apk_scatter_rows_t1", "apk_scatter_rows_t2", "apk_argmax_rows", "apk_add_rmsnorm_ragged_f32", "apk_add_rmsnorm_ragged_f16", "apk_copy",
-                                  "apk_qknorm_rope_generic_f32", "apk_qknorm_rope_generic_f16", "apk_route_topk_wide", "apk_route_topk_e64", "apk_route_topk_e128", "apk_route_group_small_e64", "apk_route_group_small_e128",
+                                  "apk_qknorm_rope_generic_f32", "apk_qknorm_rope_generic_f16", "apk_qknorm_rope_pos_f32", "apk_qknorm_rope_pos_f16", "apk_route_topk_wide", "apk_route_topk_e64", "apk_route_topk_e128", "apk_route_group_small_e64", "apk_route_group_small_e128",
                                   "apk_route_group_small_e256", "apk_route_group_small_e1024", "apk_add_assign_f32", "apk_add_assign_f16", "apk_softmax_rows", "apk_moe_count", "apk_moe_rank",
                                   "apk_add_bias_rows_f32", "apk_add_bias_rows_f16", "apk_moe_shared_hits", "apk_cast_f32_f16", "apk_cast_f16_f32", "apk_zero_u64"};
     for (const char* t : {"f32", "f16"}) {
@@ -1064,6 +1064,34 @@ int apk_qknorm_rope_norm(apk_ctx* c, void* q, void* k, const float* qw, const fl
     if (!c) return fail(APK_DECLINE_NULL, "apk_qknorm_rope_norm: ctx is NULL");
     CallScope s(c);
     return qknorm_rope_common(c, q, k, qw, kw, rope, rows, n_q, n_kv, head_dim, rot_dim, eps, dtype, nullptr, 1);
+}
+
+int apk_qknorm_rope_pos(apk_ctx* c, void* q, void* k, const void* v, const float* qw, const float* kw, const uint32_t* positions,
+                        const float* inv_freq, void* k_cache, void* v_cache, size_t capacity, size_t rows, size_t n_q,
+                        size_t n_kv, size_t head_dim, size_t rot_dim, int adjacent_pairs, float eps, int dtype) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_qknorm_rope_pos: ctx is NULL");
+    CallScope s(c);
+    const int es = elem_size(dtype);
+    if (!es) return fail(APK_DECLINE_UNSUPPORTED, "apk_qknorm_rope_pos: dtype %d", dtype);
+    if (head_dim == 0 || head_dim > 65536 || rot_dim % 2 || rot_dim > head_dim)
+        return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_pos: head_dim %zu, rot_dim %zu", head_dim, rot_dim);
+    if (rows > 64)
+        return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_pos: %zu rows (a decode-sized batch of at most 64; beyond that build the table "
+                                       "with apk_rope_table)", rows);
+    if (n_q > 65535 || n_kv > 65535) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_pos: too many heads");
+    const bool store = k_cache || v_cache;
+    if (store && (!k_cache || !v_cache || !v)) return fail(APK_DECLINE_NULL, "apk_qknorm_rope_pos: the cache store needs v, k_cache and v_cache");
+    if (store && n_kv == 0) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_pos: no k heads to store");
+    if (store && (capacity == 0 || capacity > 0xffffffffu)) return fail(APK_DECLINE_SHAPE, "apk_qknorm_rope_pos: capacity");
+    if (rows == 0 || n_q + n_kv == 0) return APK_OK;
+    if ((n_q && !q) || (n_kv && !k) || !positions || (rot_dim && !inv_freq)) return fail(APK_DECLINE_NULL, "apk_qknorm_rope_pos: NULL tensor");
+    if (int rc = set_device(c)) return rc;
+    int rows_i = (int)rows, nq_i = (int)n_q, nkv_i = (int)n_kv, hd_i = (int)head_dim, half_i = (int)(rot_dim / 2), style = adjacent_pairs ? 1 : 0;
+    uint32_t cap32 = (uint32_t)capacity;
+    void* args[] = {&q, &k, &v, &qw, &kw, &positions, &inv_freq, &k_cache, &v_cache, &cap32, &rows_i, &nq_i, &nkv_i, &hd_i, &half_i, &style,
+                    &eps, &c->fault_dev};
+    const uint64_t waves = (uint64_t)rows * (n_q + n_kv + (store ? n_kv : 0));
+    return launch(c, dtype == APK_F32 ? "apk_qknorm_rope_pos_f32" : "apk_qknorm_rope_pos_f16", (unsigned)((waves + 3) / 4), 256, 0, args);
 }
 
 int apk_qknorm_rope_kv_store(apk_ctx* c, void* q, void* k, const void* v, const float* qw, const float* kw,

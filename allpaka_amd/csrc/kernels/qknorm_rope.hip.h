@@ -449,6 +449,92 @@ extern "C" __global__ __launch_bounds__(256) void apk_qknorm_rope_generic_f16(
     qknorm_rope_generic_body<f16_t>(q, k, qw, kw, rope, rows, n_q, n_kv, hd, rot_half, norm_style, eps, qb, kb);
 }
 
+// The same step with the rotary angles taken from the rows' positions inside the kernel, for a decode-sized batch:
+// [sin, cos] of pair i of a row is sincos((pos[row] as f32) * inv_freq[i]) (rope.rs:18-22), evaluated in double and
+// rounded once, exactly what apk_rope_table writes -- so the launch equals apk_rope_table followed by the op on that
+// table, without the table (the reference's rmsnorm_rope_freq_dpos / rmsnorm_rope_store_freq_dpos,
+// gpu/cuda/kernels.rs:577-671, which read d_pos and inv_freq in the kernel so that one recorded graph serves every
+// token).  A wave per head, element-wise, any head geometry and either pairing; with k_cache / v_cache the rotated k
+// heads and the row's v heads are also narrowed to fp16 into cache row pos[row] (KvCache::store_at, kv.rs:682-697).
+// The double-precision sine and cosine make a wave long; the host takes this kernel for up to 64 rows, where the
+// launch, not the arithmetic, is the cost.
+template <typename T>
+DEV void qknorm_rope_pos_body(T* q, T* k, const T* v, const float* qw, const float* kw, const uint32_t* pos,
+                              const float* inv_freq, f16_t* k_cache, f16_t* v_cache, uint32_t capacity, int rows, int n_q,
+                              int n_kv, int hd, int rot_half, int norm_style, float eps, uint32_t* fault) {
+    typedef typename headstat<T>::acc_t acc_t;
+    const int lane = threadIdx.x & 63;
+    const uint64_t wid = ((uint64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const uint64_t heads = (uint64_t)n_q + n_kv + (v_cache ? n_kv : 0);
+    if (wid >= (uint64_t)rows * heads) return;  // whole wave
+    const uint64_t row = wid / heads;
+    const int hh = (int)(wid % heads);
+    const uint32_t p = pos[row];
+    const uint64_t kv_dim = (uint64_t)n_kv * hd;
+    const bool cache_ok = p < capacity;  // uniform per row
+    if (hh >= n_q + n_kv) {  // a v head: narrowed into the cache as it is
+        const int vh = hh - n_q - n_kv;
+        if (!cache_ok) return;
+        const T* src = v + row * kv_dim + (uint64_t)vh * hd;
+        f16_t* dst = v_cache + p * kv_dim + (uint64_t)vh * hd;
+        for (int i = lane; i < hd; i += 64) dst[i] = (f16_t)(float)src[i];
+        return;
+    }
+    const bool isq = hh < n_q;
+    T* x = isq ? q + (row * n_q + hh) * (uint64_t)hd : k + row * kv_dim + (uint64_t)(hh - n_q) * hd;
+    const float* w = isq ? qw : kw;
+    f16_t* kc = nullptr;
+    if (!isq && k_cache) {
+        if (!cache_ok && lane == 0 && hh == n_q) atomicOr(fault, APK_FAULT_CACHE_RANGE);
+        kc = cache_ok ? k_cache + p * kv_dim + (uint64_t)(hh - n_q) * hd : nullptr;
+    }
+    typename headstat<T>::scale_t scale{};
+    if (w) {
+        acc_t ss = 0;
+        for (int i = lane; i < hd; i += 64) ss = headstat<T>::sq(ss, (float)x[i]);
+        ss = group_sum<64>(ss);  // every lane's loads are consumed here, before any store below
+        scale = headstat<T>::rscale(ss, hd, eps);
+    }
+    const float posf = (float)p;
+    for (int i = lane; i < rot_half; i += 64) {
+        const int ia = norm_style ? 2 * i : i, ib = norm_style ? 2 * i + 1 : i + rot_half;
+        float a = (float)x[ia], b = (float)x[ib];
+        if (w) {
+            a = headstat<T>::apply(a, scale, w[ia]);
+            b = headstat<T>::apply(b, scale, w[ib]);
+        }
+        double sd, cd;
+        sincos((double)(posf * inv_freq[i]), &sd, &cd);  // one f32 rounding of the angle, as the reference
+        const float sn = (float)sd, cs = (float)cd;
+        const T oa = (T)(a * cs - b * sn), ob = (T)(a * sn + b * cs);
+        x[ia] = oa;
+        x[ib] = ob;
+        if (kc) {
+            kc[ia] = (f16_t)(float)oa;
+            kc[ib] = (f16_t)(float)ob;
+        }
+    }
+    for (int i = 2 * rot_half + lane; i < hd; i += 64) {  // channels past the rotary width: normalised, not rotated
+        const T o = w ? (T)headstat<T>::apply((float)x[i], scale, w[i]) : x[i];
+        if (w) x[i] = o;
+        if (kc) kc[i] = (f16_t)(float)o;
+    }
+}
+extern "C" __global__ __launch_bounds__(256) void apk_qknorm_rope_pos_f32(
+    float* q, float* k, const float* v, const float* qw, const float* kw, const uint32_t* pos, const float* inv_freq,
+    f16_t* k_cache, f16_t* v_cache, uint32_t capacity, int rows, int n_q, int n_kv, int hd, int rot_half, int norm_style,
+    float eps, uint32_t* fault) {
+    qknorm_rope_pos_body<float>(q, k, v, qw, kw, pos, inv_freq, k_cache, v_cache, capacity, rows, n_q, n_kv, hd, rot_half,
+                                norm_style, eps, fault);
+}
+extern "C" __global__ __launch_bounds__(256) void apk_qknorm_rope_pos_f16(
+    f16_t* q, f16_t* k, const f16_t* v, const float* qw, const float* kw, const uint32_t* pos, const float* inv_freq,
+    f16_t* k_cache, f16_t* v_cache, uint32_t capacity, int rows, int n_q, int n_kv, int hd, int rot_half, int norm_style,
+    float eps, uint32_t* fault) {
+    qknorm_rope_pos_body<f16_t>(q, k, v, qw, kw, pos, inv_freq, k_cache, v_cache, capacity, rows, n_q, n_kv, hd, rot_half,
+                                norm_style, eps, fault);
+}
+
 // Layer prologue for small decode batches: the residual add + RMSNorm of the hidden
 // rows and the QK-norm + RoPE of the q/k rows as ONE launch.  They are two independent
 // jobs sharing a grid (workgroups [0, rows) normalise one hidden row each, the rest

@@ -287,6 +287,23 @@ int apk_qknorm_rope_norm_kv_store(apk_ctx* ctx, void* q, void* k, const void* v,
                                   size_t capacity, size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim,
                                   float eps, int dtype);
 
+/* The same step with the rotary angles taken from the rows' positions INSIDE the launch, for a decode-sized batch
+ * (rows <= 64): [sin, cos] of pair i of row r is sincos((positions[r] as f32) * inv_freq[i]) (ops::rope_sin_cos,
+ * ops/rope.rs:18-22), the values apk_rope_table writes, so the call equals apk_rope_table(positions, inv_freq, ...)
+ * followed by apk_qknorm_rope_neox / _norm (adjacent_pairs != 0) on that table -- without the table and without its
+ * launch.  Replaces the reference's device-angle kernels rmsnorm_rope_freq_dpos / rmsnorm_rope_store_freq_dpos
+ * (gpu/cuda/kernels.rs:577-671; set_rope_inv_freq / has_device_rope_freq, gpu/stub.rs), which read the position and
+ * inv_freq in the kernel so that one recorded graph serves every token.  positions: u32[rows] and inv_freq:
+ * f32[rot_dim/2], both on the device.  With k_cache and v_cache (both or neither; then v is required) the rotated k
+ * rows and the rows of v are also narrowed to fp16 into cache row positions[r], as apk_qknorm_rope_kv_store does with
+ * cache_pos = positions; a position >= capacity skips that row's store and raises APK_FAULT_CACHE_RANGE.  Any head
+ * geometry, partial rotary included.  More than 64 rows: APK_DECLINE_SHAPE (build the table once per step with
+ * apk_rope_table and run the table form, which is the faster one from there on).  May be recorded. */
+int apk_qknorm_rope_pos(apk_ctx* ctx, void* q, void* k, const void* v, const float* qw, const float* kw,
+                        const uint32_t* positions, const float* inv_freq, void* k_cache, void* v_cache, size_t capacity,
+                        size_t rows, size_t n_q, size_t n_kv, size_t head_dim, size_t rot_dim, int adjacent_pairs,
+                        float eps, int dtype);
+
 /* Layer prologue as ONE launch: apk_add_rmsnorm_rows(x, delta, h, gamma, n, rows) and
  * apk_qknorm_rope_neox(q, k, qw, kw, rope, rows, ...) with the same arguments and the
  * same results, as two independent jobs in one grid (the reference's accelerators fuse

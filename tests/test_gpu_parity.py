@@ -626,6 +626,91 @@ def test_qknorm_rope_kv_store(be, ora, rows, n_q, n_kv, hd, f16, style, partial)
     assert f16_ulp_diff(host(kc), wkc) <= (TOL_F16_ULP if f16 else 1)
 
 
+@pytest.mark.parametrize("rows,n_q,n_kv,hd,rot,f16", [(1, 64, 8, 128, 128, True), (64, 64, 8, 128, 128, True), (6, 16, 8, 128, 128, False),
+                                                       (1, 16, 8, 128, 128, False), (8, 4, 4, 64, 32, True), (5, 2, 1, 256, 256, False),
+                                                       (3, 3, 2, 96, 64, False), (64, 1, 0, 128, 128, True), (2, 4, 2, 80, 0, False)])
+@pytest.mark.parametrize("style", [0, 1])
+@pytest.mark.parametrize("store", [False, True])
+def test_qknorm_rope_with_positions_inside_the_launch(be, ora, rows, n_q, n_kv, hd, rot, f16, style, store):
+    """A decode-sized batch with the rotary angles taken from the rows' positions in the kernel (no table): the oracle's
+    rope_sin_cos rows on the CPU side; on the device also equal to apk_rope_table followed by the table form, bit for bit,
+    wherever that form takes the same arithmetic path (heads outside 64 / 128 / 256 or a partial rotary width)."""
+    import allpaka_amd as apk
+
+    if store and n_kv == 0:
+        pytest.skip("no k heads to store")
+    s = synth()
+    g = s.rng(3, rows * 7 + hd + rot)
+    cap = 40000
+    positions = g.integers(0, 32768, size=rows).astype(np.uint32)
+    positions[0] = 0
+    q, k, qw, kw, _, _ = _qk_case(ora, 3, rows, n_q, n_kv, hd, f16, [0] * rows)
+    inv = ora.rope_inv_freq(rot, 1e6) if rot else np.zeros(0, np.float32)
+    ropes = ora.rope_table([int(p) for p in positions], inv) if rot else np.zeros((rows, 0, 2), np.float32)
+    v = s.normal_f32(g, (rows, n_kv * hd))
+    if f16:
+        v = s.to_f16_bits(v)
+    wq, wk = q.copy(), k.copy()
+    ora.qknorm_rope_rows(wq, wk, n_q, n_kv, hd, qw, kw, ropes, 1e-6, style=style)
+    tq, tk = dev(q), dev(k)
+    kc = vc = None
+    if store:
+        # a small cache addressed through a position map would hide a wrong row: the cache is as long as the context
+        kc = torch.zeros((cap, n_kv * hd), dtype=torch.float16, device="cuda")
+        vc = torch.zeros_like(kc)
+    d0 = be.stats()[1]
+    be.qknorm_rope_pos(tq, tk, dev(qw), dev(kw), dev(positions), dev(inv) if rot else torch.zeros(1, device="cuda")[:0], n_q, n_kv, hd, 1e-6,
+                       adjacent_pairs=bool(style), rot_dim=rot, v=dev(v) if store else None, k_cache=kc, v_cache=vc)
+    assert be.stats()[1] == d0 + 1  # one launch
+    gq, gk = host(tq), host(tk)
+    for got, want in ((gq, wq), (gk, wk)):
+        if f16:
+            assert f16_ulp_diff(got, want) <= TOL_F16_ULP
+        else:
+            assert rel_err_f32(got, want) <= TOL_F32 and close_idiom(got, want)
+    if store:
+        rows_used = np.unique(positions)
+        assert len(rows_used) == rows or rows > 1  # (duplicates are possible; the later row wins on both sides below)
+        wkc, wvc = np.zeros((cap, n_kv * hd), np.uint16), np.zeros((cap, n_kv * hd), np.uint16)
+        ora.kv_store_rows(gk, v, positions, wkc, wvc)  # exactly the narrowing of the k this launch produced, v bit-exact
+        if len(rows_used) == rows:
+            assert np.array_equal(host(kc)[rows_used], wkc[rows_used]) and np.array_equal(host(vc)[rows_used], wvc[rows_used])
+        untouched = np.ones(cap, bool)
+        untouched[rows_used] = False
+        assert not host(kc)[untouched].any() and not host(vc)[untouched].any()
+    # the table form on the device: the same angles (apk_rope_table), then the op
+    if rot:
+        table = be.rope_table(dev(positions), dev(inv))
+        assert np.array_equal(host(table).view(np.uint32).reshape(rows, -1), np.asarray(ropes).view(np.uint32).reshape(rows, -1)) or \
+            np.max(np.abs(host(table).reshape(rows, -1) - np.asarray(ropes).reshape(rows, -1))) <= 6e-8
+        uq, uk = dev(q), dev(k)
+        be.qknorm_rope_neox(uq, uk, dev(qw), dev(kw), table, n_q, n_kv, hd, 1e-6, rot_dim=rot) if not style else \
+            be.qknorm_rope_norm(uq, uk, dev(qw), dev(kw), table, n_q, n_kv, hd, 1e-6, rot_dim=rot)
+        if f16:
+            assert f16_ulp_diff(gq, host(uq)) <= 1 and f16_ulp_diff(gk, host(uk)) <= 1
+            assert np.mean(gq == host(uq)) > 0.9999
+        else:
+            assert rel_err_f32(gq, host(uq)) <= 2e-7 and rel_err_f32(gk, host(uk)) <= 2e-7
+    # more than a decode-sized batch is declined, nothing launched
+    if rows == 64:
+        big = torch.zeros((65, n_q * hd), dtype=tq.dtype, device="cuda")
+        bigk = torch.zeros((65, n_kv * hd), dtype=tq.dtype, device="cuda")
+        with pytest.raises(apk.Declined):
+            be.qknorm_rope_pos(big, bigk, dev(qw), dev(kw), torch.zeros(65, dtype=torch.int32, device="cuda"), dev(inv), n_q, n_kv, hd, 1e-6,
+                               adjacent_pairs=bool(style), rot_dim=rot)
+
+
+def test_qknorm_rope_pos_past_capacity_is_flagged_not_faulted(be, ora):
+    rows, n_q, n_kv, hd = 3, 2, 1, 128
+    q, k, qw, kw, inv, _ = _qk_case(ora, 3, rows, n_q, n_kv, hd, False, [1, 2, 3])
+    kc = torch.zeros((4, n_kv * hd), dtype=torch.float16, device="cuda")
+    vc = torch.zeros_like(kc)
+    with pytest.raises(AssertionError, match="position past capacity"):
+        be.qknorm_rope_pos(dev(q), dev(k), dev(qw), dev(kw), dev(np.array([1, 4, 3], np.uint32)), dev(inv), n_q, n_kv, hd, 1e-6,
+                           v=dev(k), k_cache=kc, v_cache=vc)
+    assert host(kc)[1].any() and host(kc)[3].any() and not host(kc)[[0, 2]].any()
+
+
 def test_kv_store_position_past_capacity_is_flagged_not_faulted(be, ora):
     rows, n_q, n_kv, hd = 3, 2, 1, 128
     q, k, qw, kw, inv, ropes = _qk_case(ora, 3, rows, n_q, n_kv, hd, False, [1, 2, 3])
