@@ -89,7 +89,7 @@ def main():
 
     # ~2 ms of plain copies: what runs between a restore of inputs (which ends in a wait, so the GPU goes idle and its
     # clocks drop) and the launches that are timed, so that every timed batch starts on a GPU in its streaming state
-    warm_half = 100 << 20
+    warm_half = 96 << 20  # (not the 100 MiB of the calibration copy below: a profile tells the two launch sizes apart)
     warm_buf = torch.empty(2 * warm_half, dtype=torch.uint8, device=dev)
     warm_buf.view(torch.float32).normal_()
 

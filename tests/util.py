@@ -14,6 +14,18 @@ def rel_err_f32(got, want):
     return float(np.max(np.abs(got - want) / np.maximum(np.abs(want), floor))) if got.size else 0.0
 
 
+def rel_err_strict(got, want, min_rel=1e-3):
+    """Max of |g-w| / |w| over the elements with |w| > min_rel * rms(want), no floor: the strict element-wise relative
+    error wherever an output has not cancelled to (almost) nothing.  The elements it leaves out are held to the
+    reference's idiom (close_idiom) by the callers."""
+    got = np.asarray(got, np.float64).ravel()
+    want = np.asarray(want, np.float64).ravel()
+    if got.size == 0:
+        return 0.0
+    big = np.abs(want) > min_rel * float(np.sqrt(np.mean(want * want)))
+    return float(np.max(np.abs(got[big] - want[big]) / np.abs(want[big]))) if big.any() else 0.0
+
+
 def close_idiom(got, want):
     """The reference's own closeness idiom, |a-b| < 1e-5 * (1 + |b|)
     (crates/allpaka-backend/src/ops/mod.rs:25-27), over whole arrays."""
