@@ -298,6 +298,25 @@ def main():
                 p(qk[i % len(qk)]["q"]), p(qk[i % len(qk)]["k"]), p(qw), p(kw), p(rope), rows, NQ, NKV, HD, HD, EPS, F16)), 200)
             record("layer_prologue (add_rmsnorm || qknorm_rope, one launch)", sh, us,
                    4 * rows * H * b + 4 * H + 2 * rows * (NQ + NKV) * HD * b + rows * (HD // 2) * 8 + 2 * HD * 4, note="launch-bound")
+        # a decode step's QK-norm + RoPE + K/V cache store with the rotary angles taken from the device positions inside the
+        # launch, against the table built by a launch of its own and then the table form (what a recorded decode chain
+        # runs once per token and once per layer, respectively)
+        for rows, label in ((1, "decode T=1"), (64, "batched decode, 64 rows with own positions")):
+            sh = f"qwen3-32b {label} f16"
+            nbp = 2 * rows * (NQ + NKV) * HD * b + rows * NKV * HD * b + 2 * rows * NKV * HD * 2 + rows * 4 + (HD // 2) * 4 + 2 * HD * 4
+            us = timed(lambda i: apklib.check(L.apk_qknorm_rope_pos(
+                h, p(qk[i % len(qk)]["q"]), p(qk[i % len(qk)]["k"]), p(kvp[i % len(qk)]["v"]), p(qw), p(kw), p(pos), p(inv),
+                p(kvp[i % len(qk)]["kc"]), p(kvp[i % len(qk)]["vc"]), T, rows, NQ, NKV, HD, HD, 0, EPS, F16)), 200)
+            record("qknorm_rope_pos: angles from positions in the launch + K/V cache store (one launch)", sh, us, nbp, note="launch-bound")
+
+            def table_then_op(i, rows=rows):
+                apklib.check(L.apk_rope_table(h, p(pos), p(inv), rows, HD // 2, p(rope)))
+                apklib.check(L.apk_qknorm_rope_kv_store(
+                    h, p(qk[i % len(qk)]["q"]), p(qk[i % len(qk)]["k"]), p(kvp[i % len(qk)]["v"]), p(qw), p(kw), p(rope), p(pos),
+                    p(kvp[i % len(qk)]["kc"]), p(kvp[i % len(qk)]["vc"]), T, rows, NQ, NKV, HD, HD, EPS, F16))
+            us = timed(table_then_op, 200)
+            record("rope_table, then qknorm_rope + K/V cache store (two launches)", sh, us, nbp + rows * (HD // 2) * 16, launches=2, note="launch-bound")
+        apklib.check(L.apk_rope_table(h, p(pos), p(inv), T, HD // 2, p(rope)))  # the full table again
         # the decode chain of a whole model (64 layers x 4 launches) issued op by op, and recorded once
         # and replayed with one submission; and the 3-launch form with the fused prologue
         NL = 64
