@@ -436,6 +436,20 @@ class Backend:
         self._leave()
         return ids, w
 
+    def route(self, probs, k):
+        """model::route(probs, k) (moe.rs:623-658): the top k of an already softmaxed row, renormalised -> list of
+        (expert, weight), best first."""
+        n = probs.numel()
+        k = min(k, n)
+        if k == 0:
+            return []
+        ids = torch.empty((1, k), dtype=torch.int32, device=self.device)
+        w = torch.empty((1, k), dtype=torch.float32, device=self.device)
+        self._enter()
+        check(self.L.apk_route_topk(self.h, _ptr(probs), None, 1, n, k, 1, 1.0, 2, _ptr(ids), _ptr(w)))
+        self._leave()
+        return list(zip(ids[0].tolist(), w[0].tolist()))
+
     def route_gated(self, logits, k, gating=Gating.Softmax, norm=True, scale=1.0, bias=None):
         """model::route_gated on one row -> list of (expert, weight), best first."""
         ids, w = self.route_rows(logits.reshape(1, -1), k, gating, norm, scale, bias)

@@ -2,7 +2,7 @@
 #pragma once
 
 // =========================================================================
-// MoE router: per token softmax (or sigmoid) over n_expert <= 64*EPL logits, top-k
+// MoE router: per token softmax (sigmoid == 1: sigmoid; 2: the row holds the scores already) over n_expert <= 64*EPL logits, top-k
 // by descending selection score with the LOWER INDEX winning ties, winners
 // renormalised (moe.rs:524-594).  One wave per token; lane l holds experts
 // l, l+64, l+128, ... (EPL of them).
@@ -94,9 +94,12 @@ DEV void route_token(const float* lr, const float* bias, int n_expert, int k, in
         const float inv = 1.0f / sum;
 #pragma unroll
         for (int j = 0; j < EPL; j++) score[j] *= inv;
-    } else {
+    } else if (sigmoid == 1) {
 #pragma unroll
         for (int j = 0; j < EPL; j++) score[j] = 1.0f / (1.0f + expf_ref(-lg[j], tab));
+    } else {  // the inputs are the scores already: route(probs, k) of the softmaxed row (moe.rs:623-658)
+#pragma unroll
+        for (int j = 0; j < EPL; j++) score[j] = lane + 64 * j < n_expert ? lg[j] : 0.0f;
     }
 #pragma unroll
     for (int j = 0; j < EPL; j++) {  // the selection value: the score, plus the expert's bias where the model has one

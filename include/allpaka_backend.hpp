@@ -352,6 +352,22 @@ inline std::vector<std::pair<size_t, float>> route_gated(const std::vector<float
     return out;
 }
 
+// model::route(probs, k) (moe.rs:623-658): the top k of an already softmaxed row, renormalised to sum to 1, best first.
+inline std::vector<std::pair<size_t, float>> route(const std::vector<float>& probs, size_t k) {
+    k = k < probs.size() ? k : probs.size();
+    if (k == 0) return {};
+    Dev<float> dp(probs.data(), probs.size()), dw(k);
+    Dev<uint32_t> di(k);
+    check(apk_route_topk(Gpu::get().ctx(), dp.ptr(), nullptr, 1, probs.size(), k, 1, 1.0f, 2, di.ptr(), dw.ptr()));
+    std::vector<uint32_t> ids(k);
+    std::vector<float> w(k);
+    di.read_back(ids.data());
+    dw.read_back(w.data());
+    std::vector<std::pair<size_t, float>> out;
+    for (size_t i = 0; i < k; i++) out.emplace_back(ids[i], w[i]);
+    return out;
+}
+
 // The batched router of Ffn::moe_batch (moe.rs:204-227): route_gated_into_slice for every row of
 // logits [rows][n_expert]; ids and w are [rows][k], best first.
 struct Routed {

@@ -341,12 +341,13 @@ int apk_swiglu(apk_ctx* ctx, void* gate, const void* up, size_t n, int dtype);
  * where 1 + tanh z >= 0.1, the same idiom on the values elsewhere. */
 int apk_geglu_tanh(apk_ctx* ctx, void* gate, const void* up, size_t n, int dtype);
 
-/* MoE router: softmax (sigmoid != 0: sigmoid) over n_expert logits, top-k by
- * descending selection score (+ bias when given), ties -> lower expert id,
+/* MoE router: softmax (sigmoid == 1: sigmoid; sigmoid == 2: the rows hold the scores already) over n_expert
+ * logits, top-k by descending selection score (+ bias when given), ties -> lower expert id,
  * weights renormalised over the winners when norm != 0, then * scale.  Replaces
  * model::route_gated / route_gated_into_slice per token (model/moe.rs:524-616,
- * token loop :204-227).  logits: f32[rows][n_expert]; ids: u32[rows][k];
- * w: f32[rows][k], both best-first.  n_expert <= 1024, 1 <= k <= min(n_expert, 64). */
+ * token loop :204-227); with sigmoid == 2, norm != 0, scale 1 and no bias it is the older
+ * model::route(probs, k) on softmaxed rows (model/moe.rs:623-658), bit for bit.  logits: f32[rows][n_expert];
+ * ids: u32[rows][k]; w: f32[rows][k], both best-first.  n_expert <= 1024, 1 <= k <= min(n_expert, 64). */
 int apk_route_topk(apk_ctx* ctx, const float* logits, const float* bias, size_t rows, size_t n_expert, size_t k,
                    int norm, float scale, int sigmoid, uint32_t* ids, float* w);
 

@@ -250,6 +250,13 @@ static void weights_are_named_by_host_address_inside_an_attached_mapping() {
     CHECK(gpu::detach(file.data(), file.size()));
 }
 static void route_picks_the_top_k_and_renormalises() {  // crates/allpaka-model/tests/gpu_eligible_forward.rs:88-97
+    // the test as the reference writes it: route(&[0.1, 0.5, 0.15, 0.25], 2) on probabilities
+    auto direct = route({0.1f, 0.5f, 0.15f, 0.25f}, 2);
+    CHECK(direct.size() == 2 && direct[0].first == 1 && direct[1].first == 3);
+    CHECK(direct[0].second == 0.5f / (0.5f + 0.25f) && direct[1].second == 0.25f / (0.5f + 0.25f));
+    CHECK(route({0.25f, 0.25f}, 5).size() == 2 && route({}, 2).empty());
+    auto flat = route({0.0f, 0.0f, 0.0f}, 2);  // nothing to renormalise by: 1 / k each, lower index first
+    CHECK(flat.size() == 2 && flat[0].first == 0 && flat[1].first == 1 && flat[0].second == 0.5f);
     std::vector<float> logp = {std::log(0.1f), std::log(0.5f), std::log(0.15f), std::log(0.25f)};
     auto picked = route_gated(logp, 2, Gating::Softmax, true, 1.0f, nullptr);
     CHECK(picked.size() == 2 && picked[0].first == 1 && picked[1].first == 3);

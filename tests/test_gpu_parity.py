@@ -1197,6 +1197,28 @@ def test_router_exp_is_the_host_libm_exp_over_its_whole_range(be, ora):
     assert np.array_equal(host(ids), want_ids) and np.array_equal(host(w).view(np.uint32), want_w.view(np.uint32))
 
 
+def test_route_on_probabilities_is_the_older_route(be, ora):
+    """model::route(probs, k) (moe.rs:623-658): the rows are scores already.  The reference's own vector
+    (tests/gpu_eligible_forward.rs:89-97) and random softmaxed rows, ids and weights bit for bit."""
+    got = be.route(dev(np.float32([0.1, 0.5, 0.15, 0.25])), 2)
+    assert [e for e, _ in got] == [1, 3]
+    assert np.array_equal(np.float32([x for _, x in got]), np.float32([0.5, 0.25]) / (np.float32(0.5) + np.float32(0.25)))
+    wi, ww = ora.route(np.float32([0.1, 0.5, 0.15, 0.25]), 2)
+    assert list(wi) == [1, 3] and np.array_equal(np.float32([x for _, x in got]), ww)
+    g = synth().rng(4, 4242)
+    for n, k in ((128, 8), (64, 1), (256, 8), (1000, 25), (7, 7), (5, 9)):
+        probs = synth().normal_f32(g, n)
+        ora.softmax(probs)
+        if n == 128:
+            probs[17] = probs[90] = probs[3]  # equal scores: lower index first
+        wi, ww = ora.route(probs, k)
+        got = be.route(dev(probs), k)
+        assert [e for e, _ in got] == list(wi) and np.array_equal(np.float32([x for _, x in got]), ww), (n, k)
+    zero = be.route(dev(np.zeros(6, np.float32)), 3)  # total == 0: 1 / k each
+    assert [e for e, _ in zero] == [0, 1, 2] and all(x == np.float32(1.0) / np.float32(3.0) for _, x in zero)
+    assert be.route(dev(np.zeros(4, np.float32))[:0], 3) == []
+
+
 def test_route_reference_vectors_ties_sigmoid_bias(be, ora):
     import allpaka_amd as apk
 
