@@ -240,7 +240,9 @@ def main():
     e_qk = record("qknorm_rope_neox", tag, timed(op_qkrope, reps), bytes_qkrope)
     dom = record("swiglu", tag, timed(op_swiglu, reps, refresh=lambda: restore_gates(sw, gate0), span=len(sw)), bytes_swiglu)
     dead_op = dead_fraction(sw)  # after the last batch: every set gated at most once since its refresh
-    assert max(dead_chain, dead_op) < 0.01, f"SwiGLU was timed on decayed gates: {dead_chain:.4f} / {dead_op:.4f} zero, subnormal or not finite"
+    assert dead_op < 0.01, f"SwiGLU was timed on decayed gates: {dead_op:.4f} zero, subnormal or not finite"
+    if n_sw >= args.steps + args.warmup:  # a set per step: the timed steps saw live gates too (a longer run than the pool
+        assert dead_chain < 0.01, f"the timed steps ran on decayed gates: {dead_chain:.4f}"  # allows reuses sets; it is reported, not refused)
     # QK-norm + RoPE with the K/V cache store fused in (one launch; the cache planes of one layer, capacity T)
     kvp = [dict(v=randn((T, NKV * HD)), kc=torch.empty((T, NKV * HD), dtype=torch.float16, device=dev),
                 vc=torch.empty((T, NKV * HD), dtype=torch.float16, device=dev)) for _ in range(len(qk))]
@@ -440,6 +442,7 @@ def main():
                      "traffic_source": TRAFFIC_PROFILE,
                      "algorithmic_bytes_per_launch": dom["bytes"], "avg_launch_us": dom["us"],
                      "gate_dead_fraction": {"after_timed_steps": round(dead_chain, 6), "after_per_op_timing": round(dead_op, 6),
+                                            "sets": n_sw, "a_set_per_step": n_sw >= args.steps + args.warmup,
                                             "note": "share of SwiGLU gate elements that are zero, subnormal or not finite after the "
                                                     "run; the gates are restored from a pristine copy between timed batches"},
                      "kernels": headline_kernels},
