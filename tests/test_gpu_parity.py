@@ -296,6 +296,8 @@ def test_add_rmsnorm_rows(be, ora, n, rows, f16, with_delta):
 
 @pytest.mark.parametrize("n,rows", [(2304, 1), (3584, 6), (1152, 64), (2560, 300), (3840, 2100), (5376, 700), (2560, 4200), (1024, 9000),
                                     (8192, 3), (16384, 2),
+                                    # more fp16 rows than are resident at once: 5, 3 and 4 tiles per lane, 2 or 3 waves per row
+                                    (5120, 3100), (4608, 3100), (3584, 3100),
                                     # outside the tiled kernels: the two steps run
                                     (1001, 5), (64, 100), (20488, 2)])
 @pytest.mark.parametrize("f16", [False, True])
