@@ -624,6 +624,35 @@ def other_shapes(args, L, h, apklib, synth, torch, gen, dev, randn, pool, p, tim
     record("MoE layer chain, recorded once and replayed", tagm, sorted(reps_us)[2], moe_bytes, launches=5)
     check(L.apk_graph_destroy(h, gmoe))
     del cb, se2, se
+    # the same three streaming ops on fp16 activations (the reference's MoE path is f32; a second run at half the bytes,
+    # same tables): every set of gates is gated once between two restores
+    f16 = torch.float16
+    tagh = f"qwen3-30b-a3b T={TM} f16"
+    gh = pool(TM * HM * 2 + TM * K * HM * 2, lambda: dict(hs=randn((TM, HM)), xe=torch.empty((TM * K, HM), dtype=f16, device=dev)))
+    us = timed(lambda i: check(L.apk_scatter_rows(h, p(gh[i % len(gh)]["hs"]), p(hit_row), TM, K, TM * K, HM, p(gh[i % len(gh)]["xe"]), F16)), reps)
+    record("scatter_rows (permute, token-side)", tagh, us, TM * HM * 2 + TM * K * HM * 2 + TM * K * 4)
+    del gh
+    gate_h = randn((TM * K, FM))
+    sh = [dict(gate=gate_h.clone(), up=randn((TM * K, FM))) for _ in range(max(6, int(COLD_BYTES // (2 * TM * K * FM * 2)) + 1))]
+    us = timed(lambda i: check(L.apk_swiglu(h, p(sh[i % len(sh)]["gate"]), p(sh[i % len(sh)]["up"]), TM * K * FM, F16)), reps,
+               refresh=lambda: restore_gates(sh, gate_h), span=len(sh))
+    assert dead_fraction(sh) < 0.01
+    record("swiglu", f"qwen3-30b-a3b [{TM * K}x{FM}] f16", us, 3 * TM * K * FM * 2)
+    del sh
+    ch = pool(TM * K * HM * 2 + 3 * TM * HM * 2, lambda: dict(flat=randn((TM * K, HM)), x=randn((TM, HM)),
+                                                          h=torch.empty((TM, HM), dtype=f16, device=dev)))
+    x_h = [s_["x"].clone() for s_ in ch]  # x += ... in place: restored between batches so that fp16 sums stay finite
+
+    def restore_x():
+        for s_, x0 in zip(ch, x_h):
+            s_["x"].copy_(x0)
+
+    torch.cuda.synchronize()
+    us = timed(lambda i: check(L.apk_moe_combine_add_rmsnorm(h, p(ch[i % len(ch)]["x"]), p(ch[i % len(ch)]["flat"]), p(tok_off), p(hit_row),
+                                                             p(hit_w), TM * K, p(ch[i % len(ch)]["h"]), p(gm), HM, TM, EPS, F16)), reps,
+               refresh=restore_x)
+    record("moe_combine + add + rmsnorm (one launch)", tagh, us, TM * K * HM * 2 + 3 * TM * HM * 2 + HM * 4 + TM * K * 8)
+    del ch, x_h
     # greedy pick over the vocabulary (after the output head): 1 and 64 rows of 151936 logits
     V = synth.MODELS["qwen3-32b"]["vocab"]
     lg = [randn((64, V), f32) for _ in range(17)]  # 17 x 38.9 MB
