@@ -201,6 +201,15 @@ class Backend:
         check(self.L.apk_add_assign(self.h, _ptr(a), _ptr(b), a.numel(), _dt(a)))
         self._leave()
 
+    def add_scaled_slice(self, dst, src, scale):
+        """ops::add_scaled_slice (blas.rs:25-102): dst = fma(src, scale, dst), the per-expert step of the decode MoE
+        combine (moe.rs:500-509).  A whole batch's combine is moe_combine_add_rmsnorm."""
+        assert dst.numel() == src.numel()
+        assert dst.dtype == src.dtype
+        self._enter()
+        check(self.L.apk_add_scaled(self.h, _ptr(dst), _ptr(src), dst.numel(), float(scale), _dt(dst)))
+        self._leave()
+
     def softmax(self, x):
         """ops::softmax (activation.rs:5) over each row of x (or over a 1-D x), in place."""
         assert x.dtype == torch.float32

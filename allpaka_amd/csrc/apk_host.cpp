@@ -71,7 +71,7 @@ std::vector<std::string> all_kernel_names() {
                                   "apk_embed_q4k_f16", "apk_embed_q8_0_f32", "apk_embed_q8_0_f16", "apk_route_topk",
                                   "apk_moe_permute", "apk_gather_rows", "apk_scatter_rows_t1", "apk_scatter_rows_t2", "apk_argmax_rows", "apk_add_rmsnorm_ragged_f32", "apk_add_rmsnorm_ragged_f16", "apk_copy",
                                   "apk_qknorm_rope_generic_f32", "apk_qknorm_rope_generic_f16", "apk_qknorm_rope_pos_f32", "apk_qknorm_rope_pos_f16", "apk_route_topk_wide", "apk_route_topk_e64", "apk_route_topk_e128", "apk_route_group_small_e64", "apk_route_group_small_e128",
-                                  "apk_route_group_small_e256", "apk_route_group_small_e1024", "apk_add_assign_f32", "apk_add_assign_f16", "apk_softmax_rows", "apk_moe_count", "apk_moe_rank",
+                                  "apk_route_group_small_e256", "apk_route_group_small_e1024", "apk_add_assign_f32", "apk_add_assign_f16", "apk_add_scaled_f32", "apk_add_scaled_f16", "apk_softmax_rows", "apk_moe_count", "apk_moe_rank",
                                   "apk_add_bias_rows_f32", "apk_add_bias_rows_f16", "apk_moe_shared_hits", "apk_cast_f32_f16", "apk_cast_f16_f32", "apk_zero_u64"};
     for (const char* t : {"f32", "f16"}) {
         for (const char* f : {"q5k", "q6k", "q2k", "q3k", "q5_0", "f16", "f32", "bf16"}) v.push_back(std::string("apk_embed_") + f + "_" + t);
@@ -905,6 +905,26 @@ int apk_add_assign(apk_ctx* c, void* a, const void* b, size_t n, int dtype) {
     void* args[] = {&a, &b, &n64};
     return launch_keyed(c, OP_ADD_ASSIGN, (uint32_t)dtype,
                         [&] { return std::string(dtype == APK_F32 ? "apk_add_assign_f32" : "apk_add_assign_f16"); }, (unsigned)grid, block, 0, args);
+}
+
+int apk_add_scaled(apk_ctx* c, void* dst, const void* src, size_t n, float scale, int dtype) {
+    if (!c) return fail(APK_DECLINE_NULL, "apk_add_scaled: ctx is NULL");
+    CallScope s(c);
+    const int es = elem_size(dtype);
+    if (!es) return fail(APK_DECLINE_UNSUPPORTED, "apk_add_scaled: dtype %d", dtype);
+    if (n == 0) return APK_OK;
+    if (!dst || !src) return fail(APK_DECLINE_NULL, "apk_add_scaled: NULL tensor");
+    if (dst == src) return fail(APK_DECLINE_SHAPE, "apk_add_scaled: dst and src must be two tensors");
+    if (!aligned16(dst) || !aligned16(src)) return fail(APK_DECLINE_SHAPE, "apk_add_scaled: tensors must be 16-byte aligned");
+    if (int rc = set_device(c)) return rc;
+    const uint64_t nvec = n / (16 / es);
+    const unsigned block = stream_block(nvec);
+    uint64_t grid = (nvec + block - 1) / block;
+    if (grid == 0) grid = 1;
+    if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_add_scaled: n too large");
+    uint64_t n64 = n;
+    void* args[] = {&dst, &src, &n64, &scale};
+    return launch(c, dtype == APK_F32 ? "apk_add_scaled_f32" : "apk_add_scaled_f16", (unsigned)grid, block, 0, args);
 }
 
 int apk_cast(apk_ctx* c, const void* src, int src_dtype, void* dst, int dst_dtype, size_t n) {

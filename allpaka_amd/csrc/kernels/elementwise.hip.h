@@ -106,6 +106,30 @@ extern "C" __global__ __launch_bounds__(256) void apk_add_assign_f16(f16_t* a, c
     add_assign_body<f16_t>(a, b, n);
 }
 
+// Scaled accumulate on its own: dst[i] = fma(src[i], scale, dst[i]) (ops::add_scaled_slice, blas.rs:25-102: one fused
+// multiply-add per element on both of the reference's SIMD arms, and `mul_add` in their tails), the step the decode
+// MoE combine repeats per picked expert (moe.rs:500-509).  fp16 rows: the f32 fma, rounded once.
+template <typename T> DEV void add_scaled_body(T* dst, const T* src, uint64_t n, float scale) {
+    constexpr int VEC = io<T>::VEC;
+    const uint64_t nvec = n / VEC, c = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c < nvec) {
+        float x[VEC], y[VEC];
+        io<T>::load_nt(dst + c * VEC, x);
+        io<T>::load_nt(src + c * VEC, y);
+#pragma unroll
+        for (int i = 0; i < VEC; i++) x[i] = __builtin_fmaf(y[i], scale, x[i]);
+        io<T>::store_wt(dst + c * VEC, x);
+    }
+    if (blockIdx.x == gridDim.x - 1)
+        for (uint64_t i = nvec * VEC + threadIdx.x; i < n; i += blockDim.x) dst[i] = (T)__builtin_fmaf((float)src[i], scale, (float)dst[i]);
+}
+extern "C" __global__ __launch_bounds__(256) void apk_add_scaled_f32(float* dst, const float* src, uint64_t n, float scale) {
+    add_scaled_body<float>(dst, src, n, scale);
+}
+extern "C" __global__ __launch_bounds__(256) void apk_add_scaled_f16(f16_t* dst, const f16_t* src, uint64_t n, float scale) {
+    add_scaled_body<f16_t>(dst, src, n, scale);
+}
+
 // A per-row bias: x[r][i] += bias[i] (add_bias_rows, crates/allpaka-model/src/model/loader.rs:519-523: the
 // projection biases of attention.rs:125-129).  Whole 16-byte tiles where the row length allows, else per element.
 template <typename T> DEV void add_bias_rows_body(T* x, const float* bias, uint64_t rows, uint32_t n) {

@@ -64,6 +64,7 @@ SYMBOLS = {
     "apk_dequant_rows": (_i, [_vp, _i, _vp, _sz, _sz, _sz, _sz, _vp, _i]),
     "apk_embed_rows_host_ids": (_i, [_vp, _i, _vp, _sz, _sz, _vp, _sz, _vp, _i]),
     "apk_add_assign": (_i, [_vp, _vp, _vp, _sz, _i]),
+    "apk_add_scaled": (_i, [_vp, _vp, _vp, _sz, _f, _i]),
     "apk_softmax_rows": (_i, [_vp, _vp, _sz, _sz]),
     "apk_add_rmsnorm_rows": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _f, _i]),
     "apk_qknorm_rope_neox": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _f, _i]),

@@ -206,6 +206,15 @@ inline void add_assign_slice(std::vector<float>& a, const std::vector<float>& b)
     da.read_back(a.data());
 }
 
+// ops::add_scaled_slice(dst, src, scale): dst = fma(src, scale, dst) (blas.rs:25-102); a shorter or longer src panics
+// (ops/mod.rs:403-408).
+inline void add_scaled_slice(std::vector<float>& dst, const std::vector<float>& src, float scale) {
+    if (dst.size() != src.size()) throw Panic("assertion `left == right` failed: dst.len() == src.len()");
+    Dev<float> dd(dst.data(), dst.size()), ds(src.data(), src.size());
+    check(apk_add_scaled(Gpu::get().ctx(), dd.ptr(), ds.ptr(), dst.size(), scale, APK_F32));
+    dd.read_back(dst.data());
+}
+
 // add_bias_rows(rows, bias) (model/loader.rs:519-523): every whole row of bias.len() elements gets the bias; what is
 // left of a partial last row is untouched (chunks_exact_mut).
 inline void add_bias_rows(std::vector<float>& rows, const std::vector<float>& bias) {

@@ -212,6 +212,12 @@ int apk_dequant_rows(apk_ctx* ctx, int fmt, const void* table, size_t n_rows, si
  * (ops/blas.rs:105-213) where no norm follows (where one does, apk_add_rmsnorm_rows does
  * both in one pass).  Any n; bit-exact (fp16: widen, add in f32, one rounding). */
 int apk_add_assign(apk_ctx* ctx, void* a, const void* b, size_t n, int dtype);
+
+/* Scaled accumulate on its own: dst[i] = fma(src[i], scale, dst[i]), one rounding.  Replaces ops::add_scaled_slice
+ * (ops/blas.rs:25-102), the step the decode MoE combine repeats per picked expert, best first, and once more with
+ * scale 1 for the shared expert (model/moe.rs:500-509); a whole batch's combine is apk_moe_combine_add_rmsnorm.
+ * dst, src: n elements of dtype, two tensors; fp16 rows take the f32 fma rounded once. */
+int apk_add_scaled(apk_ctx* ctx, void* dst, const void* src, size_t n, float scale, int dtype);
 /* Softmax over rows of f32 in place.  Replaces ops::softmax (ops/activation.rs:5-16) per
  * row; the router's softmax is fused into apk_route_topk, this is the op on its own.
  * Rows of at most 4096 (router widths): the reference adds the exponentials one after the

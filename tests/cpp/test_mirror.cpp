@@ -135,6 +135,15 @@ static void add_assign_slice_adds_and_rejects_length_mismatch() {  // ops/mod.rs
     CHECK((a == std::vector<float>{1.5f, 0.0f, 13.0f, 4.25f, 0.0f}));
     CHECK(throws<Panic>([] { std::vector<float> a(8), b(7); ops::add_assign_slice(a, b); }));
 }
+static void add_scaled_slice_is_one_fma_and_rejects_length_mismatch() {  // blas.rs:25-102, ops/mod.rs:403-408
+    std::vector<float> a = {1.0f, 2.0f, -3.0f, 0.1f}, b = {0.5f, -2.0f, 10.0f, 0.3f};
+    ops::add_scaled_slice(a, b, 0.7f);
+    for (size_t i = 0; i < a.size(); i++) {
+        const float d0[] = {1.0f, 2.0f, -3.0f, 0.1f};
+        CHECK(a[i] == std::fmaf(b[i], 0.7f, d0[i]));
+    }
+    CHECK(throws<Panic>([] { std::vector<float> a(64), b(8); ops::add_scaled_slice(a, b, 2.0f); }));
+}
 static std::vector<std::array<float, 2>> table_for(uint32_t pos, size_t head_dim, float base) {  // rope.rs:8-22
     std::vector<std::array<float, 2>> t(head_dim / 2);
     for (size_t i = 0; i < head_dim / 2; i++) {
@@ -430,6 +439,7 @@ int main() {
         {"geglu_tanh_is_the_tanh_gelu_of_gate_times_up", geglu_tanh_is_the_tanh_gelu_of_gate_times_up},
         {"softmax_sums_to_one_and_survives_huge_logits", softmax_sums_to_one_and_survives_huge_logits},
         {"add_assign_slice_adds_and_rejects_length_mismatch", add_assign_slice_adds_and_rejects_length_mismatch},
+        {"add_scaled_slice_is_one_fma_and_rejects_length_mismatch", add_scaled_slice_is_one_fma_and_rejects_length_mismatch},
         {"rope_is_norm_preserving_and_identity_at_position_zero", rope_is_norm_preserving_and_identity_at_position_zero},
         {"rope_neox_pairs_split_channels", rope_neox_pairs_split_channels},
         {"partial_rotary_rotates_the_head_and_passes_the_tail", partial_rotary_rotates_the_head_and_passes_the_tail},

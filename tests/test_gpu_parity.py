@@ -1076,6 +1076,66 @@ def test_add_assign_slice_bit_exact(be, ora, n, f16):
         be.add_assign_slice(ta, tb[:-1])
 
 
+@pytest.mark.parametrize("n", [1, 3, 8, 1024, 2048, 5120 * 6 + 5, 65536 * 3 + 1])
+@pytest.mark.parametrize("f16", [False, True])
+def test_add_scaled_slice_bit_exact(be, ora, n, f16):
+    """ops::add_scaled_slice (blas.rs:25-102): dst = fma(src, scale, dst), one rounding -- bit for bit the oracle's fmaf
+    (an unfused scale * src + dst differs from it in about a quarter of the elements, so a device multiply-then-add
+    would fail here); with fp16 rows the f32 fma rounded once."""
+    s = synth()
+    g = s.rng(2, n)
+    a, b = s.normal_f32(g, n), s.normal_f32(g, n)
+    for scale in (0.37109375, 1.0, -2.5e-3):
+        if f16:
+            a16, b16 = s.to_f16_bits(a), s.to_f16_bits(b)
+            w32 = ora.f16_bits_to_f32(a16)
+            ora.add_scaled_slice(w32, ora.f16_bits_to_f32(b16), scale)
+            want = ora.f32_to_f16_bits(w32)
+            ta, tb = dev(a16), dev(b16)
+        else:
+            want = a.copy()
+            ora.add_scaled_slice(want, b, scale)
+            if n >= 1024 and scale == 0.37109375:  # the check has teeth: the unfused form is a different result
+                assert np.mean((np.float32(scale) * b + a).astype(np.float32) != want) > 0.05
+            ta, tb = dev(a), dev(b)
+        be.add_scaled_slice(ta, tb, scale)
+        assert np.array_equal(host(ta), want)
+        assert np.array_equal(host(tb), b16 if f16 else b)  # the source is only read
+    with pytest.raises(AssertionError):  # a shorter source panics (ops/mod.rs:403-408)
+        be.add_scaled_slice(ta, tb[:-1], 2.0)
+    import allpaka_amd as apk
+
+    with pytest.raises(apk.Declined):  # dst and src are two tensors (a unique borrow and a shared one in the reference)
+        be.add_scaled_slice(ta, ta, 2.0)
+
+
+def test_decode_moe_combine_is_add_scaled_slice_per_pick(be, ora):
+    """The single-token combine (moe.rs:500-509): out = 0, then add_scaled_slice(out, down_i, weight_i) per picked
+    expert, best first, then the shared expert with weight 1.  Three ways here, one result: that loop on the oracle,
+    the same loop through apk_add_scaled, and apk_moe_combine_add_rmsnorm with no tok_off (hits listed in pick order)
+    on a zero residual."""
+    s = synth()
+    hidden, k = 2048, 8
+    g = s.rng(3, hidden)
+    downs = s.normal_f32(g, (k + 1, hidden))
+    logits = s.normal_f32(g, 128)
+    _ids, w = ora.route_gated(logits, k)  # best first
+    weights = [float(v) for v in w] + [1.0]
+    want = np.zeros(hidden, np.float32)
+    for i in range(k + 1):
+        ora.add_scaled_slice(want, downs[i], weights[i])
+    out = dev(np.zeros(hidden, np.float32))
+    td = dev(downs)
+    for i in range(k + 1):
+        be.add_scaled_slice(out, td[i], weights[i])
+    assert np.array_equal(host(out), want)
+    x = dev(np.zeros((1, hidden), np.float32))
+    hit_row = dev(np.arange(k + 1, dtype=np.uint32))
+    hit_w = dev(np.asarray(weights, np.float32))
+    be.moe_combine_add_rmsnorm(x, td, None, hit_row, hit_w, None, None, 1e-6)
+    assert np.array_equal(host(x)[0], want)
+
+
 @pytest.mark.parametrize("rows,n", [(1, 3), (1, 128), (5, 256), (1024, 128), (3, 1000), (2, 4096)])
 def test_softmax_rows(be, ora, rows, n):
     s = synth()
