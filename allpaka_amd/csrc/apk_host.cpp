@@ -299,12 +299,15 @@ int plan_embed(int fmt, size_t n_in, size_t t, int out_dtype, apk_plan* p) {
         threads = (n_in / 256 * 8 + 63) / 64 * 64;
         p->slices_per_row = 1;
     } else if (fmt == APK_FMT_Q6K || fmt == APK_FMT_Q5K || fmt == APK_FMT_Q2K || fmt == APK_FMT_Q3K) {
-        // decoded straight from global memory, 8 lanes per 256-element super-block (the Q4_K lane layout)
+        // decoded straight from global memory, 8 lanes per 256-element super-block (the Q4_K lane layout), the
+        // super-blocks numbered across the batch: workgroups of 256 lanes, none idle but in the last one
         p->variant = EMBED_SUPERBLOCK;
-        const size_t lanes = n_in / 256 * 8;
-        threads = (lanes + 63) / 64 * 64;
-        if (threads > 256) threads = 256;
-        p->slices_per_row = (unsigned)((lanes + threads - 1) / threads);
+        const uint64_t sbs = (uint64_t)t * (n_in / 256);
+        if (sbs > 0xffffffffu) return fail(APK_DECLINE_SHAPE, "apk_embed_rows: too large");
+        threads = (size_t)std::min<uint64_t>(256, (sbs * 8 + 63) / 64 * 64);
+        grid = (sbs * 8 + threads - 1) / threads;
+        p->slices_per_row = 0;  // a workgroup is not tied to a row
+        p->items = (unsigned)sbs;
         p->tiles_per_lane = (unsigned)(256 / (16 / oes) / 8);
     } else if (fmt == APK_FMT_Q8_0 || fmt == APK_FMT_Q5_0 || fmt == APK_FMT_F32) {
         // decoded straight from global memory: a lane owns 4 of the row's 16-byte output tiles; a row takes
@@ -323,7 +326,7 @@ int plan_embed(int fmt, size_t n_in, size_t t, int out_dtype, apk_plan* p) {
         p->slices_per_row = 1;
     }
     if (threads > 256) threads = 256;
-    grid *= p->slices_per_row;
+    if (p->variant != EMBED_SUPERBLOCK) grid *= p->slices_per_row;
     if (grid > 0x7fffffffu) return fail(APK_DECLINE_SHAPE, "apk_embed_rows: too large");
     p->grid = (unsigned)grid;
     p->block = (unsigned)threads;
@@ -1284,7 +1287,9 @@ static int embed_common(apk_ctx* c, int fmt, const void* table, size_t vocab, si
         void* args[] = {&table, &table_bytes, &vocab32, &n_i, &ids_dev, &out, &c->fault_dev, &scale, &row0};
         return launch_keyed(c, OP_EMBED, key, which, p.grid, p.block, p.shmem, args);
     }
-    void* args[] = {&table, &vocab32, &n_i, &ids_dev, &p.slices_per_row, &out, &c->fault_dev, &scale, &row0};
+    uint32_t rows32 = (uint32_t)t;  // the super-block kernels number their lanes across the batch; the others slice a row
+    void* args[] = {&table, &vocab32, &n_i, &ids_dev, p.variant == EMBED_SUPERBLOCK ? (void*)&rows32 : (void*)&p.slices_per_row, &out,
+                    &c->fault_dev, &scale, &row0};
     return launch_keyed(c, OP_EMBED, key, which, p.grid, p.block, 0, args);
 }
 

@@ -310,25 +310,28 @@ DEV void embed_direct_body(const uint8_t* table, uint32_t vocab, int n_in, const
 // lanes per super-block, lane L owning tiles 8k + L of it (k = 0 .. 3 for fp16 output, 0 .. 7 for
 // f32): the super-block's header and scale fields are fetched once per lane for all its tiles
 // (the compiler merges the identical loads), and for every k the 8 lanes write one whole line.
+// Super-blocks are numbered across the batch (lane j of the launch serves super-block j / 8, of row (j / 8) / nsb), so
+// that a row whose super-blocks do not fill whole waves (5120 columns: 160 lanes) leaves no lane idle: the row
+// number and the token id are per lane (one division; the id loads of a wave hit one or two words).
 template <int FMT, typename TO>
 DEV void embed_direct_sb_body(const uint8_t* __restrict__ table, uint32_t vocab, int n_in, const uint32_t* __restrict__ ids,
-                              uint32_t chunks, TO* __restrict__ out, uint32_t* fault, float scale, uint32_t row0) {
+                              uint32_t rows, TO* __restrict__ out, uint32_t* fault, float scale, uint32_t row0) {
     constexpr int OPT = io<TO>::VEC, K = 256 / OPT / 8;
-    const uint32_t t = blockIdx.x / chunks, chunk = blockIdx.x - t * chunks;
-    const uint32_t id = ids ? ids[t] : row0 + (uint32_t)t;  // no id list: the rows row0, row0 + 1, ...
-    if (id >= vocab) {  // uniform
-        if (threadIdx.x == 0 && chunk == 0) atomicOr(fault, APK_FAULT_TOKEN_RANGE);
-        return;
-    }
     const uint32_t nsb = (uint32_t)n_in / 256;
-    const uint32_t j = chunk * blockDim.x + threadIdx.x, L = j & 7u;
-    const bool live = (j >> 3) < nsb;
-    const uint32_t sb = min(j >> 3, nsb - 1u);  // a lane past the last super-block re-reads it and stores nothing
-    const uint8_t* row = table + (uint64_t)id * ((uint64_t)nsb * dqd<FMT>::BB);
+    const uint64_t j = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t L = (uint32_t)j & 7u;
+    const uint32_t total = rows * nsb;  // the host keeps the batch's super-blocks below 2^32
+    const bool inside = (j >> 3) < total;
+    const uint32_t sbc = inside ? (uint32_t)(j >> 3) : total - 1u;  // a lane past the last super-block re-reads it and stores nothing
+    const uint32_t t = sbc / nsb, sb = sbc - t * nsb;
+    const uint32_t id = ids ? ids[t] : row0 + t;  // no id list: the rows row0, row0 + 1, ...
+    const bool ok = id < vocab;
+    if (!ok && inside && sb == 0 && L == 0) atomicOr(fault, APK_FAULT_TOKEN_RANGE);
+    const uint8_t* row = table + (uint64_t)(ok ? id : 0u) * ((uint64_t)nsb * dqd<FMT>::BB);  // a bad id reads row 0 and stores nothing
     float o[K][OPT];
 #pragma unroll
     for (int k = 0; k < K; k++) dqd<FMT>::template tile<OPT>(row, sb * 256u + (8u * k + L) * OPT, o[k]);
-    if (!live) return;
+    if (!inside || !ok) return;
     TO* orow = out + (uint64_t)t * n_in + (uint64_t)sb * 256;
 #pragma unroll
     for (int k = 0; k < K; k++) {
@@ -338,14 +341,14 @@ DEV void embed_direct_sb_body(const uint8_t* __restrict__ table, uint32_t vocab,
 }
 #define APK_EMBED_DIRECT_SB(NAME, FMT)                                                                                   \
     extern "C" __global__ __launch_bounds__(256) void apk_embed_##NAME##_f32(                                            \
-        const uint8_t* table, uint32_t vocab, int n_in, const uint32_t* ids, uint32_t chunks, float* out, uint32_t* fault, \
+        const uint8_t* table, uint32_t vocab, int n_in, const uint32_t* ids, uint32_t rows, float* out, uint32_t* fault, \
         float scale, uint32_t row0) {                                                                                    \
-        embed_direct_sb_body<FMT, float>(table, vocab, n_in, ids, chunks, out, fault, scale, row0);                      \
+        embed_direct_sb_body<FMT, float>(table, vocab, n_in, ids, rows, out, fault, scale, row0);                        \
     }                                                                                                                    \
     extern "C" __global__ __launch_bounds__(256) void apk_embed_##NAME##_f16(                                            \
-        const uint8_t* table, uint32_t vocab, int n_in, const uint32_t* ids, uint32_t chunks, f16_t* out, uint32_t* fault, \
+        const uint8_t* table, uint32_t vocab, int n_in, const uint32_t* ids, uint32_t rows, f16_t* out, uint32_t* fault, \
         float scale, uint32_t row0) {                                                                                    \
-        embed_direct_sb_body<FMT, f16_t>(table, vocab, n_in, ids, chunks, out, fault, scale, row0);                      \
+        embed_direct_sb_body<FMT, f16_t>(table, vocab, n_in, ids, rows, out, fault, scale, row0);                        \
     }
 APK_EMBED_DIRECT_SB(q6k, 2) APK_EMBED_DIRECT_SB(q5k, 1) APK_EMBED_DIRECT_SB(q2k, 4) APK_EMBED_DIRECT_SB(q3k, 5)
 

@@ -257,14 +257,18 @@ def test_embed_plans_cover_every_tile_of_a_row(L, kernels, bounds):
                     assert rc == 0, (fmt, n_in, t)
                     name = common(p, kernels, bounds)
                     assert name == f"apk_embed_{names[fmt]}_{'f32' if out_dtype == F32 else 'f16'}"
-                    assert p.grid == t * p.slices_per_row and p.block <= 256
+                    assert p.block <= 256
+                    if fmt in (1, 2, 4, 5):  # 8 lanes per super-block, super-blocks numbered across the batch: no idle lane but at the end
+                        lanes = t * (n_in // 256) * 8
+                        assert p.items * 8 == lanes and p.slices_per_row == 0
+                        assert p.block == min(256, -(-lanes // 64) * 64)
+                        assert p.grid * p.block >= lanes > (p.grid - 1) * p.block
+                        assert p.tiles_per_lane * 8 * (16 // oes) == 256
+                        continue
+                    assert p.grid == t * p.slices_per_row
                     tiles = n_in // (16 // oes)
                     if fmt == 0:  # Q4_K: the workgroup loops over the row's super-blocks, 8 lanes each
                         assert p.slices_per_row == 1 and p.block == min(256, -(-(n_in // 256 * 8) // 64) * 64)
-                    elif fmt in (1, 2, 4, 5):  # 8 lanes per super-block, chunks of up to 32 super-blocks
-                        lanes = n_in // 256 * 8
-                        assert p.slices_per_row * p.block >= lanes > (p.slices_per_row - 1) * p.block
-                        assert p.tiles_per_lane * 8 * (16 // oes) == 256
                     elif fmt in (3, 6, 8):  # four output tiles per lane
                         assert p.tiles_per_lane == 4
                         assert p.slices_per_row * p.block * 4 >= tiles > (p.slices_per_row - 1) * p.block * 4
