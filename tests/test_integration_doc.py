@@ -1,4 +1,4 @@
-"""The Rust binding printed in INTEGRATION.md against include/apk_hip.h: every exported function is declared there
+"""The Rust binding printed in the integration guide (GUIDE below) against include/apk_hip.h: every exported function is declared there
 once, with the same number of arguments and the same type for each, and the two #[repr(C)] structs list the header's
 fields in the header's order.  (Rust is not in this image, so the binding cannot be compiled here; this keeps the
 text a maintainer would paste from drifting away from the header it binds.)"""
@@ -6,6 +6,7 @@ import os
 import re
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GUIDE = "INTEGRATION.md"
 
 
 def _strip_c_comments(text):
@@ -66,7 +67,7 @@ def header_struct(name):
 
 
 def rust_binding():
-    md = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    md = open(os.path.join(ROOT, GUIDE)).read()
     start = md.index("// crates/allpaka-hip-sys/src/lib.rs")
     block = md[start:md.index("```", start)]
     block = re.sub(r"//[^\n]*", "", block)
@@ -118,7 +119,7 @@ def test_the_arm_has_an_item_for_every_entry_of_the_stub_arm():
         decode_greedy_continue prefill_begin prefill_replay prefill_graph_key multi_stage prefill_end prefill_end_output
         prefill_abort prefill_attn_block prefill_gdn_block shared_activation_stats set_rope_inv_freq_swa set_quant_gemm
         set_attn_window""".split()
-    md = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    md = open(os.path.join(ROOT, GUIDE)).read()
     start = md.index("// crates/allpaka-backend/src/gpu/hip/mod.rs")
     arm = md[start:md.index("\n```", start)]
     defined = set(re.findall(r"^pub fn ([a-z_0-9]+)", arm, flags=re.M)) | set(re.findall(r"pub use super::common::([a-z_]+);", arm))
@@ -147,18 +148,18 @@ def test_the_printed_build_script_builds_every_source_the_makefile_links():
         else:
             sources.add(f)
     sources.add("apk_kernels.hip")
-    md = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    md = open(os.path.join(ROOT, GUIDE)).read()
     start = md.index("// crates/allpaka-hip-sys/build.rs")
     build_rs = md[start:md.index("\n```", start)]
     missing = sorted(f for f in sources if f not in build_rs)
-    assert missing == [], f"build.rs in INTEGRATION.md does not build {missing}"
+    assert missing == [], f"build.rs in {GUIDE} does not build {missing}"
     # every file it names exists in this repository
     for f in re.findall(r"\{src\}/(apk_[a-z_]+\.[a-zA-Z]+)", build_rs):
         assert os.path.exists(os.path.join(ROOT, "allpaka_amd", "csrc", f)), f
 
 
 def test_every_entry_named_in_the_mapping_tables_exists():
-    md = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    md = open(os.path.join(ROOT, GUIDE)).read()
     c = header_functions()
     structs = {"apk_attn_prologue", "apk_plan", "apk_ctx", "apk_graph", "apk_hip", "apk_status", "apk_dq_fmt", "apk_kernels", "apk_embed", "apk_host", "apk_noalloc", "apk_noalloc_setup"}
     named = set(re.findall(r"\bapk_[a-z0-9_]+\b", md))
