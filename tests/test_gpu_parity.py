@@ -172,6 +172,41 @@ def test_embed_long_rows_take_several_workgroups(be, ora, fmt_name, n_in, out_f1
     assert np.array_equal(host(out).view(v), want.view(v))
 
 
+@pytest.mark.parametrize("fmt_name", ["Q4K", "Q5K", "Q6K", "Q8_0", "Q2K", "Q3K", "Q5_0", "F16", "F32", "BF16"])
+@pytest.mark.parametrize("hidden", [512, 1280])
+def test_embed_device_ids_out_of_vocab_leave_their_rows_and_raise_the_flag(be, ora, fmt_name, hidden):
+    """Ids that live on the device cannot be checked before the launch: a row whose id is >= vocab is left as it
+    was, its neighbours (which may share a wave, a workgroup or neither with it) are gathered as usual, and the
+    status word reports it once read -- for every format's kernel, fp16 and f32 output."""
+    fmt, vocab = ora.FMT[fmt_name], 9
+    g = np.random.default_rng(hidden + fmt)
+    rb = ora.expected_bytes(fmt, hidden)
+    raw = g.integers(0, 256, size=vocab * rb, dtype=np.uint8)
+    if fmt_name in _SCALE_OFFS:
+        bb, offs = _SCALE_OFFS[fmt_name]
+        for o in offs:
+            raw.reshape(-1, bb)[:, o + 1] &= 0x3B  # finite, small f16 scale fields
+    elif fmt_name == "F32":
+        raw = synth().normal_f32(synth().rng(4, hidden), vocab * hidden).view(np.uint8).copy()
+    else:
+        raw.view(np.uint16)[:] &= np.uint16(0xBFFF)
+    table = dev(raw)
+    ids = np.array([4, 9, 0, 8, 0xFFFFFFFF, 2, 2, 100, 7], np.uint32)
+    good = ids < vocab
+    for out_f16 in (False, True):
+        want = ora.embed_rows(raw, fmt, vocab, hidden, np.where(good, ids, 0).astype(np.uint32), out_f16=out_f16)
+        out = torch.full((ids.size, hidden), 3.0, dtype=torch.float16 if out_f16 else torch.float32, device="cuda")
+        assert be.take_faults() == 0
+        rc = be.L.apk_embed_rows(be.h, fmt, table.data_ptr(), vocab, hidden, dev(ids).data_ptr(), ids.size, out.data_ptr(),
+                                 1 if out_f16 else 0)
+        assert rc == 0
+        got = host(out)
+        v = np.uint16 if out_f16 else np.uint32
+        assert np.array_equal(got[good].view(v), want[good].view(v))
+        assert np.all(got[~good].view(v) == (0x4200 if out_f16 else 0x40400000))  # still 3.0
+        assert be.take_faults() & 1 and be.take_faults() == 0  # APK_FAULT_TOKEN_RANGE, cleared by the read
+
+
 def test_embed_subnormal_scales_and_reference_vectors(be, ora):
     import allpaka_amd as apk
 
