@@ -130,3 +130,34 @@ def test_head_rows_and_permuted_rows_past_four_gigabytes(be, ora):
     for r in (0, T - 1, T, 3 * T + 77, 524287, 524288, T * kk - 1):
         assert torch.equal(xg[r], hs[r % T]), r
     assert be.take_faults() == 0
+
+
+@pytest.mark.parametrize("fmt_name", ["Q4K", "Q6K", "Q8_0", "F16"])
+def test_embedding_rows_past_four_gigabytes_of_output(be, ora, fmt_name):
+    """420 000 gathered rows of 5120 fp16 columns are 4.3 GB of output: rows from the start, the 2^31- and 2^32-byte
+    marks and the very end against the oracle (a format of each kernel family: the hand-laid Q4_K kernel, the
+    super-block kernels whose lanes are numbered across the batch, the four-tiles-per-lane kernels, the staged ones)."""
+    fmt, vocab, hidden, T = ora.FMT[fmt_name], 600, 5120, 420000
+    rb = ora.expected_bytes(fmt, hidden)
+    g = np.random.default_rng(fmt)
+    raw = g.integers(0, 256, size=vocab * rb, dtype=np.uint8)
+    offs = {"Q4K": (144, [0, 2]), "Q6K": (210, [208]), "Q8_0": (34, [0])}.get(fmt_name)
+    if offs:
+        for o in offs[1]:
+            raw.reshape(-1, offs[0])[:, o + 1] &= 0x3B  # finite, small f16 scale fields
+    else:
+        raw.view(np.uint16)[:] &= np.uint16(0xBFFF)
+    ids = g.integers(0, vocab, size=T, dtype=np.uint32)
+    out = torch.empty((T, hidden), dtype=torch.float16, device="cuda")
+    table = torch.from_numpy(raw).cuda()
+    rc = be.L.apk_embed_rows(be.h, fmt, table.data_ptr(), vocab, hidden, torch.from_numpy(ids.view(np.int32)).cuda().data_ptr(), T,
+                             out.data_ptr(), 1)
+    assert rc == 0
+    be.sync()
+    per_row = hidden * 2
+    pick = sorted({0, 1, (1 << 31) // per_row - 1, (1 << 31) // per_row, (1 << 31) // per_row + 1, (1 << 32) // per_row - 1,
+                   (1 << 32) // per_row, (1 << 32) // per_row + 1, T - 2, T - 1})
+    want = ora.embed_rows(raw, fmt, vocab, hidden, ids[pick], out_f16=True)
+    for i, r in enumerate(pick):
+        assert np.array_equal(bits(out[r]), want[i].view(np.uint16)), (fmt_name, r)
+    assert be.take_faults() == 0
