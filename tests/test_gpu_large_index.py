@@ -129,6 +129,27 @@ def test_head_rows_and_permuted_rows_past_four_gigabytes(be, ora):
     xg = be.gather_rows(hs, tok)
     for r in (0, T - 1, T, 3 * T + 77, 524287, 524288, T * kk - 1):
         assert torch.equal(xg[r], hs[r % T]), r
+    del xg
+    # the combine over the same 4.3 GB of rows (its hits past the 4 GiB mark are those of expert 7 for tokens >= 65 424):
+    # x += sum of hit_w * flat[hit_row], then the norm -- chosen tokens against the oracle on their own eight rows
+    flat = torch.randn((T * kk, cols), generator=gen, device="cuda")
+    hit_w = torch.rand((T, kk), generator=gen, device="cuda")
+    x = torch.randn((T, cols), generator=gen, device="cuda")
+    hb = torch.empty_like(x)
+    gamma = (1 + 0.05 * torch.randn(cols, generator=gen, device="cuda")).contiguous()
+    picks = [0, 1, 65423, 65424, 65425, T - 1]
+    before = {t: x[t].cpu().numpy().copy() for t in picks}
+    tok_off = (torch.arange(T + 1, device="cuda", dtype=torch.int32) * kk).contiguous()
+    be.moe_combine_add_rmsnorm(x, flat, tok_off, hit_row.view(-1), hit_w.view(-1), hb, gamma, 1e-6)
+    for t in picks:
+        rows_t = hit_row[t].cpu().numpy().astype(np.int64)
+        wx = before[t].reshape(1, -1).copy()
+        wh = np.zeros_like(wx)
+        small = np.stack([flat[int(r)].cpu().numpy() for r in rows_t])
+        ora.moe_combine_add_rmsnorm(wx, small, np.array([0, kk], np.uint32), np.arange(kk, dtype=np.uint32),
+                                    hit_w[t].cpu().numpy().copy(), wh, gamma.cpu().numpy(), 1e-6)
+        assert np.array_equal(x[t].cpu().numpy().view(np.uint32), wx[0].view(np.uint32)), t
+        assert np.allclose(hb[t].cpu().numpy(), wh[0], rtol=1e-5, atol=1e-6), t
     assert be.take_faults() == 0
 
 
