@@ -65,7 +65,7 @@ typedef struct apk_plan {
     unsigned waves_per_row;   /* waves that share one row (0 where rows are not the unit)                  */
     unsigned rows_per_block;  /* rows (or row items) a workgroup takes when each wave or lane group owns one */
     unsigned lanes_per_row;   /* lanes that cover one row or one head                                      */
-    unsigned slices_per_row;  /* workgroup-sized slices a row is cut into                                  */
+    unsigned slices_per_row;  /* workgroup-sized slices a row is cut into (0: workgroups are not tied to rows) */
     unsigned items;           /* work items of the launch before it is rounded up to whole workgroups      */
 } apk_plan;
 
